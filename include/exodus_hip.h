@@ -1,0 +1,129 @@
+/*
+ * exodus_hip.h -- C ABI of libexodus_hip.so, the gfx950 (MI355X) implementation of the
+ * EXODUS neuron-dynamics path.
+ *
+ * Conventions shared by every entry point
+ *   - All tensors are device pointers to contiguous fp32.  "(n,t)" means a row-major matrix
+ *     of n rows (one row = one neuron of one batch element) by t time steps, time contiguous;
+ *     "(n)" is one value per row.  Offsets are 64-bit: n*t may exceed 2^31.
+ *   - The library never allocates, frees or synchronises.  Kernels are enqueued on `stream`
+ *     (a hipStream_t passed as void*; NULL = the null stream) of the CURRENT device; the caller
+ *     selects the device that owns the pointers.
+ *   - Return value: 0 on success, otherwise a hipError_t value (1 = invalid value for a bad
+ *     argument detected on the host before any launch).  exodus_hip_error_string() names it.
+ *   - n == 0 or t == 0 is a successful no-op (per-row outputs are then left untouched).
+ *   - Thread safe: no global state.
+ *
+ * The first six entry points map one-to-one onto the six production functions the reference
+ * exports from its CUDA extension (reference cuda/bindings.cu:362-373), so that the same unit
+ * tests can be written against either.  The "fused" entry points below them are what the
+ * autograd Functions call: one pass per direction.
+ */
+#ifndef EXODUS_HIP_H
+#define EXODUS_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ABI version of this header; bumped on any signature change. */
+#define EXODUS_HIP_ABI_VERSION 1
+
+int exodus_hip_abi_version(void);
+const char *exodus_hip_error_string(int status);
+
+/* ---------------------------------------------------------------------------------------------
+ * One-to-one counterparts of the reference bindings
+ * ------------------------------------------------------------------------------------------- */
+
+/* Replaces lifForward (reference cuda/bindings.cu:14-70, kernel cuda/lif_kernels.h:40-93).
+ * Per row, for each step:  v = (v - count*membr_subtract) * alpha + input;  if apply_theta_low
+ * and v < theta_low: v = theta_low;  count = v >= theta ? min((unsigned)(v/theta), cap) : 0.
+ * Writes count as float to out_spikes and v (before its own reset) to out_vmem.
+ * max_num_spikes < 0 means no cap.  theta_low may be NULL when apply_theta_low == 0. */
+int exodus_lif_forward(float *out_spikes, float *out_vmem, const float *input,
+                       const float *vmem_post_initial, const float *alpha,
+                       const float *membr_subtract, const float *theta, const float *theta_low,
+                       int apply_theta_low, int max_num_spikes, int64_t n, int64_t t,
+                       void *stream);
+
+/* Replaces lifBackward (reference cuda/bindings.cu:72-110, kernel cuda/lif_kernels.h:122-168).
+ * input_grad_i = nc_i g_i + sum_{j>i} g_j nc_i prod_{k=i+1..j} (alpha - membr_subtract*surr_{k-1}) nc_k,
+ * evaluated as the linear-time reverse recurrence lambda_t = nc_t (g_t + (alpha - membr_subtract*surr_t) lambda_{t+1}).
+ * As in the reference, `membr_subtract` here is alpha times the subtract value. */
+int exodus_lif_backward(float *input_grad, const float *surr, const float *output_grad,
+                        const float *not_clipped, const float *alpha, const float *membr_subtract,
+                        int64_t n, int64_t t, void *stream);
+
+/* Replaces lifBackwardAlpha (reference cuda/bindings.cu:112-158, kernel cuda/lif_kernels.h:199-246).
+ * alpha_grad = sum_j D_j g_j with D_0 = vmem_post_initial, D_j = nc_j (alpha (1 - c surr_{j-1}) D_{j-1} + vmem_post_{j-1}).
+ * gate_initial == 0 reproduces the reference exactly (D_0 enters step 1 even when step 0 was clipped);
+ * gate_initial != 0 multiplies D_0 by nc_0 first, which is the exact derivative. */
+int exodus_lif_backward_alpha(float *alpha_grad, const float *surr, const float *output_grad,
+                              const float *vmem_post, const float *vmem_post_initial,
+                              const float *not_clipped, const float *alpha,
+                              const float *membr_subtract, int gate_initial, int64_t n, int64_t t,
+                              void *stream);
+
+/* Replaces leakyForward (reference cuda/bindings.cu:163-193, kernel cuda/leaky_kernels.h:29-58).
+ * out_t = alpha * out_{t-1} + input_t, out_{-1} = vmem_initial. */
+int exodus_leaky_forward(float *out, const float *input, const float *vmem_initial,
+                         const float *alpha, int64_t n, int64_t t, void *stream);
+
+/* Replaces leakyBackward (reference cuda/bindings.cu:195-221, kernel cuda/leaky_kernels.h:82-110).
+ * input_grad_t = alpha * input_grad_{t+1} + output_grad_t. */
+int exodus_leaky_backward(float *input_grad, const float *output_grad, const float *alpha,
+                          int64_t n, int64_t t, void *stream);
+
+/* Replaces leakyBackwardAlpha (reference cuda/bindings.cu:223-257, kernel cuda/leaky_kernels.h:133-165).
+ * alpha_grad = sum_t input_grad_t * output_{t-1}, output_{-1} = vmem_initial (the same sum the
+ * reference accumulates forward in time as sum_t D_t output_grad_t). */
+int exodus_leaky_backward_alpha(float *alpha_grad, const float *output_grad, const float *output,
+                                const float *vmem_initial, const float *alpha, int64_t n,
+                                int64_t t, void *stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Fused entry points (one pass per direction)
+ * ------------------------------------------------------------------------------------------- */
+
+/* Everything LeakyIntegrator.backward needs (reference sinabs/exodus/leaky.py:53-76) in one
+ * reverse pass: input_grad (n,t); init_grad (n) = alpha * input_grad[:,0]; and, when
+ * alpha_grad != NULL, alpha_grad (n) as above (then `output` and `vmem_initial` are required).
+ * alpha_grad, init_grad may each be NULL. */
+int exodus_leaky_backward_fused(float *input_grad, float *alpha_grad, float *init_grad,
+                                const float *output_grad, const float *output,
+                                const float *vmem_initial, const float *alpha, int64_t n,
+                                int64_t t, void *stream);
+
+/* Surrogate-gradient functions evaluated inside exodus_lif_backward_fused. */
+enum exodus_surrogate_kind {
+    EXODUS_SURR_TENSOR = 0,          /* read ds/dv from the `surr` argument                          */
+    EXODUS_SURR_SINGLE_EXP = 1,      /* p1/(theta*p0) * exp(-|v-theta|/(theta*p0))    p0=width p1=scale */
+    EXODUS_SURR_PERIODIC_EXP = 2,    /* p1*exp(-|u-theta/2|/p0)/theta, u=v-theta/2 wrapped mod theta for v>=theta */
+    EXODUS_SURR_HEAVISIDE = 3        /* (v >= theta-p0) / theta                       p0=window       */
+};
+
+/* Everything IntegrateAndFire.backward computes (reference sinabs/exodus/spike.py:229-291) in one
+ * reverse pass over the saved pre-reset membrane potential `vmem`:
+ *   s_t  = surrogate(vmem_t, theta)            (or surr_t when kind == EXODUS_SURR_TENSOR)
+ *   nc_t = apply_theta_low ? vmem_t > theta_low : 1
+ *   g_t  = s_t * grad_spikes_t + grad_vmem_t   (grad_vmem may be NULL = zeros)
+ *   lambda_t = nc_t (g_t + (alpha - alpha*c*s_t) lambda_{t+1})           -> input_grad (n,t)
+ *   init_grad  = alpha * lambda_0                                         (n), may be NULL
+ *   alpha_grad = sum_t lambda_t * vpost_{t-1}, vpost_t = vmem_t - c*count_t, vpost_{-1} = vmem_post_initial
+ *                (n), may be NULL; count_t is recomputed from vmem_t, theta and max_num_spikes.
+ * The alpha gradient is the exact one (initial step gated), see exodus_lif_backward_alpha. */
+int exodus_lif_backward_fused(float *input_grad, float *alpha_grad, float *init_grad,
+                              const float *grad_spikes, const float *grad_vmem, const float *vmem,
+                              const float *surr, const float *vmem_post_initial,
+                              const float *alpha, const float *membr_subtract, const float *theta,
+                              const float *theta_low, int apply_theta_low, int max_num_spikes,
+                              int surrogate_kind, float surr_p0, float surr_p1, int64_t n,
+                              int64_t t, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* EXODUS_HIP_H */

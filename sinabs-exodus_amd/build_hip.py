@@ -1,0 +1,45 @@
+"""Build libexodus_hip.so for gfx950 with hipcc (cross-compiles without a GPU).
+
+Usage:  python build_hip.py [--force]
+The library lands next to the Python loader (sinabs/exodus/libexodus_hip.so).
+"""
+import os
+import shutil
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+SRC = os.path.join(HERE, "csrc", "exodus_hip.hip")
+INCLUDE = os.path.join(os.path.dirname(HERE), "include")
+OUT = os.path.join(HERE, "sinabs", "exodus", "libexodus_hip.so")
+
+# -ffp-contract=off : the forward recurrences must round every multiply and add separately
+# -packed-fp32-ops disabled : keep the compiler from forming packed fp32 instructions
+FLAGS = [
+    "-O3", "-std=c++17", "--offload-arch=gfx950", "-ffp-contract=off",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-fPIC", "-shared", "-fvisibility=hidden", "-Wall", "-Wno-unused-command-line-argument",
+]
+
+
+def build(force: bool = True) -> str:
+    if not force and os.path.exists(OUT) and os.path.getmtime(OUT) >= max(
+            os.path.getmtime(SRC), os.path.getmtime(os.path.join(INCLUDE, "exodus_hip.h"))):
+        return OUT
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    cmd = [hipcc] + FLAGS + ["-I", INCLUDE, "-o", OUT + ".tmp", SRC]
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    # hipcc's host pass does not know the gfx-only target feature and says so; that line is harmless
+    noise = "packed-fp32-ops"
+    out = "\n".join(l for l in proc.stdout.splitlines() if noise not in l)
+    if proc.returncode != 0:
+        sys.stderr.write(out + "\n")
+        raise RuntimeError("hipcc failed building libexodus_hip.so")
+    if out.strip():
+        sys.stderr.write(out + "\n")
+    os.replace(OUT + ".tmp", OUT)
+    return OUT
+
+
+if __name__ == "__main__":
+    print(build(force=True))

@@ -1,0 +1,694 @@
+// libexodus_hip.so -- gfx950 kernels for the EXODUS neuron-dynamics path and their C ABI.
+//
+// Layout problem: tensors are (rows, steps) with time contiguous, the recurrences are
+// sequential in time and independent across rows.  One lane owns one row.  A wave owns 64
+// consecutive rows and walks the time axis in tiles of TT steps:
+//
+//   global -> registers : each row segment of TT floats is fetched by TT/4 adjacent lanes as
+//                         16-byte vectors, so a wave-wide load touches whole contiguous segments
+//   registers -> LDS    : stored as a [64 rows][TT] tile whose 16-byte chunks are XOR-swizzled
+//   LDS -> lane         : lane r reads row r chunk by chunk (conflict free thanks to the swizzle),
+//                         runs the recurrence for 4 steps per chunk and writes results in place
+//   LDS -> global       : same mapping as the load, again whole segments
+//
+// The next tile's global loads are issued before the current tile is computed, so HBM latency
+// overlaps the serial dependency chain.  Tiles are private to a wave (workgroup = one wave), so
+// no workgroup barrier exists anywhere; ordering between the phases only needs the in-order
+// execution of one wave's LDS instructions plus a compiler fence.
+//
+// Arithmetic of the forward recurrences is written with explicit round-to-nearest multiplies and
+// adds (no fused multiply-add), in the operation order of the reference device code, so spike
+// trains are reproducible bit for bit against a scalar CPU evaluation.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "exodus_hip.h"
+
+namespace {
+
+constexpr int WAVE = 64;
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));    // one 16-byte chunk = 4 time steps
+
+__device__ __forceinline__ void wave_sync()
+{
+    // All lanes of a wave execute an instruction together and the LDS serves one wave's requests
+    // in issue order; what remains is to stop the compiler from moving LDS accesses across here.
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+template <int TT>
+struct Geom {
+    static_assert(TT == 16 || TT == 32 || TT == 64, "tile length");
+    static constexpr int CPR = TT / 4;                       // 16-byte chunks per row segment
+    static constexpr int RPI = WAVE / CPR;                   // rows fetched by one wave-wide load
+    static constexpr int NLD = CPR;                          // wave-wide loads per tile (64 rows / RPI)
+    static constexpr int ROWS_PER_BANK_LINE = (CPR >= 16) ? 1 : 16 / CPR;   // rows per 256 B of LDS
+    // float offset of logical chunk `c` of row `r` inside a tile
+    __device__ static __forceinline__ int off(int r, int c)
+    {
+        return r * TT + 4 * (c ^ ((r / ROWS_PER_BANK_LINE) & (CPR - 1)));
+    }
+};
+
+template <bool VEC>
+__device__ __forceinline__ f32x4 load4(const float *__restrict__ base, int64_t row, int64_t n_rows,
+                                        int64_t t, int64_t n_steps)
+{
+    f32x4 v = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (row < n_rows) {
+        const float *p = base + row * n_steps + t;
+        if (VEC) {
+            if (t + 3 < n_steps) v = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(p));
+        } else {
+            if (t + 0 < n_steps) v.x = __builtin_nontemporal_load(p + 0);
+            if (t + 1 < n_steps) v.y = __builtin_nontemporal_load(p + 1);
+            if (t + 2 < n_steps) v.z = __builtin_nontemporal_load(p + 2);
+            if (t + 3 < n_steps) v.w = __builtin_nontemporal_load(p + 3);
+        }
+    }
+    return v;
+}
+
+template <bool VEC>
+__device__ __forceinline__ void store4(float *__restrict__ base, int64_t row, int64_t n_rows, int64_t t,
+                                       int64_t n_steps, f32x4 v)
+{
+    if (row < n_rows) {
+        float *p = base + row * n_steps + t;
+        if (VEC) {
+            if (t + 3 < n_steps) __builtin_nontemporal_store(v, reinterpret_cast<f32x4 *>(p));
+        } else {
+            if (t + 0 < n_steps) __builtin_nontemporal_store(v.x, p + 0);
+            if (t + 1 < n_steps) __builtin_nontemporal_store(v.y, p + 1);
+            if (t + 2 < n_steps) __builtin_nontemporal_store(v.z, p + 2);
+            if (t + 3 < n_steps) __builtin_nontemporal_store(v.w, p + 3);
+        }
+    }
+}
+
+__device__ __forceinline__ float get(const f32x4 &v, int e) { return v[e]; }
+__device__ __forceinline__ void put(f32x4 &v, int e, float x) { v[e] = x; }
+
+// ---------------------------------------------------------------------------------------------
+// The scan driver.  Op supplies:
+//   NIN, NOUT          number of (n,t) inputs / outputs; output j reuses the LDS slot of input j
+//   REVERSE            walk time from the last step to the first
+//   in[NIN], out[NOUT] device pointers
+//   State, init(State&, row, valid), step(State&, const float* x, float* y), finish(State&, row)
+// ---------------------------------------------------------------------------------------------
+template <class Op, int TT, bool VEC>
+__global__ void __launch_bounds__(WAVE) scan_kernel(const Op op, const int64_t n_rows, const int64_t n_steps)
+{
+    using G = Geom<TT>;
+    constexpr int NIN = Op::NIN, NOUT = Op::NOUT;
+    constexpr int NSLOT = NIN > NOUT ? NIN : NOUT;
+    constexpr int TILE = WAVE * TT;                           // floats per tile
+    extern __shared__ f32x4 lds_raw[];
+    float *lds = reinterpret_cast<float *>(lds_raw);
+    (void)NSLOT;
+
+    const int lane = threadIdx.x;
+    const int64_t row0 = static_cast<int64_t>(blockIdx.x) * WAVE;
+    const int64_t my_row = row0 + lane;
+    const bool row_ok = my_row < n_rows;
+
+    typename Op::State st;
+    op.init(st, row_ok ? my_row : n_rows - 1, row_ok);
+
+    const int l_chunk = lane % G::CPR;                        // which 16 B of the segment this lane moves
+    const int l_row = lane / G::CPR;                          // first row this lane moves
+    const int64_t n_tiles = (n_steps + TT - 1) / TT;
+
+    f32x4 pre[NIN > 0 ? NIN : 1][G::NLD];
+
+    auto fetch = [&](int64_t tile) {
+        const int64_t t = tile * TT + 4 * l_chunk;
+#pragma unroll
+        for (int j = 0; j < NIN; ++j)
+#pragma unroll
+            for (int i = 0; i < G::NLD; ++i)
+                pre[j][i] = load4<VEC>(op.in[j], row0 + l_row + i * G::RPI, n_rows, t, n_steps);
+    };
+
+    fetch(Op::REVERSE ? n_tiles - 1 : 0);
+
+    for (int64_t it = 0; it < n_tiles; ++it) {
+        const int64_t tile = Op::REVERSE ? n_tiles - 1 - it : it;
+        const int64_t t0 = tile * TT;
+        const int n_valid = (n_steps - t0) < TT ? static_cast<int>(n_steps - t0) : TT;
+
+        // registers -> LDS
+#pragma unroll
+        for (int j = 0; j < NIN; ++j)
+#pragma unroll
+            for (int i = 0; i < G::NLD; ++i)
+                *reinterpret_cast<f32x4 *>(lds + j * TILE + G::off(l_row + i * G::RPI, l_chunk)) = pre[j][i];
+
+        // next tile's loads stay in flight during the compute and store phases below
+        if (it + 1 < n_tiles) fetch(Op::REVERSE ? tile - 1 : tile + 1);
+
+        wave_sync();
+
+        // the recurrence: lane = row, 4 steps per 16-byte chunk
+#pragma unroll
+        for (int qq = 0; qq < G::CPR; ++qq) {
+            const int q = Op::REVERSE ? G::CPR - 1 - qq : qq;
+            f32x4 xin[NIN > 0 ? NIN : 1];
+            f32x4 yout[NOUT > 0 ? NOUT : 1];
+#pragma unroll
+            for (int j = 0; j < NIN; ++j)
+                xin[j] = *reinterpret_cast<const f32x4 *>(lds + j * TILE + G::off(lane, q));
+#pragma unroll
+            for (int j = 0; j < NOUT; ++j) yout[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ee = 0; ee < 4; ++ee) {
+                const int e = Op::REVERSE ? 3 - ee : ee;
+                if (4 * q + e < n_valid) {
+                    float x[NIN > 0 ? NIN : 1];
+                    float y[NOUT > 0 ? NOUT : 1];
+#pragma unroll
+                    for (int j = 0; j < NIN; ++j) x[j] = get(xin[j], e);
+                    op.step(st, x, y);
+#pragma unroll
+                    for (int j = 0; j < NOUT; ++j) put(yout[j], e, y[j]);
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < NOUT; ++j)
+                *reinterpret_cast<f32x4 *>(lds + j * TILE + G::off(lane, q)) = yout[j];
+        }
+
+        if (NOUT > 0) {
+            wave_sync();
+            // LDS -> global, whole row segments per group of CPR lanes
+            const int64_t t = t0 + 4 * l_chunk;
+#pragma unroll
+            for (int j = 0; j < NOUT; ++j)
+#pragma unroll
+                for (int i = 0; i < G::NLD; ++i) {
+                    const f32x4 v = *reinterpret_cast<const f32x4 *>(lds + j * TILE + G::off(l_row + i * G::RPI, l_chunk));
+                    store4<VEC>(op.out[j], row0 + l_row + i * G::RPI, n_rows, t, n_steps, v);
+                }
+        }
+        wave_sync();
+    }
+
+    if (row_ok) op.finish(st, my_row);
+}
+
+// ---------------------------------------------------------------------------------------------
+// per-row helpers
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ float spike_count(float v, float theta, unsigned cap)
+{
+    // count = v >= theta ? min(unsigned(v / theta), cap) : 0      (IEEE division, truncation)
+    if (v >= theta) {
+        const unsigned k = static_cast<unsigned>(__fdiv_rn(v, theta));
+        return static_cast<float>(k < cap ? k : cap);
+    }
+    return 0.f;
+}
+
+template <int KIND>
+__device__ __forceinline__ float surrogate(float v, float theta, float p0, float p1, float row_a, float row_b)
+{
+    // row_a / row_b are per-row constants prepared in init()
+    if (KIND == EXODUS_SURR_SINGLE_EXP) {
+        // p1/(theta*p0) * exp(-|v - theta| / (theta*p0));  row_a = theta*p0, row_b = p1/(theta*p0)
+        return row_b * expf(-fabsf(v - theta) / row_a);
+    } else if (KIND == EXODUS_SURR_PERIODIC_EXP) {
+        // row_a = theta/2, row_b = p1/theta is NOT used so that the operation order stays
+        // p1 * (exp(.) / theta)
+        float u = v - row_a;
+        if (v >= theta) u = fmodf(u, theta);                 // u > 0 here, so fmod == floor-mod
+        return p1 * (expf(-fabsf(u - row_a) / p0) / theta);
+    } else {
+        // Heaviside window: row_a = theta - p0, row_b = 1/theta
+        return v >= row_a ? row_b : 0.f;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Ops
+// ---------------------------------------------------------------------------------------------
+struct LeakyFwdOp {
+    static constexpr int NIN = 1, NOUT = 1;
+    static constexpr bool REVERSE = false;
+    const float *in[1];
+    float *out[1];
+    const float *v_init, *alpha;
+    struct State { float v, a; };
+    __device__ __forceinline__ void init(State &s, int64_t row, bool) const
+    {
+        s.v = v_init[row];
+        s.a = alpha[row];
+    }
+    __device__ __forceinline__ void step(State &s, const float *x, float *y) const
+    {
+        s.v = __fadd_rn(__fmul_rn(s.v, s.a), x[0]);
+        y[0] = s.v;
+    }
+    __device__ __forceinline__ void finish(State &, int64_t) const {}
+};
+
+// reverse pass of the leaky integrator; optional alpha gradient and optional input-gradient store
+template <bool ALPHA, bool WRITE_GI>
+struct LeakyBwdOp {
+    static constexpr int NIN = ALPHA ? 2 : 1, NOUT = WRITE_GI ? 1 : 0;
+    static constexpr bool REVERSE = true;
+    const float *in[NIN];                                     // [0] output_grad, [1] forward output
+    float *out[1];
+    const float *v_init, *alpha;
+    float *alpha_grad, *init_grad;
+    struct State { float g, a; double acc; };
+    __device__ __forceinline__ void init(State &s, int64_t row, bool) const
+    {
+        s.g = 0.f;
+        s.a = alpha[row];
+        s.acc = 0.0;
+    }
+    __device__ __forceinline__ void step(State &s, const float *x, float *y) const
+    {
+        if (ALPHA) s.acc += static_cast<double>(s.g) * static_cast<double>(x[1]);   // g_{u+1} * out_u
+        s.g = __fadd_rn(__fmul_rn(s.g, s.a), x[0]);
+        if (WRITE_GI) y[0] = s.g;
+    }
+    __device__ __forceinline__ void finish(State &s, int64_t row) const
+    {
+        if (init_grad) init_grad[row] = __fmul_rn(s.a, s.g);
+        if (ALPHA) {
+            s.acc += static_cast<double>(s.g) * static_cast<double>(v_init[row]);
+            alpha_grad[row] = static_cast<float>(s.acc);
+        }
+    }
+};
+
+struct LifFwdOp {
+    static constexpr int NIN = 1, NOUT = 2;                   // out[0] = v_mem (in place of x), out[1] = spikes
+    static constexpr bool REVERSE = false;
+    const float *in[1];
+    float *out[2];
+    const float *v_init, *alpha, *c, *theta, *theta_low;
+    int apply_low;
+    unsigned cap;
+    struct State { float v, a, c, th, lo, cnt; };
+    __device__ __forceinline__ void init(State &s, int64_t row, bool) const
+    {
+        s.v = v_init[row];
+        s.a = alpha[row];
+        s.c = c[row];
+        s.th = theta[row];
+        s.lo = apply_low ? theta_low[row] : 0.f;
+        s.cnt = 0.f;
+    }
+    __device__ __forceinline__ void step(State &s, const float *x, float *y) const
+    {
+        float v = __fsub_rn(s.v, __fmul_rn(s.cnt, s.c));
+        v = __fmul_rn(v, s.a);
+        v = __fadd_rn(v, x[0]);
+        if (apply_low && v < s.lo) v = s.lo;
+        s.cnt = spike_count(v, s.th, cap);
+        s.v = v;
+        y[0] = v;
+        y[1] = s.cnt;
+    }
+    __device__ __forceinline__ void finish(State &, int64_t) const {}
+};
+
+// One reverse pass for the spiking layer: input gradient, initial-state gradient and alpha gradient.
+//   slot 0: grad wrt spikes (in) / input gradient (out);  slot 1: v_mem;  then grad wrt v_mem
+//   (HAS_GV) and the surrogate tensor (KIND == EXODUS_SURR_TENSOR)
+template <int KIND, bool HAS_GV, bool ALPHA>
+struct LifBwdOp {
+    static constexpr int GV_SLOT = 2, SURR_SLOT = HAS_GV ? 3 : 2;
+    static constexpr int NIN = 2 + (HAS_GV ? 1 : 0) + (KIND == EXODUS_SURR_TENSOR ? 1 : 0), NOUT = 1;
+    static constexpr bool REVERSE = true;
+    const float *in[NIN];
+    float *out[1];
+    const float *v_init, *alpha, *c, *theta, *theta_low;
+    float *alpha_grad, *init_grad;
+    int apply_low;
+    unsigned cap;
+    float p0, p1;
+    struct State { float lam, a, ac, c, th, lo, ra, rb; double acc; };
+    __device__ __forceinline__ void init(State &s, int64_t row, bool) const
+    {
+        s.lam = 0.f;
+        s.a = alpha[row];
+        s.c = c[row];
+        s.ac = __fmul_rn(s.a, s.c);
+        s.th = theta[row];
+        s.lo = apply_low ? theta_low[row] : 0.f;
+        s.acc = 0.0;
+        if (KIND == EXODUS_SURR_SINGLE_EXP) {
+            s.ra = __fmul_rn(s.th, p0);
+            s.rb = __fdiv_rn(p1, s.ra);
+        } else if (KIND == EXODUS_SURR_PERIODIC_EXP) {
+            s.ra = __fmul_rn(s.th, 0.5f);
+            s.rb = 0.f;
+        } else {
+            s.ra = __fsub_rn(s.th, p0);
+            s.rb = __fdiv_rn(1.f, s.th);
+        }
+    }
+    __device__ __forceinline__ void step(State &s, const float *x, float *y) const
+    {
+        const float v = x[1];
+        float sg;
+        if constexpr (KIND == EXODUS_SURR_TENSOR) sg = x[SURR_SLOT];
+        else sg = surrogate<KIND>(v, s.th, p0, p1, s.ra, s.rb);
+        float g = __fmul_rn(sg, x[0]);
+        if constexpr (HAS_GV) g = __fadd_rn(g, x[GV_SLOT]);
+        if (ALPHA) {
+            const float vpost = __fsub_rn(v, __fmul_rn(s.c, spike_count(v, s.th, cap)));
+            s.acc += static_cast<double>(s.lam) * static_cast<double>(vpost);       // lambda_{u+1} * vpost_u
+        }
+        const float f = __fsub_rn(s.a, __fmul_rn(s.ac, sg));
+        const float lam = __fadd_rn(g, __fmul_rn(f, s.lam));
+        s.lam = (apply_low && !(v > s.lo)) ? 0.f : lam;
+        y[0] = s.lam;
+    }
+    __device__ __forceinline__ void finish(State &s, int64_t row) const
+    {
+        if (init_grad) init_grad[row] = __fmul_rn(s.a, s.lam);
+        if (ALPHA) {
+            s.acc += static_cast<double>(s.lam) * static_cast<double>(v_init[row]);
+            alpha_grad[row] = static_cast<float>(s.acc);
+        }
+    }
+};
+
+// counterpart of the reference's lifBackward: surrogate, g and the clip mask come as tensors
+struct LifBwdTensorsOp {
+    static constexpr int NIN = 3, NOUT = 1;                   // in: g, surr, not_clipped
+    static constexpr bool REVERSE = true;
+    const float *in[3];
+    float *out[1];
+    const float *alpha, *csub;
+    struct State { float lam, a, cs; };
+    __device__ __forceinline__ void init(State &s, int64_t row, bool) const
+    {
+        s.lam = 0.f;
+        s.a = alpha[row];
+        s.cs = csub[row];
+    }
+    __device__ __forceinline__ void step(State &s, const float *x, float *y) const
+    {
+        const float f = __fsub_rn(s.a, __fmul_rn(s.cs, x[1]));
+        s.lam = __fmul_rn(x[2], __fadd_rn(x[0], __fmul_rn(f, s.lam)));
+        y[0] = s.lam;
+    }
+    __device__ __forceinline__ void finish(State &, int64_t) const {}
+};
+
+// counterpart of the reference's lifBackwardAlpha: forward in time, D recurrence
+struct LifBwdAlphaTensorsOp {
+    static constexpr int NIN = 4, NOUT = 0;                   // in: g, surr, not_clipped, v_post
+    static constexpr bool REVERSE = false;
+    const float *in[4];
+    float *out[1];
+    const float *v_init, *alpha, *c;
+    float *alpha_grad;
+    int gate_initial;
+    struct State { float d, a, c, s_prev, vp_prev; double acc; bool first; };
+    __device__ __forceinline__ void init(State &s, int64_t row, bool) const
+    {
+        s.d = v_init[row];
+        s.a = alpha[row];
+        s.c = c[row];
+        s.s_prev = 0.f;
+        s.vp_prev = 0.f;
+        s.acc = 0.0;
+        s.first = true;
+    }
+    __device__ __forceinline__ void step(State &s, const float *x, float *) const
+    {
+        if (s.first) {
+            const float d0 = __fmul_rn(x[2], s.d);
+            s.acc = static_cast<double>(d0) * static_cast<double>(x[0]);
+            if (gate_initial) s.d = d0;
+            s.first = false;
+        } else {
+            // D = D * (alpha * (1 - c*s_prev)) with the factor formed in double, as the reference's
+            // "1.0 -" literal makes it
+            const double fac = static_cast<double>(s.a) * (1.0 - static_cast<double>(__fmul_rn(s.c, s.s_prev)));
+            float d = static_cast<float>(static_cast<double>(s.d) * fac);
+            d = __fadd_rn(d, s.vp_prev);
+            d = __fmul_rn(d, x[2]);
+            s.d = d;
+            s.acc += static_cast<double>(d) * static_cast<double>(x[0]);
+        }
+        s.s_prev = x[1];
+        s.vp_prev = x[3];
+    }
+    __device__ __forceinline__ void finish(State &s, int64_t row) const { alpha_grad[row] = static_cast<float>(s.acc); }
+};
+
+// ---------------------------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------------------------
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+template <class Op, int TT>
+int launch(const Op &op, int64_t n, int64_t t, void *stream)
+{
+    constexpr int NSLOT = Op::NIN > Op::NOUT ? Op::NIN : Op::NOUT;
+    const size_t lds_bytes = static_cast<size_t>(NSLOT) * WAVE * TT * sizeof(float);
+    const int64_t n_blocks = (n + WAVE - 1) / WAVE;
+    if (n_blocks > 0x7fffffffLL) return hipErrorInvalidValue;
+    bool vec = (t % 4) == 0;
+    for (int j = 0; j < Op::NIN; ++j) vec = vec && aligned16(op.in[j]);
+    for (int j = 0; j < Op::NOUT; ++j) vec = vec && aligned16(op.out[j]);
+    const dim3 grid(static_cast<unsigned>(n_blocks)), block(WAVE);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (vec)
+        hipLaunchKernelGGL((scan_kernel<Op, TT, true>), grid, block, lds_bytes, s, op, n, t);
+    else
+        hipLaunchKernelGGL((scan_kernel<Op, TT, false>), grid, block, lds_bytes, s, op, n, t);
+    return static_cast<int>(hipGetLastError());
+}
+
+inline bool bad_dims(int64_t n, int64_t t) { return n < 0 || t < 0 || (t > 0 && n > INT64_MAX / t); }
+
+template <int KIND, bool HAS_GV, bool ALPHA>
+int launch_lif_bwd(float *input_grad, float *alpha_grad, float *init_grad, const float *grad_spikes,
+                   const float *grad_vmem, const float *vmem, const float *surr, const float *v_init,
+                   const float *alpha, const float *c, const float *theta, const float *theta_low,
+                   int apply_low, int max_spikes, float p0, float p1, int64_t n, int64_t t, void *stream)
+{
+    using Op = LifBwdOp<KIND, HAS_GV, ALPHA>;
+    Op op;
+    op.in[0] = grad_spikes;
+    op.in[1] = vmem;
+    if constexpr (HAS_GV) op.in[Op::GV_SLOT] = grad_vmem;
+    if constexpr (KIND == EXODUS_SURR_TENSOR) op.in[Op::SURR_SLOT] = surr;
+    op.out[0] = input_grad;
+    op.v_init = v_init;
+    op.alpha = alpha;
+    op.c = c;
+    op.theta = theta;
+    op.theta_low = theta_low;
+    op.alpha_grad = alpha_grad;
+    op.init_grad = init_grad;
+    op.apply_low = apply_low;
+    op.cap = static_cast<unsigned>(max_spikes);
+    op.p0 = p0;
+    op.p1 = p1;
+    if constexpr (Op::NIN <= 2) return launch<Op, 32>(op, n, t, stream);
+    else return launch<Op, 16>(op, n, t, stream);
+}
+
+template <int KIND>
+int dispatch_lif_bwd(bool has_gv, bool want_alpha, float *input_grad, float *alpha_grad, float *init_grad,
+                     const float *grad_spikes, const float *grad_vmem, const float *vmem, const float *surr,
+                     const float *v_init, const float *alpha, const float *c, const float *theta,
+                     const float *theta_low, int apply_low, int max_spikes, float p0, float p1, int64_t n,
+                     int64_t t, void *stream)
+{
+#define EXODUS_CALL(GV, AL)                                                                                     \
+    return launch_lif_bwd<KIND, GV, AL>(input_grad, alpha_grad, init_grad, grad_spikes, grad_vmem, vmem, surr, \
+                                        v_init, alpha, c, theta, theta_low, apply_low, max_spikes, p0, p1, n,  \
+                                        t, stream)
+    if (has_gv) {
+        if (want_alpha) EXODUS_CALL(true, true);
+        EXODUS_CALL(true, false);
+    }
+    if (want_alpha) EXODUS_CALL(false, true);
+    EXODUS_CALL(false, false);
+#undef EXODUS_CALL
+}
+
+}  // namespace
+
+// ---------------------------------------------------------------------------------------------
+// C ABI
+// ---------------------------------------------------------------------------------------------
+extern "C" {
+
+#define EXODUS_API __attribute__((visibility("default")))
+
+EXODUS_API int exodus_hip_abi_version(void) { return EXODUS_HIP_ABI_VERSION; }
+
+EXODUS_API const char *exodus_hip_error_string(int status)
+{
+    return hipGetErrorString(static_cast<hipError_t>(status));
+}
+
+EXODUS_API int exodus_lif_forward(float *out_spikes, float *out_vmem, const float *input,
+                                  const float *vmem_post_initial, const float *alpha,
+                                  const float *membr_subtract, const float *theta, const float *theta_low,
+                                  int apply_theta_low, int max_num_spikes, int64_t n, int64_t t, void *stream)
+{
+    if (bad_dims(n, t)) return hipErrorInvalidValue;
+    if (n == 0 || t == 0) return hipSuccess;
+    if (!out_spikes || !out_vmem || !input || !vmem_post_initial || !alpha || !membr_subtract || !theta ||
+        (apply_theta_low && !theta_low))
+        return hipErrorInvalidValue;
+    LifFwdOp op;
+    op.in[0] = input;
+    op.out[0] = out_vmem;
+    op.out[1] = out_spikes;
+    op.v_init = vmem_post_initial;
+    op.alpha = alpha;
+    op.c = membr_subtract;
+    op.theta = theta;
+    op.theta_low = theta_low;
+    op.apply_low = apply_theta_low ? 1 : 0;
+    op.cap = static_cast<unsigned>(max_num_spikes);           // negative -> no cap
+    return launch<LifFwdOp, 32>(op, n, t, stream);
+}
+
+EXODUS_API int exodus_lif_backward(float *input_grad, const float *surr, const float *output_grad,
+                                   const float *not_clipped, const float *alpha, const float *membr_subtract,
+                                   int64_t n, int64_t t, void *stream)
+{
+    if (bad_dims(n, t)) return hipErrorInvalidValue;
+    if (n == 0 || t == 0) return hipSuccess;
+    if (!input_grad || !surr || !output_grad || !not_clipped || !alpha || !membr_subtract)
+        return hipErrorInvalidValue;
+    LifBwdTensorsOp op;
+    op.in[0] = output_grad;
+    op.in[1] = surr;
+    op.in[2] = not_clipped;
+    op.out[0] = input_grad;
+    op.alpha = alpha;
+    op.csub = membr_subtract;
+    return launch<LifBwdTensorsOp, 16>(op, n, t, stream);
+}
+
+EXODUS_API int exodus_lif_backward_alpha(float *alpha_grad, const float *surr, const float *output_grad,
+                                         const float *vmem_post, const float *vmem_post_initial,
+                                         const float *not_clipped, const float *alpha,
+                                         const float *membr_subtract, int gate_initial, int64_t n, int64_t t,
+                                         void *stream)
+{
+    if (bad_dims(n, t)) return hipErrorInvalidValue;
+    if (n == 0 || t == 0) return hipSuccess;
+    if (!alpha_grad || !surr || !output_grad || !vmem_post || !vmem_post_initial || !not_clipped || !alpha ||
+        !membr_subtract)
+        return hipErrorInvalidValue;
+    LifBwdAlphaTensorsOp op;
+    op.in[0] = output_grad;
+    op.in[1] = surr;
+    op.in[2] = not_clipped;
+    op.in[3] = vmem_post;
+    op.out[0] = nullptr;
+    op.v_init = vmem_post_initial;
+    op.alpha = alpha;
+    op.c = membr_subtract;
+    op.alpha_grad = alpha_grad;
+    op.gate_initial = gate_initial ? 1 : 0;
+    return launch<LifBwdAlphaTensorsOp, 16>(op, n, t, stream);
+}
+
+EXODUS_API int exodus_leaky_forward(float *out, const float *input, const float *vmem_initial,
+                                    const float *alpha, int64_t n, int64_t t, void *stream)
+{
+    if (bad_dims(n, t)) return hipErrorInvalidValue;
+    if (n == 0 || t == 0) return hipSuccess;
+    if (!out || !input || !vmem_initial || !alpha) return hipErrorInvalidValue;
+    LeakyFwdOp op;
+    op.in[0] = input;
+    op.out[0] = out;
+    op.v_init = vmem_initial;
+    op.alpha = alpha;
+    return launch<LeakyFwdOp, 32>(op, n, t, stream);
+}
+
+EXODUS_API int exodus_leaky_backward_fused(float *input_grad, float *alpha_grad, float *init_grad,
+                                           const float *output_grad, const float *output,
+                                           const float *vmem_initial, const float *alpha, int64_t n, int64_t t,
+                                           void *stream)
+{
+    if (bad_dims(n, t)) return hipErrorInvalidValue;
+    if (n == 0 || t == 0) return hipSuccess;
+    if (!output_grad || !alpha) return hipErrorInvalidValue;
+    if (alpha_grad && (!output || !vmem_initial)) return hipErrorInvalidValue;
+    if (!input_grad && !alpha_grad) return hipErrorInvalidValue;
+    if (alpha_grad) {
+        if (input_grad) {
+            LeakyBwdOp<true, true> op;
+            op.in[0] = output_grad; op.in[1] = output; op.out[0] = input_grad;
+            op.v_init = vmem_initial; op.alpha = alpha; op.alpha_grad = alpha_grad; op.init_grad = init_grad;
+            return launch<LeakyBwdOp<true, true>, 32>(op, n, t, stream);
+        }
+        LeakyBwdOp<true, false> op;
+        op.in[0] = output_grad; op.in[1] = output; op.out[0] = nullptr;
+        op.v_init = vmem_initial; op.alpha = alpha; op.alpha_grad = alpha_grad; op.init_grad = init_grad;
+        return launch<LeakyBwdOp<true, false>, 32>(op, n, t, stream);
+    }
+    LeakyBwdOp<false, true> op;
+    op.in[0] = output_grad; op.out[0] = input_grad;
+    op.v_init = vmem_initial; op.alpha = alpha; op.alpha_grad = nullptr; op.init_grad = init_grad;
+    return launch<LeakyBwdOp<false, true>, 32>(op, n, t, stream);
+}
+
+EXODUS_API int exodus_leaky_backward(float *input_grad, const float *output_grad, const float *alpha,
+                                     int64_t n, int64_t t, void *stream)
+{
+    if (!input_grad) return hipErrorInvalidValue;
+    return exodus_leaky_backward_fused(input_grad, nullptr, nullptr, output_grad, nullptr, nullptr, alpha, n, t,
+                                       stream);
+}
+
+EXODUS_API int exodus_leaky_backward_alpha(float *alpha_grad, const float *output_grad, const float *output,
+                                           const float *vmem_initial, const float *alpha, int64_t n, int64_t t,
+                                           void *stream)
+{
+    if (!alpha_grad) return hipErrorInvalidValue;
+    return exodus_leaky_backward_fused(nullptr, alpha_grad, nullptr, output_grad, output, vmem_initial, alpha, n,
+                                       t, stream);
+}
+
+EXODUS_API int exodus_lif_backward_fused(float *input_grad, float *alpha_grad, float *init_grad,
+                                         const float *grad_spikes, const float *grad_vmem, const float *vmem,
+                                         const float *surr, const float *vmem_post_initial, const float *alpha,
+                                         const float *membr_subtract, const float *theta, const float *theta_low,
+                                         int apply_theta_low, int max_num_spikes, int surrogate_kind,
+                                         float surr_p0, float surr_p1, int64_t n, int64_t t, void *stream)
+{
+    if (bad_dims(n, t)) return hipErrorInvalidValue;
+    if (n == 0 || t == 0) return hipSuccess;
+    if (!input_grad || !grad_spikes || !vmem || !alpha || !membr_subtract || !theta) return hipErrorInvalidValue;
+    if (apply_theta_low && !theta_low) return hipErrorInvalidValue;
+    if (alpha_grad && !vmem_post_initial) return hipErrorInvalidValue;
+    if (surrogate_kind == EXODUS_SURR_TENSOR && !surr) return hipErrorInvalidValue;
+    const bool gv = grad_vmem != nullptr, al = alpha_grad != nullptr;
+#define EXODUS_KIND(K)                                                                                         \
+    return dispatch_lif_bwd<K>(gv, al, input_grad, alpha_grad, init_grad, grad_spikes, grad_vmem, vmem, surr, \
+                               vmem_post_initial, alpha, membr_subtract, theta, theta_low,                    \
+                               apply_theta_low ? 1 : 0, max_num_spikes, surr_p0, surr_p1, n, t, stream)
+    switch (surrogate_kind) {
+        case EXODUS_SURR_TENSOR: EXODUS_KIND(EXODUS_SURR_TENSOR);
+        case EXODUS_SURR_SINGLE_EXP: EXODUS_KIND(EXODUS_SURR_SINGLE_EXP);
+        case EXODUS_SURR_PERIODIC_EXP: EXODUS_KIND(EXODUS_SURR_PERIODIC_EXP);
+        case EXODUS_SURR_HEAVISIDE: EXODUS_KIND(EXODUS_SURR_HEAVISIDE);
+        default: return hipErrorInvalidValue;
+    }
+#undef EXODUS_KIND
+}
+
+}  // extern "C"

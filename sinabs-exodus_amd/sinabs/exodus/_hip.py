@@ -1,0 +1,288 @@
+"""ctypes loader for ``libexodus_hip.so`` and thin tensor-level wrappers around its C ABI.
+
+This module plays the role of the reference's ``exodus_cuda`` pybind module
+(reference cuda/bindings.cu:362-373): same six functions, same argument order, plus the two
+fused backward entry points.  Tensors must live on a HIP device, be ``float32`` and contiguous;
+anything else raises, as the reference's ``CHECK_INPUT`` asserts do
+(reference cuda/bindings.cu:7-10).  There is no CPU path: if the shared library is missing the
+import of this module fails with an ``ImportError`` that says how to build it.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from typing import Optional
+
+import torch  # must be imported before the library so both share one HIP runtime
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libexodus_hip.so")
+
+SURR_TENSOR, SURR_SINGLE_EXP, SURR_PERIODIC_EXP, SURR_HEAVISIDE = 0, 1, 2, 3
+ABI_VERSION = 1
+
+_p = ctypes.c_void_p
+_i64 = ctypes.c_int64
+_int = ctypes.c_int
+_f = ctypes.c_float
+
+_SIGNATURES = {
+    "exodus_hip_abi_version": ([], _int),
+    "exodus_hip_error_string": ([_int], ctypes.c_char_p),
+    "exodus_lif_forward": ([_p] * 8 + [_int, _int, _i64, _i64, _p], _int),
+    "exodus_lif_backward": ([_p] * 6 + [_i64, _i64, _p], _int),
+    "exodus_lif_backward_alpha": ([_p] * 8 + [_int, _i64, _i64, _p], _int),
+    "exodus_leaky_forward": ([_p] * 4 + [_i64, _i64, _p], _int),
+    "exodus_leaky_backward": ([_p] * 3 + [_i64, _i64, _p], _int),
+    "exodus_leaky_backward_alpha": ([_p] * 5 + [_i64, _i64, _p], _int),
+    "exodus_leaky_backward_fused": ([_p] * 7 + [_i64, _i64, _p], _int),
+    "exodus_lif_backward_fused": ([_p] * 12 + [_int, _int, _int, _f, _f, _i64, _i64, _p], _int),
+}
+
+
+def _load() -> ctypes.CDLL:
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} not found. Build it with `python build_hip.py` in the package root "
+            "(needs hipcc; cross-compiles for gfx950 without a GPU). There is no CPU fallback."
+        )
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (argtypes, restype) in _SIGNATURES.items():
+        fn = getattr(lib, name)  # AttributeError here = library/header mismatch
+        fn.argtypes = argtypes
+        fn.restype = restype
+    got = lib.exodus_hip_abi_version()
+    if got != ABI_VERSION:
+        raise ImportError(f"libexodus_hip.so has ABI version {got}, this package expects {ABI_VERSION}")
+    return lib
+
+
+lib = _load()
+
+
+class ExodusHipError(RuntimeError):
+    pass
+
+
+def _check(status: int, what: str) -> None:
+    if status != 0:
+        msg = lib.exodus_hip_error_string(status)
+        raise ExodusHipError(f"{what} failed: {msg.decode() if msg else status} (hipError {status})")
+
+
+def _dev(x: torch.Tensor, name: str, like: Optional[torch.Tensor] = None) -> torch.Tensor:
+    if not isinstance(x, torch.Tensor):
+        raise TypeError(f"{name} must be a tensor")
+    if not x.is_cuda:
+        raise RuntimeError(f"{name} must be a tensor on a HIP device (got {x.device}); there is no CPU path")
+    if x.dtype != torch.float32:
+        raise RuntimeError(f"{name} must be float32 (got {x.dtype})")
+    if not x.is_contiguous():
+        raise RuntimeError(f"{name} must be contiguous")
+    if like is not None and x.device != like.device:
+        raise RuntimeError(f"{name} and the first tensor must be on the same device")
+    return x
+
+
+def _rows(x: torch.Tensor, name: str, n: int) -> torch.Tensor:
+    if x.ndim != 1 or x.shape[0] != n:
+        raise RuntimeError(f"{name} must have shape ({n},), got {tuple(x.shape)}")
+    return x
+
+
+def _mat(x: torch.Tensor, name: str, n: int, t: int) -> torch.Tensor:
+    if x.ndim != 2 or x.shape[0] != n or x.shape[1] != t:
+        raise RuntimeError(f"{name} must have shape ({n}, {t}), got {tuple(x.shape)}")
+    return x
+
+
+def _ptr(x: Optional[torch.Tensor]):
+    return None if x is None else ctypes.c_void_p(x.data_ptr())
+
+
+def _stream(x: torch.Tensor):
+    return ctypes.c_void_p(torch.cuda.current_stream(x.device).cuda_stream)
+
+
+# ------------------------------------------------------------------------------------------
+# the six functions of the reference extension, same names and argument order
+# ------------------------------------------------------------------------------------------
+
+def lifForward(outputSpikes, vmem, input, vmemPostInitial, alpha, membrSubtract, theta, thetaLow,
+               applyThetaLow: bool, maxNumSpikes: int) -> None:
+    """reference cuda/bindings.cu:14-70; fills the caller-allocated ``outputSpikes`` and ``vmem``."""
+    _dev(input, "input")
+    if input.ndim != 2:
+        raise RuntimeError("input must be 2-D (rows, time)")
+    n, t = input.shape
+    _mat(_dev(outputSpikes, "outputSpikes", input), "outputSpikes", n, t)
+    _mat(_dev(vmem, "vmem", input), "vmem", n, t)
+    for nm, x in (("vmemPostInitial", vmemPostInitial), ("alpha", alpha), ("membrSubtract", membrSubtract),
+                  ("theta", theta)):
+        _rows(_dev(x, nm, input), nm, n)
+    if applyThetaLow:
+        _rows(_dev(thetaLow, "thetaLow", input), "thetaLow", n)
+    else:
+        thetaLow = None
+    with torch.cuda.device(input.device):
+        _check(lib.exodus_lif_forward(_ptr(outputSpikes), _ptr(vmem), _ptr(input), _ptr(vmemPostInitial),
+                                      _ptr(alpha), _ptr(membrSubtract), _ptr(theta), _ptr(thetaLow),
+                                      int(bool(applyThetaLow)), int(maxNumSpikes), n, t, _stream(input)),
+               "exodus_lif_forward")
+
+
+def lifBackward(surr, outputGrad, notClipped, alpha, membrSubtract) -> torch.Tensor:
+    """reference cuda/bindings.cu:72-110; ``membrSubtract`` is alpha times the subtract value."""
+    _dev(surr, "surr")
+    if surr.ndim != 2:
+        raise RuntimeError("surr must be 2-D (rows, time)")
+    n, t = surr.shape
+    _mat(_dev(outputGrad, "outputGrad", surr), "outputGrad", n, t)
+    _mat(_dev(notClipped, "notClipped", surr), "notClipped", n, t)
+    _rows(_dev(alpha, "alpha", surr), "alpha", n)
+    _rows(_dev(membrSubtract, "membrSubtract", surr), "membrSubtract", n)
+    inputGrad = torch.empty_like(surr)
+    with torch.cuda.device(surr.device):
+        _check(lib.exodus_lif_backward(_ptr(inputGrad), _ptr(surr), _ptr(outputGrad), _ptr(notClipped),
+                                       _ptr(alpha), _ptr(membrSubtract), n, t, _stream(surr)),
+               "exodus_lif_backward")
+    return inputGrad
+
+
+def lifBackwardAlpha(surr, outputGrad, vmemPost, vmemPostInitial, notClipped, alpha, membrSubtract,
+                     gateInitial: bool = False) -> torch.Tensor:
+    """reference cuda/bindings.cu:112-158.  ``gateInitial=False`` is the reference's arithmetic."""
+    _dev(surr, "surr")
+    if surr.ndim != 2:
+        raise RuntimeError("surr must be 2-D (rows, time)")
+    n, t = surr.shape
+    for nm, x in (("outputGrad", outputGrad), ("vmemPost", vmemPost), ("notClipped", notClipped)):
+        _mat(_dev(x, nm, surr), nm, n, t)
+    for nm, x in (("vmemPostInitial", vmemPostInitial), ("alpha", alpha), ("membrSubtract", membrSubtract)):
+        _rows(_dev(x, nm, surr), nm, n)
+    alphaGrad = torch.zeros_like(alpha)
+    with torch.cuda.device(surr.device):
+        _check(lib.exodus_lif_backward_alpha(_ptr(alphaGrad), _ptr(surr), _ptr(outputGrad), _ptr(vmemPost),
+                                             _ptr(vmemPostInitial), _ptr(notClipped), _ptr(alpha),
+                                             _ptr(membrSubtract), int(bool(gateInitial)), n, t, _stream(surr)),
+               "exodus_lif_backward_alpha")
+    return alphaGrad
+
+
+def leakyForward(input, vmemInitial, alpha) -> torch.Tensor:
+    """reference cuda/bindings.cu:163-193."""
+    _dev(input, "input")
+    if input.ndim != 2:
+        raise RuntimeError("input must be 2-D (rows, time)")
+    n, t = input.shape
+    _rows(_dev(vmemInitial, "vmemInitial", input), "vmemInitial", n)
+    _rows(_dev(alpha, "alpha", input), "alpha", n)
+    out = torch.empty_like(input)
+    with torch.cuda.device(input.device):
+        _check(lib.exodus_leaky_forward(_ptr(out), _ptr(input), _ptr(vmemInitial), _ptr(alpha), n, t,
+                                        _stream(input)), "exodus_leaky_forward")
+    return out
+
+
+def leakyBackward(outputGrad, alpha) -> torch.Tensor:
+    """reference cuda/bindings.cu:195-221."""
+    _dev(outputGrad, "outputGrad")
+    if outputGrad.ndim != 2:
+        raise RuntimeError("outputGrad must be 2-D (rows, time)")
+    n, t = outputGrad.shape
+    _rows(_dev(alpha, "alpha", outputGrad), "alpha", n)
+    inputGrad = torch.empty_like(outputGrad)
+    with torch.cuda.device(outputGrad.device):
+        _check(lib.exodus_leaky_backward(_ptr(inputGrad), _ptr(outputGrad), _ptr(alpha), n, t,
+                                         _stream(outputGrad)), "exodus_leaky_backward")
+    return inputGrad
+
+
+def leakyBackwardAlpha(outputGrad, output, vmemInitial, alpha) -> torch.Tensor:
+    """reference cuda/bindings.cu:223-257."""
+    _dev(outputGrad, "outputGrad")
+    if outputGrad.ndim != 2:
+        raise RuntimeError("outputGrad must be 2-D (rows, time)")
+    n, t = outputGrad.shape
+    _mat(_dev(output, "output", outputGrad), "output", n, t)
+    _rows(_dev(vmemInitial, "vmemInitial", outputGrad), "vmemInitial", n)
+    _rows(_dev(alpha, "alpha", outputGrad), "alpha", n)
+    alphaGrad = torch.zeros_like(alpha)
+    with torch.cuda.device(outputGrad.device):
+        _check(lib.exodus_leaky_backward_alpha(_ptr(alphaGrad), _ptr(outputGrad), _ptr(output),
+                                               _ptr(vmemInitial), _ptr(alpha), n, t, _stream(outputGrad)),
+               "exodus_leaky_backward_alpha")
+    return alphaGrad
+
+
+# ------------------------------------------------------------------------------------------
+# fused backward passes (what the autograd Functions use)
+# ------------------------------------------------------------------------------------------
+
+def leakyBackwardFused(outputGrad, alpha, output=None, vmemInitial=None, needAlphaGrad: bool = False,
+                       inputGrad: Optional[torch.Tensor] = None):
+    """One reverse pass: returns (inputGrad, alphaGrad | None, initGrad)."""
+    _dev(outputGrad, "outputGrad")
+    if outputGrad.ndim != 2:
+        raise RuntimeError("outputGrad must be 2-D (rows, time)")
+    n, t = outputGrad.shape
+    _rows(_dev(alpha, "alpha", outputGrad), "alpha", n)
+    if needAlphaGrad:
+        _mat(_dev(output, "output", outputGrad), "output", n, t)
+        _rows(_dev(vmemInitial, "vmemInitial", outputGrad), "vmemInitial", n)
+    if inputGrad is None:
+        inputGrad = torch.empty_like(outputGrad)
+    else:
+        _mat(_dev(inputGrad, "inputGrad", outputGrad), "inputGrad", n, t)
+    initGrad = torch.zeros_like(alpha)
+    alphaGrad = torch.zeros_like(alpha) if needAlphaGrad else None
+    with torch.cuda.device(outputGrad.device):
+        _check(lib.exodus_leaky_backward_fused(_ptr(inputGrad), _ptr(alphaGrad), _ptr(initGrad), _ptr(outputGrad),
+                                               _ptr(output) if needAlphaGrad else None,
+                                               _ptr(vmemInitial) if needAlphaGrad else None, _ptr(alpha), n, t,
+                                               _stream(outputGrad)), "exodus_leaky_backward_fused")
+    return inputGrad, alphaGrad, initGrad
+
+
+def lifBackwardFused(gradSpikes, gradVmem, vmem, vmemPostInitial, alpha, membrSubtract, theta, thetaLow,
+                     applyThetaLow: bool, maxNumSpikes: int, surrogateKind: int, surrP0: float = 0.0,
+                     surrP1: float = 0.0, surr: Optional[torch.Tensor] = None, needAlphaGrad: bool = False,
+                     inputGrad: Optional[torch.Tensor] = None):
+    """One reverse pass over the saved membrane potential: returns (inputGrad, alphaGrad | None, initGrad).
+
+    ``membrSubtract`` is the plain subtract value here (not pre-multiplied by alpha).
+    """
+    _dev(vmem, "vmem")
+    if vmem.ndim != 2:
+        raise RuntimeError("vmem must be 2-D (rows, time)")
+    n, t = vmem.shape
+    _mat(_dev(gradSpikes, "gradSpikes", vmem), "gradSpikes", n, t)
+    if gradVmem is not None:
+        _mat(_dev(gradVmem, "gradVmem", vmem), "gradVmem", n, t)
+    for nm, x in (("alpha", alpha), ("membrSubtract", membrSubtract), ("theta", theta)):
+        _rows(_dev(x, nm, vmem), nm, n)
+    if applyThetaLow:
+        _rows(_dev(thetaLow, "thetaLow", vmem), "thetaLow", n)
+    else:
+        thetaLow = None
+    if needAlphaGrad:
+        _rows(_dev(vmemPostInitial, "vmemPostInitial", vmem), "vmemPostInitial", n)
+    if surrogateKind == SURR_TENSOR:
+        _mat(_dev(surr, "surr", vmem), "surr", n, t)
+    else:
+        surr = None
+    if inputGrad is None:
+        inputGrad = torch.empty_like(vmem)
+    else:
+        _mat(_dev(inputGrad, "inputGrad", vmem), "inputGrad", n, t)
+    initGrad = torch.zeros_like(alpha)
+    alphaGrad = torch.zeros_like(alpha) if needAlphaGrad else None
+    with torch.cuda.device(vmem.device):
+        _check(lib.exodus_lif_backward_fused(_ptr(inputGrad), _ptr(alphaGrad), _ptr(initGrad), _ptr(gradSpikes),
+                                             _ptr(gradVmem), _ptr(vmem), _ptr(surr),
+                                             _ptr(vmemPostInitial) if needAlphaGrad else None, _ptr(alpha),
+                                             _ptr(membrSubtract), _ptr(theta), _ptr(thetaLow),
+                                             int(bool(applyThetaLow)), int(maxNumSpikes), int(surrogateKind),
+                                             float(surrP0), float(surrP1), n, t, _stream(vmem)),
+               "exodus_lif_backward_fused")
+    return inputGrad, alphaGrad, initGrad
