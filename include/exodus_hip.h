@@ -123,6 +123,41 @@ int exodus_lif_backward_fused(float *input_grad, float *alpha_grad, float *init_
                               int surrogate_kind, float surr_p0, float surr_p1, int64_t n,
                               int64_t t, void *stream);
 
+/* ---------------------------------------------------------------------------------------------
+ * Synapse + membrane in one kernel per direction.  The reference composes this stage from four
+ * passes: input * alpha_syn (reference sinabs/exodus/layers/lif.py:190-191), LeakyIntegrator
+ * (lif.py:194-198), (1 - alpha_mem) * i_syn (lif.py:206-209) and IntegrateAndFire (lif.py:245-254),
+ * and lets torch autograd chain their gradients.  These two entry points compute the same
+ * values with the operations in the same order.
+ * ------------------------------------------------------------------------------------------- */
+
+/* Per row and step:
+ *   xin = decay_early ? input*alpha_syn : input;  i = i*alpha_syn + xin;
+ *   u = norm_input ? (1 - alpha_mem)*i : i;       v = (v - count*membr_subtract)*alpha_mem + u;
+ *   clamp at theta_low if apply_theta_low;        count = v >= theta ? min((unsigned)(v/theta), cap) : 0
+ * Writes count to out_spikes, v (before reset) to out_vmem and i to out_isyn, all (n,t). */
+int exodus_synlif_forward(float *out_spikes, float *out_vmem, float *out_isyn, const float *input,
+                          const float *vmem_post_initial, const float *isyn_initial,
+                          const float *alpha_mem, const float *alpha_syn, const float *membr_subtract,
+                          const float *theta, const float *theta_low, int apply_theta_low,
+                          int max_num_spikes, int decay_early, int norm_input, int64_t n, int64_t t,
+                          void *stream);
+
+/* Reverse pass of the above from the saved vmem and isyn.  grad_vmem and grad_isyn (gradients
+ * arriving at the vmem / isyn outputs) must be both given or both NULL.  Outputs: grad_input (n,t)
+ * and, each optional (NULL = not wanted), the per-row alpha_mem_grad, alpha_syn_grad,
+ * vmem_init_grad, isyn_init_grad.  surrogate_kind must be one of the in-kernel kinds (1..3).
+ * alpha_syn_grad with decay_early divides by alpha_syn and is therefore undefined for rows
+ * whose alpha_syn is exactly 0. */
+int exodus_synlif_backward(float *grad_input, float *alpha_mem_grad, float *alpha_syn_grad,
+                           float *vmem_init_grad, float *isyn_init_grad, const float *grad_spikes,
+                           const float *grad_vmem, const float *grad_isyn, const float *vmem,
+                           const float *isyn, const float *vmem_post_initial, const float *isyn_initial,
+                           const float *alpha_mem, const float *alpha_syn, const float *membr_subtract,
+                           const float *theta, const float *theta_low, int apply_theta_low,
+                           int max_num_spikes, int decay_early, int norm_input, int surrogate_kind,
+                           float surr_p0, float surr_p1, int64_t n, int64_t t, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -98,6 +98,10 @@ __device__ __forceinline__ void put(f32x4 &v, int e, float x) { v[e] = x; }
 //   REVERSE            walk time from the last step to the first
 //   in[NIN], out[NOUT] device pointers
 //   State, init(State&, row, valid), step(State&, const float* x, float* y), finish(State&, row)
+//   NDER (0 or 1)      one more (n,t) output that is a pure function of output DER_SRC and of
+//                      NROWP per-row constants: it is computed while the tile is written back
+//                      (stash(State&, float* p) / derive(const float* p, f32x4 v)), so it needs no
+//                      LDS tile of its own
 // ---------------------------------------------------------------------------------------------
 template <class Op, int TT, bool VEC>
 __global__ void __launch_bounds__(WAVE) scan_kernel(const Op op, const int64_t n_rows, const int64_t n_steps)
@@ -106,9 +110,10 @@ __global__ void __launch_bounds__(WAVE) scan_kernel(const Op op, const int64_t n
     constexpr int NIN = Op::NIN, NOUT = Op::NOUT;
     constexpr int NSLOT = NIN > NOUT ? NIN : NOUT;
     constexpr int TILE = WAVE * TT;                           // floats per tile
+    constexpr int NDER = Op::NDER, NROWP = Op::NROWP;
     extern __shared__ f32x4 lds_raw[];
     float *lds = reinterpret_cast<float *>(lds_raw);
-    (void)NSLOT;
+    float *rowp = lds + NSLOT * TILE;                         // [64 rows][NROWP] constants for derive()
 
     const int lane = threadIdx.x;
     const int64_t row0 = static_cast<int64_t>(blockIdx.x) * WAVE;
@@ -117,6 +122,12 @@ __global__ void __launch_bounds__(WAVE) scan_kernel(const Op op, const int64_t n
 
     typename Op::State st;
     op.init(st, row_ok ? my_row : n_rows - 1, row_ok);
+    if constexpr (NDER > 0) {
+        float consts[NROWP > 0 ? NROWP : 1];
+        op.stash(st, consts);
+#pragma unroll
+        for (int k = 0; k < NROWP; ++k) rowp[lane * NROWP + k] = consts[k];
+    }
 
     const int l_chunk = lane % G::CPR;                        // which 16 B of the segment this lane moves
     const int l_row = lane / G::CPR;                          // first row this lane moves
@@ -191,6 +202,11 @@ __global__ void __launch_bounds__(WAVE) scan_kernel(const Op op, const int64_t n
                 for (int i = 0; i < G::NLD; ++i) {
                     const f32x4 v = *reinterpret_cast<const f32x4 *>(lds + j * TILE + G::off(l_row + i * G::RPI, l_chunk));
                     store4<VEC>(op.out[j], row0 + l_row + i * G::RPI, n_rows, t, n_steps, v);
+                    if constexpr (NDER > 0) {
+                        if (j == Op::DER_SRC)
+                            store4<VEC>(op.der, row0 + l_row + i * G::RPI, n_rows, t, n_steps,
+                                        op.derive(rowp + (l_row + i * G::RPI) * NROWP, v));
+                    }
                 }
         }
         wave_sync();
@@ -235,6 +251,7 @@ __device__ __forceinline__ float surrogate(float v, float theta, float p0, float
 // Ops
 // ---------------------------------------------------------------------------------------------
 struct LeakyFwdOp {
+    static constexpr int NDER = 0, NROWP = 0;
     static constexpr int NIN = 1, NOUT = 1;
     static constexpr bool REVERSE = false;
     const float *in[1];
@@ -257,6 +274,7 @@ struct LeakyFwdOp {
 // reverse pass of the leaky integrator; optional alpha gradient and optional input-gradient store
 template <bool ALPHA, bool WRITE_GI>
 struct LeakyBwdOp {
+    static constexpr int NDER = 0, NROWP = 0;
     static constexpr int NIN = ALPHA ? 2 : 1, NOUT = WRITE_GI ? 1 : 0;
     static constexpr bool REVERSE = true;
     const float *in[NIN];                                     // [0] output_grad, [1] forward output
@@ -286,11 +304,20 @@ struct LeakyBwdOp {
     }
 };
 
+__device__ __forceinline__ f32x4 spike_count4(f32x4 v, float theta, unsigned cap)
+{
+    return f32x4{spike_count(v.x, theta, cap), spike_count(v.y, theta, cap), spike_count(v.z, theta, cap),
+                 spike_count(v.w, theta, cap)};
+}
+
 struct LifFwdOp {
-    static constexpr int NIN = 1, NOUT = 2;                   // out[0] = v_mem (in place of x), out[1] = spikes
+    // out[0] = v_mem (in place of x); the spike raster is a function of v_mem and the row's
+    // threshold, so it is produced on the way out instead of occupying a second tile
+    static constexpr int NIN = 1, NOUT = 1, NDER = 1, NROWP = 1, DER_SRC = 0;
     static constexpr bool REVERSE = false;
     const float *in[1];
-    float *out[2];
+    float *out[1];
+    float *der;
     const float *v_init, *alpha, *c, *theta, *theta_low;
     int apply_low;
     unsigned cap;
@@ -304,6 +331,8 @@ struct LifFwdOp {
         s.lo = apply_low ? theta_low[row] : 0.f;
         s.cnt = 0.f;
     }
+    __device__ __forceinline__ void stash(const State &s, float *p) const { p[0] = s.th; }
+    __device__ __forceinline__ f32x4 derive(const float *p, f32x4 v) const { return spike_count4(v, p[0], cap); }
     __device__ __forceinline__ void step(State &s, const float *x, float *y) const
     {
         float v = __fsub_rn(s.v, __fmul_rn(s.cnt, s.c));
@@ -313,7 +342,52 @@ struct LifFwdOp {
         s.cnt = spike_count(v, s.th, cap);
         s.v = v;
         y[0] = v;
-        y[1] = s.cnt;
+    }
+    __device__ __forceinline__ void finish(State &, int64_t) const {}
+};
+
+// Synapse + membrane in one pass (what the layer otherwise composes from a scaling, a leaky
+// integrator, another scaling and the spiking stage):
+//   xin = decay_early ? x * a_syn : x;   i = i * a_syn + xin;   u = norm_input ? (1 - a_mem) * i : i
+//   v = (v - count*c) * a_mem + u;  clamp;  count from v
+// out[0] = v_mem (in place of x), out[1] = i_syn, derived = spikes
+struct SynLifFwdOp {
+    static constexpr int NIN = 1, NOUT = 2, NDER = 1, NROWP = 1, DER_SRC = 0;
+    static constexpr bool REVERSE = false;
+    const float *in[1];
+    float *out[2];
+    float *der;
+    const float *v_init, *i_init, *alpha_mem, *alpha_syn, *c, *theta, *theta_low;
+    int apply_low, decay_early, norm_input;
+    unsigned cap;
+    struct State { float v, i, am, as, k, c, th, lo, cnt; };
+    __device__ __forceinline__ void init(State &s, int64_t row, bool) const
+    {
+        s.v = v_init[row];
+        s.i = i_init[row];
+        s.am = alpha_mem[row];
+        s.as = alpha_syn[row];
+        s.k = __fsub_rn(1.0f, s.am);
+        s.c = c[row];
+        s.th = theta[row];
+        s.lo = apply_low ? theta_low[row] : 0.f;
+        s.cnt = 0.f;
+    }
+    __device__ __forceinline__ void stash(const State &s, float *p) const { p[0] = s.th; }
+    __device__ __forceinline__ f32x4 derive(const float *p, f32x4 v) const { return spike_count4(v, p[0], cap); }
+    __device__ __forceinline__ void step(State &s, const float *x, float *y) const
+    {
+        const float xin = decay_early ? __fmul_rn(x[0], s.as) : x[0];
+        s.i = __fadd_rn(__fmul_rn(s.i, s.as), xin);
+        const float u = norm_input ? __fmul_rn(s.k, s.i) : s.i;
+        float v = __fsub_rn(s.v, __fmul_rn(s.cnt, s.c));
+        v = __fmul_rn(v, s.am);
+        v = __fadd_rn(v, u);
+        if (apply_low && v < s.lo) v = s.lo;
+        s.cnt = spike_count(v, s.th, cap);
+        s.v = v;
+        y[0] = v;
+        y[1] = s.i;
     }
     __device__ __forceinline__ void finish(State &, int64_t) const {}
 };
@@ -323,6 +397,7 @@ struct LifFwdOp {
 //   (HAS_GV) and the surrogate tensor (KIND == EXODUS_SURR_TENSOR)
 template <int KIND, bool HAS_GV, bool ALPHA>
 struct LifBwdOp {
+    static constexpr int NDER = 0, NROWP = 0;
     static constexpr int GV_SLOT = 2, SURR_SLOT = HAS_GV ? 3 : 2;
     static constexpr int NIN = 2 + (HAS_GV ? 1 : 0) + (KIND == EXODUS_SURR_TENSOR ? 1 : 0), NOUT = 1;
     static constexpr bool REVERSE = true;
@@ -381,8 +456,93 @@ struct LifBwdOp {
     }
 };
 
+// Reverse pass of the fused synapse + membrane stage.  With lambda_t = dL/du_t (membrane adjoint)
+// and mu_t = dL/di_t (synapse adjoint):
+//   lambda_t = nc_t (g_t + (a_mem - a_mem c s_t) lambda_{t+1}),   g_t = s_t * grad_spikes_t [+ grad_vmem_t]
+//   mu_t     = a_syn mu_{t+1} + k lambda_t [+ grad_isyn_t],       k = norm_input ? 1 - a_mem : 1
+//   grad_x_t = decay_early ? a_syn mu_t : mu_t
+//   grad_alpha_mem = sum_t lambda_t vpost_{t-1}  -  (norm_input ? sum_t lambda_t i_t : 0)
+//   grad_alpha_syn = decay_early ? (sum_t mu_t i_t) / a_syn : sum_t mu_t i_{t-1}
+//   grad_v_init = a_mem lambda_0,  grad_i_init = a_syn mu_0
+// slots: 0 grad_spikes (in) / grad_x (out), 1 v_mem, 2 i_syn, then grad_vmem and grad_isyn (EXTRA)
+template <int KIND, bool EXTRA>
+struct SynLifBwdOp {
+    static_assert(KIND != EXODUS_SURR_TENSOR, "the fused stage evaluates its surrogate in-kernel");
+    static constexpr int NDER = 0, NROWP = 0;
+    static constexpr int NIN = EXTRA ? 5 : 3, NOUT = 1;
+    static constexpr bool REVERSE = true;
+    const float *in[NIN];
+    float *out[1];
+    const float *v_init, *i_init, *alpha_mem, *alpha_syn, *c, *theta, *theta_low;
+    float *alpha_mem_grad, *alpha_syn_grad, *v_init_grad, *i_init_grad;
+    int apply_low, decay_early, norm_input;
+    unsigned cap;
+    float p0, p1;
+    struct State { float lam, mu, am, as, amc, k, c, th, lo, ra, rb; double acc_m, acc_s; };
+    __device__ __forceinline__ void init(State &s, int64_t row, bool) const
+    {
+        s.lam = 0.f;
+        s.mu = 0.f;
+        s.am = alpha_mem[row];
+        s.as = alpha_syn[row];
+        s.c = c[row];
+        s.amc = __fmul_rn(s.am, s.c);
+        s.k = norm_input ? __fsub_rn(1.0f, s.am) : 1.0f;
+        s.th = theta[row];
+        s.lo = apply_low ? theta_low[row] : 0.f;
+        s.acc_m = 0.0;
+        s.acc_s = 0.0;
+        if (KIND == EXODUS_SURR_SINGLE_EXP) {
+            s.ra = __fmul_rn(s.th, p0);
+            s.rb = __fdiv_rn(p1, s.ra);
+        } else if (KIND == EXODUS_SURR_PERIODIC_EXP) {
+            s.ra = __fmul_rn(s.th, 0.5f);
+            s.rb = 0.f;
+        } else {
+            s.ra = __fsub_rn(s.th, p0);
+            s.rb = __fdiv_rn(1.f, s.th);
+        }
+    }
+    __device__ __forceinline__ void step(State &s, const float *x, float *y) const
+    {
+        const float v = x[1], i = x[2];
+        const float sg = surrogate<KIND>(v, s.th, p0, p1, s.ra, s.rb);
+        float g = __fmul_rn(sg, x[0]);
+        if constexpr (EXTRA) g = __fadd_rn(g, x[3]);
+        const float vpost = __fsub_rn(v, __fmul_rn(s.c, spike_count(v, s.th, cap)));
+        s.acc_m += static_cast<double>(s.lam) * static_cast<double>(vpost);         // lambda_{u+1} * vpost_u
+        if (!decay_early) s.acc_s += static_cast<double>(s.mu) * static_cast<double>(i);   // mu_{u+1} * i_u
+        const float f = __fsub_rn(s.am, __fmul_rn(s.amc, sg));
+        const float lam = __fadd_rn(g, __fmul_rn(f, s.lam));
+        s.lam = (apply_low && !(v > s.lo)) ? 0.f : lam;
+        if (norm_input) s.acc_m -= static_cast<double>(s.lam) * static_cast<double>(i);
+        float du = __fmul_rn(s.lam, s.k);
+        if constexpr (EXTRA) du = __fadd_rn(du, x[4]);
+        s.mu = __fadd_rn(__fmul_rn(s.mu, s.as), du);
+        if (decay_early) s.acc_s += static_cast<double>(s.mu) * static_cast<double>(i);    // mu_u * i_u
+        y[0] = decay_early ? __fmul_rn(s.mu, s.as) : s.mu;
+    }
+    __device__ __forceinline__ void finish(State &s, int64_t row) const
+    {
+        if (v_init_grad) v_init_grad[row] = __fmul_rn(s.am, s.lam);
+        if (i_init_grad) i_init_grad[row] = __fmul_rn(s.as, s.mu);
+        if (alpha_mem_grad) {
+            s.acc_m += static_cast<double>(s.lam) * static_cast<double>(v_init[row]);
+            alpha_mem_grad[row] = static_cast<float>(s.acc_m);
+        }
+        if (alpha_syn_grad) {
+            if (decay_early)
+                s.acc_s = s.acc_s / static_cast<double>(s.as);
+            else
+                s.acc_s += static_cast<double>(s.mu) * static_cast<double>(i_init[row]);
+            alpha_syn_grad[row] = static_cast<float>(s.acc_s);
+        }
+    }
+};
+
 // counterpart of the reference's lifBackward: surrogate, g and the clip mask come as tensors
 struct LifBwdTensorsOp {
+    static constexpr int NDER = 0, NROWP = 0;
     static constexpr int NIN = 3, NOUT = 1;                   // in: g, surr, not_clipped
     static constexpr bool REVERSE = true;
     const float *in[3];
@@ -406,6 +566,7 @@ struct LifBwdTensorsOp {
 
 // counterpart of the reference's lifBackwardAlpha: forward in time, D recurrence
 struct LifBwdAlphaTensorsOp {
+    static constexpr int NDER = 0, NROWP = 0;
     static constexpr int NIN = 4, NOUT = 0;                   // in: g, surr, not_clipped, v_post
     static constexpr bool REVERSE = false;
     const float *in[4];
@@ -456,7 +617,7 @@ template <class Op, int TT>
 int launch(const Op &op, int64_t n, int64_t t, void *stream)
 {
     constexpr int NSLOT = Op::NIN > Op::NOUT ? Op::NIN : Op::NOUT;
-    const size_t lds_bytes = static_cast<size_t>(NSLOT) * WAVE * TT * sizeof(float);
+    const size_t lds_bytes = (static_cast<size_t>(NSLOT) * WAVE * TT + WAVE * Op::NROWP) * sizeof(float);
     const int64_t n_blocks = (n + WAVE - 1) / WAVE;
     if (n_blocks > 0x7fffffffLL) return hipErrorInvalidValue;
     bool vec = (t % 4) == 0;
@@ -521,6 +682,44 @@ int dispatch_lif_bwd(bool has_gv, bool want_alpha, float *input_grad, float *alp
 #undef EXODUS_CALL
 }
 
+template <int KIND, bool EXTRA>
+int launch_synlif_bwd(float *grad_input, float *alpha_mem_grad, float *alpha_syn_grad, float *v_init_grad,
+                      float *i_init_grad, const float *grad_spikes, const float *grad_vmem, const float *grad_isyn,
+                      const float *vmem, const float *isyn, const float *v_init, const float *i_init,
+                      const float *alpha_mem, const float *alpha_syn, const float *c, const float *theta,
+                      const float *theta_low, int apply_low, int max_spikes, int decay_early, int norm_input,
+                      float p0, float p1, int64_t n, int64_t t, void *stream)
+{
+    using Op = SynLifBwdOp<KIND, EXTRA>;
+    Op op;
+    op.in[0] = grad_spikes;
+    op.in[1] = vmem;
+    op.in[2] = isyn;
+    if constexpr (EXTRA) {
+        op.in[3] = grad_vmem;
+        op.in[4] = grad_isyn;
+    }
+    op.out[0] = grad_input;
+    op.v_init = v_init;
+    op.i_init = i_init;
+    op.alpha_mem = alpha_mem;
+    op.alpha_syn = alpha_syn;
+    op.c = c;
+    op.theta = theta;
+    op.theta_low = theta_low;
+    op.alpha_mem_grad = alpha_mem_grad;
+    op.alpha_syn_grad = alpha_syn_grad;
+    op.v_init_grad = v_init_grad;
+    op.i_init_grad = i_init_grad;
+    op.apply_low = apply_low;
+    op.decay_early = decay_early;
+    op.norm_input = norm_input;
+    op.cap = static_cast<unsigned>(max_spikes);
+    op.p0 = p0;
+    op.p1 = p1;
+    return launch<Op, 16>(op, n, t, stream);
+}
+
 }  // namespace
 
 // ---------------------------------------------------------------------------------------------
@@ -550,7 +749,7 @@ EXODUS_API int exodus_lif_forward(float *out_spikes, float *out_vmem, const floa
     LifFwdOp op;
     op.in[0] = input;
     op.out[0] = out_vmem;
-    op.out[1] = out_spikes;
+    op.der = out_spikes;
     op.v_init = vmem_post_initial;
     op.alpha = alpha;
     op.c = membr_subtract;
@@ -689,6 +888,80 @@ EXODUS_API int exodus_lif_backward_fused(float *input_grad, float *alpha_grad, f
         default: return hipErrorInvalidValue;
     }
 #undef EXODUS_KIND
+}
+
+EXODUS_API int exodus_synlif_forward(float *out_spikes, float *out_vmem, float *out_isyn, const float *input,
+                                     const float *vmem_post_initial, const float *isyn_initial,
+                                     const float *alpha_mem, const float *alpha_syn, const float *membr_subtract,
+                                     const float *theta, const float *theta_low, int apply_theta_low,
+                                     int max_num_spikes, int decay_early, int norm_input, int64_t n, int64_t t,
+                                     void *stream)
+{
+    if (bad_dims(n, t)) return hipErrorInvalidValue;
+    if (n == 0 || t == 0) return hipSuccess;
+    if (!out_spikes || !out_vmem || !out_isyn || !input || !vmem_post_initial || !isyn_initial || !alpha_mem ||
+        !alpha_syn || !membr_subtract || !theta || (apply_theta_low && !theta_low))
+        return hipErrorInvalidValue;
+    SynLifFwdOp op;
+    op.in[0] = input;
+    op.out[0] = out_vmem;
+    op.out[1] = out_isyn;
+    op.der = out_spikes;
+    op.v_init = vmem_post_initial;
+    op.i_init = isyn_initial;
+    op.alpha_mem = alpha_mem;
+    op.alpha_syn = alpha_syn;
+    op.c = membr_subtract;
+    op.theta = theta;
+    op.theta_low = theta_low;
+    op.apply_low = apply_theta_low ? 1 : 0;
+    op.decay_early = decay_early ? 1 : 0;
+    op.norm_input = norm_input ? 1 : 0;
+    op.cap = static_cast<unsigned>(max_num_spikes);
+    return launch<SynLifFwdOp, 32>(op, n, t, stream);
+}
+
+EXODUS_API int exodus_synlif_backward(float *grad_input, float *alpha_mem_grad, float *alpha_syn_grad,
+                                      float *vmem_init_grad, float *isyn_init_grad, const float *grad_spikes,
+                                      const float *grad_vmem, const float *grad_isyn, const float *vmem,
+                                      const float *isyn, const float *vmem_post_initial, const float *isyn_initial,
+                                      const float *alpha_mem, const float *alpha_syn, const float *membr_subtract,
+                                      const float *theta, const float *theta_low, int apply_theta_low,
+                                      int max_num_spikes, int decay_early, int norm_input, int surrogate_kind,
+                                      float surr_p0, float surr_p1, int64_t n, int64_t t, void *stream)
+{
+    if (bad_dims(n, t)) return hipErrorInvalidValue;
+    if (n == 0 || t == 0) return hipSuccess;
+    if (!grad_input || !grad_spikes || !vmem || !isyn || !alpha_mem || !alpha_syn || !membr_subtract || !theta)
+        return hipErrorInvalidValue;
+    if (apply_theta_low && !theta_low) return hipErrorInvalidValue;
+    if (alpha_mem_grad && !vmem_post_initial) return hipErrorInvalidValue;
+    if (alpha_syn_grad && !decay_early && !isyn_initial) return hipErrorInvalidValue;
+    if ((grad_vmem == nullptr) != (grad_isyn == nullptr)) return hipErrorInvalidValue;   // both or neither
+    const bool extra = grad_vmem != nullptr;
+#define EXODUS_SYN(K)                                                                                           \
+    do {                                                                                                        \
+        if (extra)                                                                                              \
+            return launch_synlif_bwd<K, true>(grad_input, alpha_mem_grad, alpha_syn_grad, vmem_init_grad,       \
+                                              isyn_init_grad, grad_spikes, grad_vmem, grad_isyn, vmem, isyn,    \
+                                              vmem_post_initial, isyn_initial, alpha_mem, alpha_syn,            \
+                                              membr_subtract, theta, theta_low, apply_theta_low ? 1 : 0,        \
+                                              max_num_spikes, decay_early ? 1 : 0, norm_input ? 1 : 0, surr_p0, \
+                                              surr_p1, n, t, stream);                                           \
+        return launch_synlif_bwd<K, false>(grad_input, alpha_mem_grad, alpha_syn_grad, vmem_init_grad,          \
+                                           isyn_init_grad, grad_spikes, grad_vmem, grad_isyn, vmem, isyn,       \
+                                           vmem_post_initial, isyn_initial, alpha_mem, alpha_syn,               \
+                                           membr_subtract, theta, theta_low, apply_theta_low ? 1 : 0,           \
+                                           max_num_spikes, decay_early ? 1 : 0, norm_input ? 1 : 0, surr_p0,    \
+                                           surr_p1, n, t, stream);                                              \
+    } while (0)
+    switch (surrogate_kind) {
+        case EXODUS_SURR_SINGLE_EXP: EXODUS_SYN(EXODUS_SURR_SINGLE_EXP);
+        case EXODUS_SURR_PERIODIC_EXP: EXODUS_SYN(EXODUS_SURR_PERIODIC_EXP);
+        case EXODUS_SURR_HEAVISIDE: EXODUS_SYN(EXODUS_SURR_HEAVISIDE);
+        default: return hipErrorInvalidValue;
+    }
+#undef EXODUS_SYN
 }
 
 }  // extern "C"

@@ -37,6 +37,8 @@ _SIGNATURES = {
     "exodus_leaky_backward_alpha": ([_p] * 5 + [_i64, _i64, _p], _int),
     "exodus_leaky_backward_fused": ([_p] * 7 + [_i64, _i64, _p], _int),
     "exodus_lif_backward_fused": ([_p] * 12 + [_int, _int, _int, _f, _f, _i64, _i64, _p], _int),
+    "exodus_synlif_forward": ([_p] * 11 + [_int, _int, _int, _int, _i64, _i64, _p], _int),
+    "exodus_synlif_backward": ([_p] * 17 + [_int, _int, _int, _int, _int, _f, _f, _i64, _i64, _p], _int),
 }
 
 
@@ -286,3 +288,71 @@ def lifBackwardFused(gradSpikes, gradVmem, vmem, vmemPostInitial, alpha, membrSu
                                              float(surrP0), float(surrP1), n, t, _stream(vmem)),
                "exodus_lif_backward_fused")
     return inputGrad, alphaGrad, initGrad
+
+
+def synLifForward(input, vmemPostInitial, isynInitial, alphaMem, alphaSyn, membrSubtract, theta, thetaLow,
+                  applyThetaLow: bool, maxNumSpikes: int, decayEarly: bool, normInput: bool,
+                  out: Optional[tuple] = None):
+    """Fused synapse + membrane forward: returns (spikes, vmem, isyn), all (n, t)."""
+    _dev(input, "input")
+    if input.ndim != 2:
+        raise RuntimeError("input must be 2-D (rows, time)")
+    n, t = input.shape
+    for nm, x in (("vmemPostInitial", vmemPostInitial), ("isynInitial", isynInitial), ("alphaMem", alphaMem),
+                  ("alphaSyn", alphaSyn), ("membrSubtract", membrSubtract), ("theta", theta)):
+        _rows(_dev(x, nm, input), nm, n)
+    if applyThetaLow:
+        _rows(_dev(thetaLow, "thetaLow", input), "thetaLow", n)
+    else:
+        thetaLow = None
+    if out is None:
+        out = (torch.empty_like(input), torch.empty_like(input), torch.empty_like(input))
+    spikes, vmem, isyn = out
+    for nm, x in (("spikes", spikes), ("vmem", vmem), ("isyn", isyn)):
+        _mat(_dev(x, nm, input), nm, n, t)
+    with torch.cuda.device(input.device):
+        _check(lib.exodus_synlif_forward(_ptr(spikes), _ptr(vmem), _ptr(isyn), _ptr(input), _ptr(vmemPostInitial),
+                                         _ptr(isynInitial), _ptr(alphaMem), _ptr(alphaSyn), _ptr(membrSubtract),
+                                         _ptr(theta), _ptr(thetaLow), int(bool(applyThetaLow)), int(maxNumSpikes),
+                                         int(bool(decayEarly)), int(bool(normInput)), n, t, _stream(input)),
+               "exodus_synlif_forward")
+    return spikes, vmem, isyn
+
+
+def synLifBackward(gradSpikes, gradVmem, gradIsyn, vmem, isyn, vmemPostInitial, isynInitial, alphaMem, alphaSyn,
+                   membrSubtract, theta, thetaLow, applyThetaLow: bool, maxNumSpikes: int, decayEarly: bool,
+                   normInput: bool, surrogateKind: int, surrP0: float, surrP1: float,
+                   inputGrad: Optional[torch.Tensor] = None):
+    """Fused reverse pass: returns (inputGrad, alphaMemGrad, alphaSynGrad, vmemInitGrad, isynInitGrad)."""
+    _dev(vmem, "vmem")
+    if vmem.ndim != 2:
+        raise RuntimeError("vmem must be 2-D (rows, time)")
+    n, t = vmem.shape
+    _mat(_dev(gradSpikes, "gradSpikes", vmem), "gradSpikes", n, t)
+    _mat(_dev(isyn, "isyn", vmem), "isyn", n, t)
+    if (gradVmem is None) != (gradIsyn is None):
+        raise RuntimeError("gradVmem and gradIsyn must be given together")
+    if gradVmem is not None:
+        _mat(_dev(gradVmem, "gradVmem", vmem), "gradVmem", n, t)
+        _mat(_dev(gradIsyn, "gradIsyn", vmem), "gradIsyn", n, t)
+    for nm, x in (("vmemPostInitial", vmemPostInitial), ("isynInitial", isynInitial), ("alphaMem", alphaMem),
+                  ("alphaSyn", alphaSyn), ("membrSubtract", membrSubtract), ("theta", theta)):
+        _rows(_dev(x, nm, vmem), nm, n)
+    if applyThetaLow:
+        _rows(_dev(thetaLow, "thetaLow", vmem), "thetaLow", n)
+    else:
+        thetaLow = None
+    if inputGrad is None:
+        inputGrad = torch.empty_like(vmem)
+    else:
+        _mat(_dev(inputGrad, "inputGrad", vmem), "inputGrad", n, t)
+    per_row = [torch.zeros_like(alphaMem) for _ in range(4)]
+    with torch.cuda.device(vmem.device):
+        _check(lib.exodus_synlif_backward(_ptr(inputGrad), *[_ptr(x) for x in per_row], _ptr(gradSpikes),
+                                          _ptr(gradVmem), _ptr(gradIsyn), _ptr(vmem), _ptr(isyn),
+                                          _ptr(vmemPostInitial), _ptr(isynInitial), _ptr(alphaMem), _ptr(alphaSyn),
+                                          _ptr(membrSubtract), _ptr(theta), _ptr(thetaLow),
+                                          int(bool(applyThetaLow)), int(maxNumSpikes), int(bool(decayEarly)),
+                                          int(bool(normInput)), int(surrogateKind), float(surrP0), float(surrP1),
+                                          n, t, _stream(vmem)), "exodus_synlif_backward")
+    return (inputGrad, *per_row)
