@@ -8,7 +8,7 @@ tolerance rtol 1e-4 / atol 1e-5.
 import pytest
 import torch
 
-from _util import ATOL, RTOL, assert_close, gen, lif_case
+from _util import ATOL, RTOL, assert_close, assert_close_rowscaled, gen, lif_case
 
 pytestmark = pytest.mark.gpu
 
@@ -101,7 +101,9 @@ def test_lif_backward_tensor_entry_points(hip, ref, n, t):
         assert_close(got, want, f"lifBackwardAlpha gate={gate}", **tol)
 
 
-SURROGATES = [("single", 1, 0.5, 1.0), ("single", 1, 0.3, 2.0), ("periodic", 2, 0.5, 1.0), ("periodic", 2, 0.25, 0.7),
+# parameters chosen so that |alpha (1 - c s)| stays <= 1 for the random rows of lif_case (c <= 0.8,
+# theta >= 0.5): the gradient recurrence is then contractive and the element-wise tolerance applies
+SURROGATES = [("single", 1, 0.5, 1.0), ("single", 1, 0.7, 0.6), ("periodic", 2, 0.5, 1.0), ("periodic", 2, 0.25, 0.7),
               ("heaviside", 3, 0.5, 0.0), ("heaviside", 3, 1.0, 0.0)]
 
 
@@ -142,6 +144,27 @@ def test_lif_backward_fused(hip, ref, n, t, name, kind, p0, p1, cap, use_lo, use
     gi3, ga3, ginit3 = hip.lifBackwardFused(D(c["go"]), D(gv), D(wv), None, D(c["alpha"]), D(c["c"]), D(c["theta"]),
                                             D(c["lo"]), use_lo, cap, kind, p0, p1)
     assert ga3 is None and torch.equal(gi3, gi) and torch.equal(ginit3, ginit)
+
+
+def test_lif_backward_fused_expanding_recurrence(hip, ref):
+    """A sharp, tall surrogate (width 0.3, scale 2) makes |alpha (1 - c s)| reach ~8: gradients grow
+    to 1e5 along a row and fp32 rounding is amplified alike in the reference's quadratic sum and in
+    the reverse recurrence.  Both are then accurate relative to the row's magnitude, which is what
+    is asserted; the float64 recurrence is the yardstick."""
+    n, t = 1000, 300
+    c = lif_case(n * 1000 + t + 4, n, t, lo=False)
+    fn = ref.SingleExponential(0.3, 2.0)
+    ws, wv = ref.lif_forward(c["x"], c["v0"], c["alpha"], c["c"], c["theta"], None, False, -1)
+    surr = fn(wv, c["theta"].unsqueeze(1))
+    gi64, ga64, _ = ref.lif_backward_recurrence_f64(surr, surr * c["go"], torch.ones_like(surr), c["alpha"], c["c"],
+                                                    wv - c["c"].unsqueeze(1) * ws, c["v0"])
+    want_gi, _, _ = ref.integrate_and_fire_backward(c["go"], None, wv, ws, c["v0"], c["alpha"], c["c"], c["theta"],
+                                                    None, fn, False)
+    gi, ga, _ = hip.lifBackwardFused(D(c["go"]), None, D(wv), D(c["v0"]), D(c["alpha"]), D(c["c"]), D(c["theta"]),
+                                     None, False, -1, 1, 0.3, 2.0, needAlphaGrad=True)
+    assert_close_rowscaled(want_gi, gi64, "reference quadratic sum vs float64")
+    assert_close_rowscaled(gi, gi64, "HIP reverse recurrence vs float64")
+    assert_close_rowscaled(ga, ga64, "HIP alpha gradient vs float64", atol=ATOL * t ** 0.5)
 
 
 def test_unaligned_pointers_take_the_scalar_path(hip, ref):
