@@ -22,6 +22,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 #include "exodus_hip.h"
 
 namespace {
@@ -29,6 +31,30 @@ namespace {
 constexpr int WAVE = 64;
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));    // one 16-byte chunk = 4 time steps
+
+// streaming (non-temporal) hints on the (n,t) tensors, which are read once and written once
+#ifndef EXODUS_NT_LOAD
+#define EXODUS_NT_LOAD 1
+#endif
+#ifndef EXODUS_NT_STORE
+#define EXODUS_NT_STORE 1
+#endif
+template <class T> __device__ __forceinline__ T ld_stream(const T *p)
+{
+#if EXODUS_NT_LOAD
+    return __builtin_nontemporal_load(p);
+#else
+    return *p;
+#endif
+}
+template <class T> __device__ __forceinline__ void st_stream(T v, T *p)
+{
+#if EXODUS_NT_STORE
+    __builtin_nontemporal_store(v, p);
+#else
+    *p = v;
+#endif
+}
 
 __device__ __forceinline__ void wave_sync()
 {
@@ -55,18 +81,19 @@ struct Geom {
 
 template <bool VEC>
 __device__ __forceinline__ f32x4 load4(const float *__restrict__ base, int64_t row, int64_t n_rows,
-                                        int64_t t, int64_t n_steps)
+                                       int64_t t, int64_t n_steps)
 {
+    // t may be negative (before the row's first step) or beyond the row's end: those lanes load nothing
     f32x4 v = f32x4{0.f, 0.f, 0.f, 0.f};
     if (row < n_rows) {
         const float *p = base + row * n_steps + t;
         if (VEC) {
-            if (t + 3 < n_steps) v = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(p));
+            if (t >= 0 && t + 3 < n_steps) v = ld_stream(reinterpret_cast<const f32x4 *>(p));
         } else {
-            if (t + 0 < n_steps) v.x = __builtin_nontemporal_load(p + 0);
-            if (t + 1 < n_steps) v.y = __builtin_nontemporal_load(p + 1);
-            if (t + 2 < n_steps) v.z = __builtin_nontemporal_load(p + 2);
-            if (t + 3 < n_steps) v.w = __builtin_nontemporal_load(p + 3);
+            if (t + 0 >= 0 && t + 0 < n_steps) v.x = ld_stream(p + 0);
+            if (t + 1 >= 0 && t + 1 < n_steps) v.y = ld_stream(p + 1);
+            if (t + 2 >= 0 && t + 2 < n_steps) v.z = ld_stream(p + 2);
+            if (t + 3 >= 0 && t + 3 < n_steps) v.w = ld_stream(p + 3);
         }
     }
     return v;
@@ -79,12 +106,12 @@ __device__ __forceinline__ void store4(float *__restrict__ base, int64_t row, in
     if (row < n_rows) {
         float *p = base + row * n_steps + t;
         if (VEC) {
-            if (t + 3 < n_steps) __builtin_nontemporal_store(v, reinterpret_cast<f32x4 *>(p));
+            if (t >= 0 && t + 3 < n_steps) st_stream(v, reinterpret_cast<f32x4 *>(p));
         } else {
-            if (t + 0 < n_steps) __builtin_nontemporal_store(v.x, p + 0);
-            if (t + 1 < n_steps) __builtin_nontemporal_store(v.y, p + 1);
-            if (t + 2 < n_steps) __builtin_nontemporal_store(v.z, p + 2);
-            if (t + 3 < n_steps) __builtin_nontemporal_store(v.w, p + 3);
+            if (t + 0 >= 0 && t + 0 < n_steps) st_stream(v.x, p + 0);
+            if (t + 1 >= 0 && t + 1 < n_steps) st_stream(v.y, p + 1);
+            if (t + 2 >= 0 && t + 2 < n_steps) st_stream(v.z, p + 2);
+            if (t + 3 >= 0 && t + 3 < n_steps) st_stream(v.w, p + 3);
         }
     }
 }
@@ -102,9 +129,17 @@ __device__ __forceinline__ void put(f32x4 &v, int e, float x) { v[e] = x; }
 //                      NROWP per-row constants: it is computed while the tile is written back
 //                      (stash(State&, float* p) / derive(const float* p, f32x4 v)), so it needs no
 //                      LDS tile of its own
+//
+// Tiles are aligned to memory, not to the rows.  Row r starts at float offset base + r*n_steps,
+// which in general is not a multiple of the tile length, so a tile that started at the row's first
+// step would straddle 128-byte lines on every access.  Instead tile k of row r covers the steps
+// [k*TT - shift_r, (k+1)*TT - shift_r) with shift_r = (base + r*n_steps) mod TT: every wave-wide
+// load and store then moves whole aligned TT*4-byte segments, and only the first and last tile
+// of a row are partial (their out-of-row steps are masked per lane).
 // ---------------------------------------------------------------------------------------------
 template <class Op, int TT, bool VEC>
-__global__ void __launch_bounds__(WAVE) scan_kernel(const Op op, const int64_t n_rows, const int64_t n_steps)
+__global__ void __launch_bounds__(WAVE) scan_kernel(const Op op, const int64_t n_rows, const int64_t n_steps,
+                                                    const int64_t n_tiles, const int base_shift)
 {
     using G = Geom<TT>;
     constexpr int NIN = Op::NIN, NOUT = Op::NOUT;
@@ -131,39 +166,29 @@ __global__ void __launch_bounds__(WAVE) scan_kernel(const Op op, const int64_t n
 
     const int l_chunk = lane % G::CPR;                        // which 16 B of the segment this lane moves
     const int l_row = lane / G::CPR;                          // first row this lane moves
-    const int64_t n_tiles = (n_steps + TT - 1) / TT;
+    // misalignment of a row's first step relative to a TT-float boundary
+    auto shift_of = [&](int64_t row) { return static_cast<int>((base_shift + row * n_steps) & (TT - 1)); };
+    const int my_shift = shift_of(my_row);
+    int mv_shift[G::NLD];                                     // shifts of the rows this lane moves
+#pragma unroll
+    for (int i = 0; i < G::NLD; ++i) mv_shift[i] = shift_of(row0 + l_row + i * G::RPI);
 
     f32x4 pre[NIN > 0 ? NIN : 1][G::NLD];
 
     auto fetch = [&](int64_t tile) {
-        const int64_t t = tile * TT + 4 * l_chunk;
 #pragma unroll
-        for (int j = 0; j < NIN; ++j)
+        for (int i = 0; i < G::NLD; ++i) {
+            const int64_t t = tile * TT - mv_shift[i] + 4 * l_chunk;
 #pragma unroll
-            for (int i = 0; i < G::NLD; ++i)
+            for (int j = 0; j < NIN; ++j)
                 pre[j][i] = load4<VEC>(op.in[j], row0 + l_row + i * G::RPI, n_rows, t, n_steps);
+        }
     };
 
-    fetch(Op::REVERSE ? n_tiles - 1 : 0);
-
-    for (int64_t it = 0; it < n_tiles; ++it) {
-        const int64_t tile = Op::REVERSE ? n_tiles - 1 - it : it;
-        const int64_t t0 = tile * TT;
-        const int n_valid = (n_steps - t0) < TT ? static_cast<int>(n_steps - t0) : TT;
-
-        // registers -> LDS
-#pragma unroll
-        for (int j = 0; j < NIN; ++j)
-#pragma unroll
-            for (int i = 0; i < G::NLD; ++i)
-                *reinterpret_cast<f32x4 *>(lds + j * TILE + G::off(l_row + i * G::RPI, l_chunk)) = pre[j][i];
-
-        // next tile's loads stay in flight during the compute and store phases below
-        if (it + 1 < n_tiles) fetch(Op::REVERSE ? tile - 1 : tile + 1);
-
-        wave_sync();
-
-        // the recurrence: lane = row, 4 steps per 16-byte chunk
+    // the recurrence over one tile: lane = row, 4 steps per 16-byte chunk.  GUARD masks the steps
+    // that fall outside the row (first and last tile only).
+    auto compute = [&](int64_t t_first, auto guard) {
+        constexpr bool GUARD = decltype(guard)::value;
 #pragma unroll
         for (int qq = 0; qq < G::CPR; ++qq) {
             const int q = Op::REVERSE ? G::CPR - 1 - qq : qq;
@@ -177,7 +202,8 @@ __global__ void __launch_bounds__(WAVE) scan_kernel(const Op op, const int64_t n
 #pragma unroll
             for (int ee = 0; ee < 4; ++ee) {
                 const int e = Op::REVERSE ? 3 - ee : ee;
-                if (4 * q + e < n_valid) {
+                const int64_t t = t_first + 4 * q + e;
+                if (!GUARD || (t >= 0 && t < n_steps)) {
                     float x[NIN > 0 ? NIN : 1];
                     float y[NOUT > 0 ? NOUT : 1];
 #pragma unroll
@@ -191,15 +217,40 @@ __global__ void __launch_bounds__(WAVE) scan_kernel(const Op op, const int64_t n
             for (int j = 0; j < NOUT; ++j)
                 *reinterpret_cast<f32x4 *>(lds + j * TILE + G::off(lane, q)) = yout[j];
         }
+    };
+
+    fetch(Op::REVERSE ? n_tiles - 1 : 0);
+
+    for (int64_t it = 0; it < n_tiles; ++it) {
+        const int64_t tile = Op::REVERSE ? n_tiles - 1 - it : it;
+
+        // registers -> LDS
+#pragma unroll
+        for (int j = 0; j < NIN; ++j)
+#pragma unroll
+            for (int i = 0; i < G::NLD; ++i)
+                *reinterpret_cast<f32x4 *>(lds + j * TILE + G::off(l_row + i * G::RPI, l_chunk)) = pre[j][i];
+
+        // next tile's loads stay in flight during the compute and store phases below
+        if (it + 1 < n_tiles) fetch(Op::REVERSE ? tile - 1 : tile + 1);
+
+        wave_sync();
+
+        // a tile is interior when it lies inside the row for every possible shift (0..TT-1)
+        const bool interior = tile >= 1 && (tile + 1) * TT <= n_steps;
+        if (interior)
+            compute(tile * TT - my_shift, std::false_type{});
+        else
+            compute(tile * TT - my_shift, std::true_type{});
 
         if (NOUT > 0) {
             wave_sync();
-            // LDS -> global, whole row segments per group of CPR lanes
-            const int64_t t = t0 + 4 * l_chunk;
+            // LDS -> global, whole aligned segments per group of CPR lanes
 #pragma unroll
-            for (int j = 0; j < NOUT; ++j)
+            for (int i = 0; i < G::NLD; ++i) {
+                const int64_t t = tile * TT - mv_shift[i] + 4 * l_chunk;
 #pragma unroll
-                for (int i = 0; i < G::NLD; ++i) {
+                for (int j = 0; j < NOUT; ++j) {
                     const f32x4 v = *reinterpret_cast<const f32x4 *>(lds + j * TILE + G::off(l_row + i * G::RPI, l_chunk));
                     store4<VEC>(op.out[j], row0 + l_row + i * G::RPI, n_rows, t, n_steps, v);
                     if constexpr (NDER > 0) {
@@ -208,6 +259,7 @@ __global__ void __launch_bounds__(WAVE) scan_kernel(const Op op, const int64_t n
                                         op.derive(rowp + (l_row + i * G::RPI) * NROWP, v));
                     }
                 }
+            }
         }
         wave_sync();
     }
@@ -623,12 +675,22 @@ int launch(const Op &op, int64_t n, int64_t t, void *stream)
     bool vec = (t % 4) == 0;
     for (int j = 0; j < Op::NIN; ++j) vec = vec && aligned16(op.in[j]);
     for (int j = 0; j < Op::NOUT; ++j) vec = vec && aligned16(op.out[j]);
+    // Tiles are aligned to the first tensor's address (allocators hand out >= 256-byte aligned
+    // blocks, so in practice every tensor shares this alignment).  Row shifts are
+    // (base_shift + r*t) mod TT, i.e. base_shift plus multiples of g = gcd(t, TT); the largest one
+    // decides how many tiles cover a row.
+    const void *first = Op::NIN > 0 ? static_cast<const void *>(op.in[0]) : static_cast<const void *>(op.out[0]);
+    const int base_shift = static_cast<int>((reinterpret_cast<uintptr_t>(first) / sizeof(float)) % TT);
+    int64_t g = t % TT == 0 ? TT : t % TT;
+    for (int64_t b = TT; b != 0;) { const int64_t r = g % b; g = b; b = r; }    // gcd(t mod TT, TT)
+    const int64_t max_shift = TT - g + (base_shift % g);
+    const int64_t n_tiles = (t - 1 + max_shift) / TT + 1;
     const dim3 grid(static_cast<unsigned>(n_blocks)), block(WAVE);
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (vec)
-        hipLaunchKernelGGL((scan_kernel<Op, TT, true>), grid, block, lds_bytes, s, op, n, t);
+        hipLaunchKernelGGL((scan_kernel<Op, TT, true>), grid, block, lds_bytes, s, op, n, t, n_tiles, base_shift);
     else
-        hipLaunchKernelGGL((scan_kernel<Op, TT, false>), grid, block, lds_bytes, s, op, n, t);
+        hipLaunchKernelGGL((scan_kernel<Op, TT, false>), grid, block, lds_bytes, s, op, n, t, n_tiles, base_shift);
     return static_cast<int>(hipGetLastError());
 }
 

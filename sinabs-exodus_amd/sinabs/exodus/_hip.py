@@ -16,7 +16,8 @@ from typing import Optional
 import torch  # must be imported before the library so both share one HIP runtime
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libexodus_hip.so")
+# EXODUS_HIP_LIBRARY may point at another build of the same ABI (e.g. one compiled with other flags)
+LIB_PATH = os.environ.get("EXODUS_HIP_LIBRARY") or os.path.join(_HERE, "libexodus_hip.so")
 
 SURR_TENSOR, SURR_SINGLE_EXP, SURR_PERIODIC_EXP, SURR_HEAVISIDE = 0, 1, 2, 3
 ABI_VERSION = 1
