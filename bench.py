@@ -167,6 +167,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c5", choices=list(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also launch one plain device copy of exactly 1 GiB before the timed region, so that a "
+                         "counter run (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE) has a kernel of known traffic "
+                         "to scale its readings by")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (rows shard across GPUs without exchange; "
@@ -181,6 +185,13 @@ def main():
     torch.cuda.set_device(dev)
     wl = build_workload(args.workload, torch, hip, act, dev)
     fwd, bwd, N, T = wl["fwd"], wl["bwd"], wl["N"], wl["T"]
+
+    if args.copy_probe:
+        src = torch.ones(1 << 28, device=dev)          # 2^28 floats = 1 GiB read + 1 GiB written
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     for _ in range(args.warmup):
         fwd(); bwd()

@@ -32,6 +32,15 @@ constexpr int WAVE = 64;
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));    // one 16-byte chunk = 4 time steps
 
+// Tile lengths (time steps per tile) by number of (n,t) tensors an op keeps in LDS.  Longer tiles
+// mean longer contiguous segments per row; more slots mean more LDS per wave.
+#ifndef EXODUS_TT_1
+#define EXODUS_TT_1 32    // one or two LDS slots
+#endif
+#ifndef EXODUS_TT_3
+#define EXODUS_TT_3 32    // three or more LDS slots
+#endif
+
 // streaming (non-temporal) hints on the (n,t) tensors, which are read once and written once
 #ifndef EXODUS_NT_LOAD
 #define EXODUS_NT_LOAD 1
@@ -720,8 +729,8 @@ int launch_lif_bwd(float *input_grad, float *alpha_grad, float *init_grad, const
     op.cap = static_cast<unsigned>(max_spikes);
     op.p0 = p0;
     op.p1 = p1;
-    if constexpr (Op::NIN <= 2) return launch<Op, 32>(op, n, t, stream);
-    else return launch<Op, 16>(op, n, t, stream);
+    if constexpr (Op::NIN <= 2) return launch<Op, EXODUS_TT_1>(op, n, t, stream);
+    else return launch<Op, EXODUS_TT_3>(op, n, t, stream);
 }
 
 template <int KIND>
@@ -779,7 +788,7 @@ int launch_synlif_bwd(float *grad_input, float *alpha_mem_grad, float *alpha_syn
     op.cap = static_cast<unsigned>(max_spikes);
     op.p0 = p0;
     op.p1 = p1;
-    return launch<Op, 16>(op, n, t, stream);
+    return launch<Op, EXODUS_TT_3>(op, n, t, stream);
 }
 
 }  // namespace
@@ -819,7 +828,7 @@ EXODUS_API int exodus_lif_forward(float *out_spikes, float *out_vmem, const floa
     op.theta_low = theta_low;
     op.apply_low = apply_theta_low ? 1 : 0;
     op.cap = static_cast<unsigned>(max_num_spikes);           // negative -> no cap
-    return launch<LifFwdOp, 32>(op, n, t, stream);
+    return launch<LifFwdOp, EXODUS_TT_1>(op, n, t, stream);
 }
 
 EXODUS_API int exodus_lif_backward(float *input_grad, const float *surr, const float *output_grad,
@@ -837,7 +846,7 @@ EXODUS_API int exodus_lif_backward(float *input_grad, const float *surr, const f
     op.out[0] = input_grad;
     op.alpha = alpha;
     op.csub = membr_subtract;
-    return launch<LifBwdTensorsOp, 16>(op, n, t, stream);
+    return launch<LifBwdTensorsOp, EXODUS_TT_3>(op, n, t, stream);
 }
 
 EXODUS_API int exodus_lif_backward_alpha(float *alpha_grad, const float *surr, const float *output_grad,
@@ -862,7 +871,7 @@ EXODUS_API int exodus_lif_backward_alpha(float *alpha_grad, const float *surr, c
     op.c = membr_subtract;
     op.alpha_grad = alpha_grad;
     op.gate_initial = gate_initial ? 1 : 0;
-    return launch<LifBwdAlphaTensorsOp, 16>(op, n, t, stream);
+    return launch<LifBwdAlphaTensorsOp, EXODUS_TT_3>(op, n, t, stream);
 }
 
 EXODUS_API int exodus_leaky_forward(float *out, const float *input, const float *vmem_initial,
@@ -876,7 +885,7 @@ EXODUS_API int exodus_leaky_forward(float *out, const float *input, const float 
     op.out[0] = out;
     op.v_init = vmem_initial;
     op.alpha = alpha;
-    return launch<LeakyFwdOp, 32>(op, n, t, stream);
+    return launch<LeakyFwdOp, EXODUS_TT_1>(op, n, t, stream);
 }
 
 EXODUS_API int exodus_leaky_backward_fused(float *input_grad, float *alpha_grad, float *init_grad,
@@ -894,17 +903,17 @@ EXODUS_API int exodus_leaky_backward_fused(float *input_grad, float *alpha_grad,
             LeakyBwdOp<true, true> op;
             op.in[0] = output_grad; op.in[1] = output; op.out[0] = input_grad;
             op.v_init = vmem_initial; op.alpha = alpha; op.alpha_grad = alpha_grad; op.init_grad = init_grad;
-            return launch<LeakyBwdOp<true, true>, 32>(op, n, t, stream);
+            return launch<LeakyBwdOp<true, true>, EXODUS_TT_1>(op, n, t, stream);
         }
         LeakyBwdOp<true, false> op;
         op.in[0] = output_grad; op.in[1] = output; op.out[0] = nullptr;
         op.v_init = vmem_initial; op.alpha = alpha; op.alpha_grad = alpha_grad; op.init_grad = init_grad;
-        return launch<LeakyBwdOp<true, false>, 32>(op, n, t, stream);
+        return launch<LeakyBwdOp<true, false>, EXODUS_TT_1>(op, n, t, stream);
     }
     LeakyBwdOp<false, true> op;
     op.in[0] = output_grad; op.out[0] = input_grad;
     op.v_init = vmem_initial; op.alpha = alpha; op.alpha_grad = nullptr; op.init_grad = init_grad;
-    return launch<LeakyBwdOp<false, true>, 32>(op, n, t, stream);
+    return launch<LeakyBwdOp<false, true>, EXODUS_TT_1>(op, n, t, stream);
 }
 
 EXODUS_API int exodus_leaky_backward(float *input_grad, const float *output_grad, const float *alpha,
@@ -980,7 +989,7 @@ EXODUS_API int exodus_synlif_forward(float *out_spikes, float *out_vmem, float *
     op.decay_early = decay_early ? 1 : 0;
     op.norm_input = norm_input ? 1 : 0;
     op.cap = static_cast<unsigned>(max_num_spikes);
-    return launch<SynLifFwdOp, 32>(op, n, t, stream);
+    return launch<SynLifFwdOp, EXODUS_TT_1>(op, n, t, stream);
 }
 
 EXODUS_API int exodus_synlif_backward(float *grad_input, float *alpha_mem_grad, float *alpha_syn_grad,
