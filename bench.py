@@ -43,7 +43,11 @@ WORKLOADS = {
 
 # HBM traffic per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by the
 # reading of a plain copy of known size); bytes per launch of the dominant kernel, or None.
-MEASURED_TRAFFIC = {}
+MEASURED_TRAFFIC = {
+    # profiles/synlif_c5_pmc.md: FETCH_SIZE x2 + WRITE_SIZE x1 (KiB), factors from the 1 GiB probe kernel
+    ("c5", "exodus_synlif_backward"): 33.79e9,
+    ("c5", "exodus_synlif_forward"): 33.64e9,
+}
 
 
 def build_workload(key, torch, hip, act, dev):
@@ -168,7 +172,7 @@ def main():
     ap.add_argument("--workload", default="c5", choices=list(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-probe", action="store_true",
-                    help="also launch one plain device copy of exactly 1 GiB before the timed region, so that a "
+                    help="also launch one plain elementwise kernel (torch.neg) over exactly 1 GiB before the timed region, so that a "
                          "counter run (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE) has a kernel of known traffic "
                          "to scale its readings by")
     args = ap.parse_args()
@@ -189,7 +193,7 @@ def main():
     if args.copy_probe:
         src = torch.ones(1 << 28, device=dev)          # 2^28 floats = 1 GiB read + 1 GiB written
         dst = torch.empty_like(src)
-        dst.copy_(src)
+        torch.neg(src, out=dst)                        # a plain elementwise kernel: 1 GiB in, 1 GiB out
         torch.cuda.synchronize()
         del src, dst
 
