@@ -21,7 +21,8 @@ kernels; finite differences).
 ``clip_mode`` selects how the lower bound is applied: ``"relu"`` is
 ``relu(v - lo) + lo`` (upstream's formulation as recalled), ``"max"`` is ``max(v, lo)``
 (what the reference device code does, cuda/lif_kernels.h:75-77).  They agree exactly on
-clipped steps and differ by at most one rounding of ``(v - lo) + lo`` on the others.
+clipped steps and differ by at most one rounding of ``(v - lo) + lo`` on the others.  In both
+modes the derivative is 0 where ``v <= lo`` (the convention of Gradient_analysis.ipynb cell 7).
 """
 from __future__ import annotations
 
@@ -73,7 +74,10 @@ def lif_step(x_t, state: Dict[str, torch.Tensor], alpha_mem, alpha_syn, spike_th
         if clip_mode == "relu":
             v = torch.nn.functional.relu(v - min_v_mem) + min_v_mem
         elif clip_mode == "max":
-            v = torch.maximum(v, torch.as_tensor(min_v_mem, dtype=v.dtype).expand_as(v))
+            # value max(v, lo); derivative 0 where v <= lo (as relu gives it, and unlike
+            # torch.maximum, which splits the gradient at v == lo)
+            lo_t = torch.as_tensor(min_v_mem, dtype=v.dtype, device=v.device).expand_as(v)
+            v = torch.where(v > lo_t, v, lo_t)
         else:
             raise ValueError(clip_mode)
     new_state = {"v_mem": v}

@@ -69,7 +69,8 @@ class StatefulLayer(nn.Module):
 
     def __repr__(self):
         shown = ("tau_mem", "tau_syn", "spike_threshold", "min_v_mem", "norm_input")
-        parts = [f"{k}={v}" for k, v in self._param_dict.items() if k in shown and v is not None]
+        plain = lambda v: v.item() if isinstance(v, torch.Tensor) and v.numel() == 1 else v
+        parts = [f"{k}={plain(v)}" for k, v in self._param_dict.items() if k in shown and v is not None]
         return f"{self.__class__.__name__}({', '.join(parts)})"
 
     def __deepcopy__(self, memo=None):
@@ -112,11 +113,13 @@ class LIF(StatefulLayer):
         else:
             self.tau_mem = nn.Parameter(as_f32(tau_mem))
             self.tau_syn = nn.Parameter(as_f32(tau_syn)) if has_syn else None
-        self.spike_threshold = spike_threshold
+        # fixed (non-trainable) parameters, so that they follow the module across devices
+        self.spike_threshold = (nn.Parameter(as_f32(spike_threshold), requires_grad=False)
+                                if spike_threshold is not None else None)
         self.spike_fn = spike_fn
         self.reset_fn = reset_fn
         self.surrogate_grad_fn = surrogate_grad_fn
-        self.min_v_mem = min_v_mem
+        self.min_v_mem = nn.Parameter(as_f32(min_v_mem), requires_grad=False) if min_v_mem is not None else None
         self.train_alphas = train_alphas
         self.norm_input = norm_input
         self.record_states = record_states

@@ -11,11 +11,12 @@ from ..spike import IntegrateAndFire
 __all__ = ["LIF", "LIFSqueeze"]
 
 
-def expand_to_1d_contiguous(value: Union[float, torch.Tensor], shape: Tuple[int]) -> torch.Tensor:
+def expand_to_1d_contiguous(value: Union[float, torch.Tensor], shape: Tuple[int], device=None) -> torch.Tensor:
     """Broadcast ``value`` to ``shape`` (so per-channel tensors line up with the batch dimension),
     then flatten to a contiguous float32 vector with one entry per row of the (N, T) matrices
-    (reference sinabs/exodus/layers/lif.py:20-44)."""
-    return torch.as_tensor(value).expand(shape).float().flatten().contiguous()
+    (reference sinabs/exodus/layers/lif.py:20-44).  ``device`` moves plain numbers and stray CPU
+    tensors next to the states."""
+    return torch.as_tensor(value, device=device).expand(shape).float().flatten().contiguous()
 
 
 class LIF(LIFBase):
@@ -116,7 +117,7 @@ class LIF(LIFBase):
     def _forward_synaptic(self, input_2d: torch.Tensor) -> torch.Tensor:
         """Exponential synapse i_t = alpha_syn * i_{t-1} + x_t (x pre-scaled by alpha_syn when
         ``decay_early``) -- reference lif.py:185-198."""
-        alpha_syn = expand_to_1d_contiguous(self.alpha_syn_calculated, self.v_mem.shape)
+        alpha_syn = expand_to_1d_contiguous(self.alpha_syn_calculated, self.v_mem.shape, self.v_mem.device)
         if self.decay_early:
             input_2d = input_2d * alpha_syn.unsqueeze(1)
         return LeakyIntegrator.apply(input_2d.contiguous(), alpha_syn, self.i_syn.flatten().contiguous())
@@ -124,7 +125,8 @@ class LIF(LIFBase):
     def _forward_membrane(self, i_syn_2d: torch.Tensor):
         """Membrane stage: returns (output, post-reset v_mem), both (N, T) -- reference lif.py:200-258."""
         state_shape = self.v_mem.shape
-        alpha_mem = expand_to_1d_contiguous(self.alpha_mem_calculated, state_shape)
+        dev = self.v_mem.device
+        alpha_mem = expand_to_1d_contiguous(self.alpha_mem_calculated, state_shape, dev)
 
         if self.norm_input:
             i_syn_2d = (1.0 - alpha_mem.unsqueeze(1)) * i_syn_2d
@@ -136,13 +138,13 @@ class LIF(LIFBase):
             v_mem = LeakyIntegrator.apply(i_syn_2d.contiguous(), alpha_mem, self.v_mem.flatten().contiguous())
             return v_mem, v_mem
 
-        spike_threshold = expand_to_1d_contiguous(self.spike_threshold, state_shape)
-        min_v_mem = None if self.min_v_mem is None else expand_to_1d_contiguous(self.min_v_mem, state_shape)
+        spike_threshold = expand_to_1d_contiguous(self.spike_threshold, state_shape, dev)
+        min_v_mem = None if self.min_v_mem is None else expand_to_1d_contiguous(self.min_v_mem, state_shape, dev)
         membrane_subtract = self.reset_fn.subtract_value
         if membrane_subtract is None:
             membrane_subtract = spike_threshold
         else:
-            membrane_subtract = expand_to_1d_contiguous(membrane_subtract, state_shape)
+            membrane_subtract = expand_to_1d_contiguous(membrane_subtract, state_shape, dev)
 
         output_2d, v_mem_2d = IntegrateAndFire.apply(
             i_syn_2d.contiguous(),

@@ -1,0 +1,166 @@
+"""CPU-only checks: the C-ABI library loads and exports everything the header declares, and the
+host-side mirror of the reference API (layers, conversion, argument handling) behaves.  No kernel
+is launched here."""
+import ctypes
+import os
+import re
+import subprocess
+
+import pytest
+import torch
+import torch.nn as nn
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "exodus_hip.h")
+LIB = os.path.join(ROOT, "sinabs-exodus_amd", "sinabs", "exodus", "libexodus_hip.so")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(exodus_[a-z_]+)\s*\(", text)))
+
+
+def test_header_declares_the_expected_entry_points():
+    names = declared_functions()
+    for must in ("exodus_lif_forward", "exodus_lif_backward", "exodus_lif_backward_alpha", "exodus_leaky_forward",
+                 "exodus_leaky_backward", "exodus_leaky_backward_alpha", "exodus_leaky_backward_fused",
+                 "exodus_lif_backward_fused", "exodus_synlif_forward", "exodus_synlif_backward",
+                 "exodus_hip_abi_version", "exodus_hip_error_string"):
+        assert must in names
+
+
+def test_library_exports_every_declared_symbol():
+    assert os.path.exists(LIB), "build the library first: python sinabs-exodus_amd/build_hip.py"
+    import torch  # noqa: F401  (loads the HIP runtime the library links against)
+    lib = ctypes.CDLL(LIB)
+    for name in declared_functions():
+        assert hasattr(lib, name), f"{name} declared in exodus_hip.h but not exported"
+    exported = subprocess.run(["nm", "-D", "--defined-only", LIB], capture_output=True, text=True).stdout
+    extra = [l.split()[-1] for l in exported.splitlines() if " T " in l and not l.split()[-1].startswith("exodus_")]
+    assert not extra, f"unexpected exported symbols: {extra}"
+    lib.exodus_hip_abi_version.restype = ctypes.c_int
+    assert lib.exodus_hip_abi_version() == 1
+
+
+def test_loader_signatures_cover_the_header():
+    from sinabs.exodus import _hip
+    assert sorted(_hip._SIGNATURES) == declared_functions()
+
+
+def test_functions_reject_cpu_tensors_and_bad_arguments():
+    from sinabs.exodus.leaky import LeakyIntegrator
+    from sinabs.exodus.spike import IntegrateAndFire, classify_surrogate
+    from sinabs.exodus._compat import activation as act
+    from sinabs.exodus import _hip
+
+    x = torch.rand(2, 10); r = torch.full((2,), 0.5)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        LeakyIntegrator.apply(x, r, r)
+    with pytest.raises(ValueError, match="2D"):
+        LeakyIntegrator.apply(x[0], r, r)
+    with pytest.raises(ValueError, match="contiguous"):
+        LeakyIntegrator.apply(torch.rand(10, 2).t(), r, r)
+    with pytest.raises(ValueError, match="1D"):
+        LeakyIntegrator.apply(x, r.unsqueeze(0), r)
+    with pytest.raises(ValueError, match="between 0 and 1"):
+        IntegrateAndFire.apply(x, torch.tensor([0.5, 1.5]), r, r, r, None, act.Heaviside())
+    with pytest.raises(ValueError, match="greater than `min_v_mem`"):
+        IntegrateAndFire.apply(x, r, r, torch.ones(2), None, torch.tensor([1.2, 0.0]), act.Heaviside())
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        IntegrateAndFire.apply(x, r, r, torch.ones(2), None, None, act.Heaviside())
+
+    assert classify_surrogate(act.SingleExponential(0.3, 2.0)) == (_hip.SURR_SINGLE_EXP, 0.3, 2.0)
+    assert classify_surrogate(act.PeriodicExponential())[0] == _hip.SURR_PERIODIC_EXP
+    assert classify_surrogate(act.Heaviside(0.7)) == (_hip.SURR_HEAVISIDE, 0.7, 0.0)
+    assert classify_surrogate(lambda v, th: v)[0] == _hip.SURR_TENSOR
+
+    class SingleExponential:           # same name, foreign module: must not be mistaken for the known one
+        grad_width, grad_scale = 0.5, 1.0
+
+    assert classify_surrogate(SingleExponential())[0] == _hip.SURR_TENSOR
+
+
+def test_layer_construction_and_bookkeeping():
+    import sinabs.exodus.layers as el
+    from sinabs.exodus._compat import activation as act
+    from sinabs.exodus.layers.lif import expand_to_1d_contiguous
+
+    lif = el.LIF(tau_mem=20.0, tau_syn=5.0, min_v_mem=-1.0, train_alphas=True, spike_fn=act.MaxSpike(2))
+    assert lif.does_spike and lif.max_num_spikes_per_bin == 2 and lif.decay_early
+    assert "EXODUS" in repr(lif)
+    assert set(lif.state_dict()) == {"alpha_mem", "alpha_syn", "spike_threshold", "min_v_mem", "v_mem", "i_syn"}
+    assert torch.allclose(lif.alpha_mem_calculated, torch.exp(torch.tensor(-1 / 20.0)))
+    assert el.LIF(tau_mem=20.0, spike_fn=act.SingleSpike).max_num_spikes_per_bin == 1
+    assert el.LIF(tau_mem=20.0).max_num_spikes_per_bin is None
+    assert set(el.LIF(tau_mem=20.0).state_dict()) == {"tau_mem", "spike_threshold", "v_mem"}
+
+    iaf = el.IAF(min_v_mem=-2)
+    assert iaf.tau_mem is None and float(iaf.alpha_mem_calculated) == 1.0 and not iaf.norm_input
+    assert "tau_mem" not in iaf.arg_dict and "norm_input" not in iaf.arg_dict
+    leak = el.ExpLeak(tau_mem=10.0)
+    assert not leak.does_spike and not leak.decay_early and "spike_fn" not in leak.arg_dict
+    sq = el.IAFSqueeze(batch_size=12, min_v_mem=-1)
+    assert sq.arg_dict["batch_size"] == 12 and sq.arg_dict["num_timesteps"] == -1
+    with pytest.raises(TypeError):
+        el.LIFSqueeze(tau_mem=10.0)
+
+    with pytest.raises(NotImplementedError):
+        el.LIF(tau_mem=20.0, reset_fn=act.MembraneReset())
+    with pytest.raises(NotImplementedError):
+        el.IAF(spike_fn=torch.relu)
+
+    lif.reset_states()                                   # uninitialised: a no-op
+    lif.init_state_with_shape((3, 4))
+    assert lif.is_state_initialised() and lif.state_has_shape((3, 4)) and not lif.state_has_shape((4, 3))
+    lif.v_mem += 1.0
+    lif.reset_states()
+    assert (lif.v_mem == 0).all()
+
+    e = expand_to_1d_contiguous(torch.tensor([1.0, 2.0, 3.0]), (2, 3))
+    assert e.tolist() == [1, 2, 3, 1, 2, 3] and e.is_contiguous()
+    assert expand_to_1d_contiguous(0.5, (2, 2)).tolist() == [0.5] * 4
+
+
+def _model(layers_mod, batch_size=12):
+    return nn.Sequential(
+        nn.Conv2d(2, 8, 5, 1),
+        layers_mod.IAFSqueeze(batch_size=batch_size, min_v_mem=-1),
+        nn.AvgPool2d(2, 2),
+        nn.Conv2d(8, 16, 3, 1),
+        layers_mod.IAFSqueeze(batch_size=batch_size, min_v_mem=-2),
+        nn.AvgPool2d(2, 2),
+        nn.Flatten(),
+        nn.Linear(64, 10),
+    )
+
+
+def test_conversion_both_ways():
+    """reference tests/test_conversion.py, with the oracle's plain layers in the role of sinabs.layers"""
+    import sinabs.exodus.layers as el
+    from sinabs.exodus import conversion
+    from oracle import sinabs_layers as sl
+
+    plain = _model(sl)
+    fast = conversion.sinabs_to_exodus(plain, sinabs_layers=sl)
+    assert type(plain[1]) is sl.IAFSqueeze and type(fast[1]) is el.IAFSqueeze and len(plain) == len(fast)
+    assert fast[1].min_v_mem == plain[1].min_v_mem and fast[4].min_v_mem == plain[4].min_v_mem
+    assert fast[1].batch_size == plain[1].batch_size
+    assert torch.equal(fast[0].weight, plain[0].weight) and fast[0] is not plain[0]
+
+    fast2 = _model(el)
+    plain2 = conversion.exodus_to_sinabs(fast2, sinabs_layers=sl)
+    assert type(plain2[1]) is sl.IAFSqueeze and type(fast2[1]) is el.IAFSqueeze and len(plain2) == len(fast2)
+    assert plain2[4].min_v_mem == fast2[4].min_v_mem and plain2[1].batch_size == fast2[1].batch_size
+
+    assert set(conversion.get_module_map(sl).values()) == {el.IAF, el.IAFSqueeze, el.LIF, el.LIFSqueeze, el.ExpLeak,
+                                                           el.ExpLeakSqueeze}
+    from sinabs.exodus._compat import HAVE_UPSTREAM_SINABS
+    if not HAVE_UPSTREAM_SINABS:
+        with pytest.raises(ImportError, match="sinabs"):
+            conversion.sinabs_to_exodus(plain)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    out = subprocess.run(["python", os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert out.returncode != 0 and "one GPU" in (out.stderr + out.stdout)
