@@ -7,6 +7,7 @@ from .._compat import (LIFBase, MaxSpike, MembraneSubtract, MultiSpike, SingleEx
                        SqueezeMixin)
 from ..leaky import LeakyIntegrator
 from ..spike import IntegrateAndFire
+from ..synaptic import SynapticIntegrateAndFire, fusable
 
 __all__ = ["LIF", "LIFSqueeze"]
 
@@ -80,6 +81,9 @@ class LIF(LIFBase):
             record_states=record_states,
         )
         self.decay_early = decay_early
+        # layers with synapses run synapse and membrane in one kernel when the surrogate gradient
+        # is one the kernels can evaluate; set to False to force the two separate Functions
+        self.fuse_synapse = True
 
     def _parse_activation_fn(self, spike_fn, reset_fn):
         """Translate the spike mechanism into a per-step spike cap (reference lif.py:130-150)."""
@@ -160,21 +164,55 @@ class LIF(LIFBase):
         v_mem_2d = v_mem_2d - membrane_subtract.unsqueeze(1) * output_2d
         return output_2d, v_mem_2d
 
+    def _forward_synaptic_membrane(self, input_2d: torch.Tensor):
+        """Same values as ``_forward_synaptic`` followed by ``_forward_membrane`` (same operations
+        in the same order), computed by the fused kernels: returns (output, post-reset v_mem, i_syn)."""
+        state_shape, dev = self.v_mem.shape, self.v_mem.device
+        alpha_syn = expand_to_1d_contiguous(self.alpha_syn_calculated, state_shape, dev)
+        alpha_mem = expand_to_1d_contiguous(self.alpha_mem_calculated, state_shape, dev)
+        spike_threshold = expand_to_1d_contiguous(self.spike_threshold, state_shape, dev)
+        min_v_mem = None if self.min_v_mem is None else expand_to_1d_contiguous(self.min_v_mem, state_shape, dev)
+        membrane_subtract = self.reset_fn.subtract_value
+        if membrane_subtract is None:
+            membrane_subtract = spike_threshold
+        else:
+            membrane_subtract = expand_to_1d_contiguous(membrane_subtract, state_shape, dev)
+        output_2d, v_mem_2d, i_syn_2d = SynapticIntegrateAndFire.apply(
+            input_2d.contiguous(),
+            alpha_syn,
+            alpha_mem,
+            self.i_syn.flatten().contiguous(),
+            self.v_mem.flatten().contiguous(),
+            spike_threshold,
+            membrane_subtract,
+            min_v_mem,
+            self.surrogate_grad_fn,
+            self.max_num_spikes_per_bin,
+            self.decay_early,
+            self.norm_input,
+        )
+        v_mem_2d = v_mem_2d - membrane_subtract.unsqueeze(1) * output_2d
+        return output_2d, v_mem_2d, i_syn_2d
+
     def forward(self, input_data: torch.Tensor) -> torch.Tensor:
         """Process ``input_data`` of shape (batch, time, ...); returns a tensor of the same shape."""
         input_2d, (batch_size, time_steps, *trailing_dim) = self._prepare_input(input_data)
         self.recordings = dict()
 
         if self.tau_syn_calculated is None:
-            i_syn_2d = input_2d
+            output_2d, v_mem_2d = self._forward_membrane(input_2d)
         else:
-            i_syn_2d = self._forward_synaptic(input_2d)
+            if self.spike_fn is not None and self.fuse_synapse and fusable(self.surrogate_grad_fn):
+                # synapse and membrane in one kernel per direction
+                output_2d, v_mem_2d, i_syn_2d = self._forward_synaptic_membrane(input_2d)
+            else:
+                i_syn_2d = self._forward_synaptic(input_2d)
+                output_2d, v_mem_2d = self._forward_membrane(i_syn_2d)
             i_syn_full = self._rows_to_full(i_syn_2d, batch_size, trailing_dim)
             self.i_syn = i_syn_full[:, -1].clone()
             if self.record_states:
                 self.recordings["i_syn"] = i_syn_full
 
-        output_2d, v_mem_2d = self._forward_membrane(i_syn_2d)
         v_mem_full = self._rows_to_full(v_mem_2d, batch_size, trailing_dim)
         output_full = self._rows_to_full(output_2d, batch_size, trailing_dim)
 

@@ -91,6 +91,29 @@ def test_layer_equal_output(L, spike):
     assert torch.equal(plain.v_mem, fast.v_mem)
 
 
+@pytest.mark.parametrize("decay_early,norm_input,train_alphas", list(product((True, False), (True, False), (True, False))))
+def test_fused_synaptic_layer_equals_composed_layer(L, decay_early, norm_input, train_alphas):
+    """The layer's one-kernel synapse+membrane path and its two-Function path give identical outputs
+    and states, and gradients within fp32 tolerance, over two chained calls."""
+    el, _, act = L
+    kw = dict(tau_mem=torch.full((12,), 15.0), tau_syn=torch.full((12,), 6.0), min_v_mem=-0.8, norm_input=norm_input,
+              train_alphas=train_alphas, decay_early=decay_early, spike_fn=act.MaxSpike(2), record_states=True)
+    fused = el.LIF(**kw).cuda(); composed = el.LIF(**kw).cuda(); composed.fuse_synapse = False
+    data = torch.rand((2, 5, 60, 12), generator=gen(21)).cuda() * (6.0 if norm_input else 0.6)
+    xa = data.clone().requires_grad_(True); xb = data.clone().requires_grad_(True)
+    for k in range(2):
+        a = fused(xa[k]); b = composed(xb[k])
+        assert torch.equal(a, b) and torch.equal(fused.v_mem, composed.v_mem) and torch.equal(fused.i_syn, composed.i_syn)
+    assert a.sum() > 0
+    w = torch.rand(a.shape, generator=gen(22)).cuda()
+    ((a * w).sum() + fused.recordings["v_mem"].sum() * 0.1).backward()
+    ((b * w).sum() + composed.recordings["v_mem"].sum() * 0.1).backward()
+    assert_close(xa.grad, xb.grad, "grad input")
+    for (k, p), (_, q) in zip(fused.named_parameters(), composed.named_parameters()):
+        if q.grad is not None:
+            assert_close(p.grad, q.grad, f"grad {k}", rtol=1e-4, atol=1e-5)
+
+
 def test_record_states(L):
     el, sl, _ = L
     x = torch.rand((3, 40, 6), generator=gen(5)) * 3
