@@ -50,6 +50,52 @@ MEASURED_TRAFFIC = {
 }
 
 
+def build_layer_workload(key, torch, hip, act, dev):
+    """The same workloads on the layer's own (batch, time, neurons) layout: one kernel per direction,
+    forward keeps checkpoints only, backward re-reads the input and rebuilds v_mem / i_syn.
+    Algorithmic bytes per neuron-timestep: forward 8 (x in, spikes out), backward 12 (grad_spikes
+    and x in, grad_x out)."""
+    w = WORKLOADS[key]
+    B, T, M = w["batch"], w["steps"], w["neurons"]
+    N = B * M
+    g = torch.Generator(device=dev).manual_seed(list(WORKLOADS).index(key))
+    if key == "c1":
+        x = torch.rand(B, T, M, generator=g, device=dev) * 0.5
+    else:
+        x = torch.randn(B, T, M, generator=g, device=dev) * w["std"] + w["mean"]
+    go = torch.ones(B, T, M, device=dev)
+    rows = lambda v: torch.as_tensor(v, dtype=torch.float32, device=dev).expand(B, M).flatten().contiguous()
+    zeros = torch.zeros(N, device=dev); ones = torch.ones(N, device=dev)
+    surr = act.SingleExponential()
+    kind, p0, p1 = hip.SURR_SINGLE_EXP, surr.grad_width, surr.grad_scale
+    spikes = torch.empty_like(x); gi = torch.empty_like(x)
+    if key == "c5":
+        cfg = dict(a_mem=rows(math.exp(-1 / 20.0)), a_syn=rows(math.exp(-1 / 5.0)), lo=rows(-1.0), cap=2, norm=True)
+    elif key == "c2":
+        cfg = dict(a_mem=rows(math.exp(-1 / 20.0)), a_syn=None, lo=None, cap=1, norm=True)
+    elif key == "c1":
+        cfg = dict(a_mem=ones, a_syn=None, lo=None, cap=-1, norm=False)
+    else:
+        raise SystemExit("the layer-layout path covers the spiking workloads (c5, c2, c1)")
+    syn = cfg["a_syn"] is not None
+    holder = {}
+
+    def fwd():
+        holder["r"] = hip.layerLifForward(x, zeros, zeros if syn else None, cfg["a_mem"], cfg["a_syn"], ones, ones,
+                                          cfg["lo"], cfg["lo"] is not None, cfg["cap"], True, cfg["norm"],
+                                          outSpikes=spikes)
+
+    def bwd():
+        r = holder["r"]
+        out = hip.layerLifBackward(go, None, None, x, r["ckpt_v"], r["ckpt_i"], zeros, zeros if syn else None,
+                                   cfg["a_mem"], cfg["a_syn"], ones, ones, cfg["lo"], cfg["lo"] is not None,
+                                   cfg["cap"], True, cfg["norm"], kind, p0, p1, gradInput=gi)
+        return out[1].view(B, M).sum(0)
+
+    return dict(fwd=fwd, bwd=bwd, N=N, T=T, fwd_name="exodus_layer_lif_forward",
+                bwd_name="exodus_layer_lif_backward", bytes=(8, 12))
+
+
 def build_workload(key, torch, hip, act, dev):
     w = WORKLOADS[key]
     B, T, M = w["batch"], w["steps"], w["neurons"]
@@ -170,6 +216,9 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c5", choices=list(WORKLOADS))
+    ap.add_argument("--path", default="layer", choices=["layer", "rows"],
+                    help="layer: kernels on the layer's (batch, time, neurons) layout (what the layers run); "
+                         "rows: the (rows, time) kernels behind the autograd Functions")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also launch one plain elementwise kernel (torch.neg) over exactly 1 GiB before the timed region, so that a "
@@ -187,7 +236,11 @@ def main():
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    wl = build_workload(args.workload, torch, hip, act, dev)
+    if args.path == "layer" and args.workload != "c3":
+        wl = build_layer_workload(args.workload, torch, hip, act, dev)
+    else:
+        args.path = "rows"
+        wl = build_workload(args.workload, torch, hip, act, dev)
     fwd, bwd, N, T = wl["fwd"], wl["bwd"], wl["N"], wl["T"]
 
     if args.copy_probe:
@@ -216,7 +269,7 @@ def main():
     ms_step = wall * 1e3 / args.steps
     fwd_ms = sum(e[0].elapsed_time(e[1]) for e in ev) / args.steps
     bwd_ms = sum(e[1].elapsed_time(e[2]) for e in ev) / args.steps
-    bf, bb = WORKLOADS[args.workload]["bytes"]
+    bf, bb = wl.get("bytes", WORKLOADS[args.workload]["bytes"])
     dom = "bwd" if bwd_ms >= fwd_ms else "fwd"
     dom_ms, dom_bytes, dom_name = (bwd_ms, bb, wl["bwd_name"]) if dom == "bwd" else (fwd_ms, bf, wl["fwd_name"])
     achieved = N * T * dom_bytes / (dom_ms * 1e-3) / 1e9
@@ -235,7 +288,7 @@ def main():
         "vs_baseline": None,
         "dtype": "f32",
         "data": "synthetic",
-        "config": {"workload": WORKLOADS[args.workload]["name"], "rows": N, "time_steps": T,
+        "config": {"workload": WORKLOADS[args.workload]["name"], "path": args.path, "rows": N, "time_steps": T,
                    "algorithmic_bytes_per_neuron_timestep": bf + bb},
         "roofline": {
             "bound": "hbm", "kernel": dom_name, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",

@@ -158,6 +158,49 @@ int exodus_synlif_backward(float *grad_input, float *alpha_mem_grad, float *alph
                            int max_num_spikes, int decay_early, int norm_input, int surrogate_kind,
                            float surr_p0, float surr_p1, int64_t n, int64_t t, void *stream);
 
+/* ---------------------------------------------------------------------------------------------
+ * The spiking layer on its own memory layout.  The reference layer transposes its
+ * (batch, time, *neurons) input into (rows, time), runs the Functions and views the results back
+ * (reference sinabs/exodus/layers/lif.py:152-183, 260-307).  These entry points work on the
+ * (batch, t, neurons) tensors directly (neurons = product of the trailing dimensions, contiguous)
+ * and write only what the layer hands out.  Per-neuron vectors have batch*neurons entries, in
+ * the order of the layer's state tensors.
+ * ------------------------------------------------------------------------------------------- */
+
+/* Steps between two checkpoints; ckpt tensors hold ceil(t / interval) entries per neuron. */
+int exodus_layer_checkpoint_interval(void);
+
+/* Forward of a LIF/IAF layer with (alpha_syn != NULL) or without synaptic current; arithmetic and
+ * order as exodus_synlif_forward / exodus_lif_forward after the layer's input scalings.
+ *   out_spikes (batch,t,neurons); v_last, i_last (batch*neurons): potential after the last reset
+ *   and last synaptic current (i_last may be NULL without synapse).
+ * Optional (NULL = skip): out_vmem_rec / out_isyn_rec (batch,t,neurons) post-reset potential and
+ * synaptic current of every step; ckpt_v / ckpt_i (batch, ceil(t/interval), neurons) state at the
+ * start of every checkpoint interval, needed by exodus_layer_lif_backward; spike_sum, one double
+ * to which the total spike count is added atomically. */
+int exodus_layer_lif_forward(float *out_spikes, float *out_vmem_rec, float *out_isyn_rec, float *ckpt_v,
+                             float *ckpt_i, float *v_last, float *i_last, double *spike_sum,
+                             const float *input, const float *vmem_post_initial,
+                             const float *isyn_initial, const float *alpha_mem, const float *alpha_syn,
+                             const float *membr_subtract, const float *theta, const float *theta_low,
+                             int apply_theta_low, int max_num_spikes, int decay_early, int norm_input,
+                             int64_t batch, int64_t t, int64_t neurons, void *stream);
+
+/* Backward of the above.  Re-reads `input`, rebuilds membrane potential and synaptic current of
+ * each checkpoint interval from ckpt_v / ckpt_i and walks it in reverse.  grad_v_last /
+ * grad_i_last (batch*neurons, optional) are gradients arriving at the final states.  Outputs:
+ * grad_input (batch,t,neurons) and the optional per-neuron alpha_mem_grad, alpha_syn_grad,
+ * vmem_init_grad, isyn_init_grad.  surrogate_kind must be an in-kernel kind (1..3). */
+int exodus_layer_lif_backward(float *grad_input, float *alpha_mem_grad, float *alpha_syn_grad,
+                              float *vmem_init_grad, float *isyn_init_grad, const float *grad_spikes,
+                              const float *grad_v_last, const float *grad_i_last, const float *input,
+                              const float *ckpt_v, const float *ckpt_i, const float *vmem_post_initial,
+                              const float *isyn_initial, const float *alpha_mem, const float *alpha_syn,
+                              const float *membr_subtract, const float *theta, const float *theta_low,
+                              int apply_theta_low, int max_num_spikes, int decay_early, int norm_input,
+                              int surrogate_kind, float surr_p0, float surr_p1, int64_t batch, int64_t t,
+                              int64_t neurons, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -9,7 +9,8 @@ import subprocess
 import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-SRC = os.path.join(HERE, "csrc", "exodus_hip.hip")
+SRCS = [os.path.join(HERE, "csrc", f) for f in ("exodus_hip.hip", "exodus_layer.hip")]
+SRC = SRCS[0]
 INCLUDE = os.path.join(os.path.dirname(HERE), "include")
 OUT = os.path.join(HERE, "sinabs", "exodus", "libexodus_hip.so")
 
@@ -23,11 +24,11 @@ FLAGS = [
 
 
 def build(force: bool = True) -> str:
-    if not force and os.path.exists(OUT) and os.path.getmtime(OUT) >= max(
-            os.path.getmtime(SRC), os.path.getmtime(os.path.join(INCLUDE, "exodus_hip.h"))):
+    deps = SRCS + [os.path.join(HERE, "csrc", "exodus_common.hpp"), os.path.join(INCLUDE, "exodus_hip.h")]
+    if not force and os.path.exists(OUT) and os.path.getmtime(OUT) >= max(os.path.getmtime(d) for d in deps):
         return OUT
     hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
-    cmd = [hipcc] + FLAGS + ["-I", INCLUDE, "-o", OUT + ".tmp", SRC]
+    cmd = [hipcc] + FLAGS + ["-I", INCLUDE, "-o", OUT + ".tmp"] + SRCS
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     # hipcc's host pass does not know the gfx-only target feature and says so; that line is harmless
     noise = "packed-fp32-ops"

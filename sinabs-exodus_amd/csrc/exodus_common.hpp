@@ -1,0 +1,139 @@
+// Device-side helpers shared by the row-major (rows, time) kernels and the layer-layout
+// (batch, time, neurons) kernels of libexodus_hip.so.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "exodus_hip.h"
+
+namespace {
+
+constexpr int WAVE = 64;
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));    // one 16-byte chunk = 4 time steps
+
+// Tile lengths (time steps per tile) by number of (n,t) tensors an op keeps in LDS.  Longer tiles
+// mean longer contiguous segments per row; more slots mean more LDS per wave.
+#ifndef EXODUS_TT_1
+#define EXODUS_TT_1 32    // one or two LDS slots
+#endif
+#ifndef EXODUS_TT_3
+#define EXODUS_TT_3 32    // three or more LDS slots
+#endif
+
+// Unroll factor of the per-tile chunk loop (each chunk = 4 time steps).  Full unrolling lets the
+// compiler hoist every LDS read of the tile, which costs registers and therefore resident waves.
+#ifndef EXODUS_UNROLL_Q
+#define EXODUS_UNROLL_Q 8
+#endif
+#define EXODUS_PRAGMA(x) _Pragma(#x)
+#define EXODUS_UNROLL(n) EXODUS_PRAGMA(unroll n)
+
+// streaming (non-temporal) hints on the (n,t) tensors, which are read once and written once
+#ifndef EXODUS_NT_LOAD
+#define EXODUS_NT_LOAD 1
+#endif
+#ifndef EXODUS_NT_STORE
+#define EXODUS_NT_STORE 1
+#endif
+template <class T> __device__ __forceinline__ T ld_stream(const T *p)
+{
+#if EXODUS_NT_LOAD
+    return __builtin_nontemporal_load(p);
+#else
+    return *p;
+#endif
+}
+template <class T> __device__ __forceinline__ void st_stream(T v, T *p)
+{
+#if EXODUS_NT_STORE
+    __builtin_nontemporal_store(v, p);
+#else
+    *p = v;
+#endif
+}
+
+__device__ __forceinline__ void wave_sync()
+{
+    // All lanes of a wave execute an instruction together and the LDS serves one wave's requests
+    // in issue order; what remains is to stop the compiler from moving LDS accesses across here.
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// ---------------------------------------------------------------------------------------------
+// per-row helpers
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ float spike_count(float v, float theta, unsigned cap)
+{
+    // count = v >= theta ? min(unsigned(v / theta), cap) : 0      (IEEE division, truncation)
+    //
+    // The quotient is only formed where it can exceed 2.  For theta > 0 and fp32 v, theta:
+    //   v >= theta            <=>  RN(v/theta) >= 1
+    //   v >= 2*theta (exact)  <=>  RN(v/theta) >= 2   (no fp32 number lies strictly between the
+    //                              predecessor of 2*theta and 2*theta, and the rounding boundary
+    //                              2*theta*(1 - 2^-25) falls inside that gap)
+    // so below 2*theta the count is 0 or 1 without dividing, and a cap of 1 or 2 never divides.
+    if (v < theta) return 0.f;
+    if (theta > 0.f) {
+        if (cap <= 1u) return static_cast<float>(cap);
+        if (v < __fadd_rn(theta, theta)) return 1.f;
+        if (cap == 2u) return 2.f;
+    }
+    const unsigned k = static_cast<unsigned>(__fdiv_rn(v, theta));
+    return static_cast<float>(k < cap ? k : cap);
+}
+
+// Per-row constants of the in-kernel surrogate gradients.  Surrogate values enter gradients only
+// (tolerance rtol 1e-4), never spike decisions, so divisions by per-row constants become
+// multiplications by their reciprocals and exp() is the hardware exponential (relative error
+// about |argument| * 6e-8).
+struct SurrConst { float a, b; };
+
+template <int KIND>
+__device__ __forceinline__ SurrConst surrogate_consts(float theta, float p0, float p1)
+{
+    SurrConst k;
+    if (KIND == EXODUS_SURR_SINGLE_EXP) {
+        const float w = __fmul_rn(theta, p0);                 // p1/(theta p0) * exp(-|v - theta| / (theta p0))
+        k.a = __fdiv_rn(1.f, w);
+        k.b = __fdiv_rn(p1, w);
+    } else if (KIND == EXODUS_SURR_PERIODIC_EXP) {
+        k.a = __fmul_rn(theta, 0.5f);                          // p1 * exp(-|u - theta/2| / p0) / theta
+        k.b = __fdiv_rn(p1, theta);
+    } else {
+        k.a = __fsub_rn(theta, p0);                            // (v >= theta - p0) / theta
+        k.b = __fdiv_rn(1.f, theta);
+    }
+    return k;
+}
+
+template <int KIND>
+__device__ __forceinline__ float surrogate(float v, float theta, float inv_p0, SurrConst k)
+{
+    if (KIND == EXODUS_SURR_SINGLE_EXP) {
+        return k.b * __expf(-fabsf(v - theta) * k.a);
+    } else if (KIND == EXODUS_SURR_PERIODIC_EXP) {
+        float u = v - k.a;
+        if (v >= theta) u = fmodf(u, theta);                 // u > 0 here, so fmod == floor-mod
+        return k.b * __expf(-fabsf(u - k.a) * inv_p0);
+    } else {
+        return v >= k.a ? k.b : 0.f;
+    }
+}
+
+// Sum of many products for the per-row parameter gradients: fp32 fused multiply-adds within a
+// tile (at most TT terms), folded into an fp64 total at every tile end.
+struct TileSum {
+    float part;
+    double total;
+    __device__ __forceinline__ void clear() { part = 0.f; total = 0.0; }
+    __device__ __forceinline__ void add(float a, float b) { part = __fmaf_rn(a, b, part); }
+    __device__ __forceinline__ void sub(float a, float b) { part = __fmaf_rn(-a, b, part); }
+    __device__ __forceinline__ void fold() { total += static_cast<double>(part); part = 0.f; }
+};
+
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+}  // namespace

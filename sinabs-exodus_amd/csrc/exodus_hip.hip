@@ -25,54 +25,9 @@
 #include <type_traits>
 
 #include "exodus_hip.h"
+#include "exodus_common.hpp"
 
 namespace {
-
-constexpr int WAVE = 64;
-
-typedef float f32x4 __attribute__((ext_vector_type(4)));    // one 16-byte chunk = 4 time steps
-
-// Tile lengths (time steps per tile) by number of (n,t) tensors an op keeps in LDS.  Longer tiles
-// mean longer contiguous segments per row; more slots mean more LDS per wave.
-#ifndef EXODUS_TT_1
-#define EXODUS_TT_1 32    // one or two LDS slots
-#endif
-#ifndef EXODUS_TT_3
-#define EXODUS_TT_3 32    // three or more LDS slots
-#endif
-
-// streaming (non-temporal) hints on the (n,t) tensors, which are read once and written once
-#ifndef EXODUS_NT_LOAD
-#define EXODUS_NT_LOAD 1
-#endif
-#ifndef EXODUS_NT_STORE
-#define EXODUS_NT_STORE 1
-#endif
-template <class T> __device__ __forceinline__ T ld_stream(const T *p)
-{
-#if EXODUS_NT_LOAD
-    return __builtin_nontemporal_load(p);
-#else
-    return *p;
-#endif
-}
-template <class T> __device__ __forceinline__ void st_stream(T v, T *p)
-{
-#if EXODUS_NT_STORE
-    __builtin_nontemporal_store(v, p);
-#else
-    *p = v;
-#endif
-}
-
-__device__ __forceinline__ void wave_sync()
-{
-    // All lanes of a wave execute an instruction together and the LDS serves one wave's requests
-    // in issue order; what remains is to stop the compiler from moving LDS accesses across here.
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-}
 
 template <int TT>
 struct Geom {
@@ -133,7 +88,8 @@ __device__ __forceinline__ void put(f32x4 &v, int e, float x) { v[e] = x; }
 //   NIN, NOUT          number of (n,t) inputs / outputs; output j reuses the LDS slot of input j
 //   REVERSE            walk time from the last step to the first
 //   in[NIN], out[NOUT] device pointers
-//   State, init(State&, row, valid), step(State&, const float* x, float* y), finish(State&, row)
+//   State, init(State&, row, valid), step(State&, const float* x, float* y), end_tile(State&)
+//   (called after each tile), finish(State&, row)
 //   NDER (0 or 1)      one more (n,t) output that is a pure function of output DER_SRC and of
 //                      NROWP per-row constants: it is computed while the tile is written back
 //                      (stash(State&, float* p) / derive(const float* p, f32x4 v)), so it needs no
@@ -198,7 +154,7 @@ __global__ void __launch_bounds__(WAVE) scan_kernel(const Op op, const int64_t n
     // that fall outside the row (first and last tile only).
     auto compute = [&](int64_t t_first, auto guard) {
         constexpr bool GUARD = decltype(guard)::value;
-#pragma unroll
+        EXODUS_UNROLL(EXODUS_UNROLL_Q)
         for (int qq = 0; qq < G::CPR; ++qq) {
             const int q = Op::REVERSE ? G::CPR - 1 - qq : qq;
             f32x4 xin[NIN > 0 ? NIN : 1];
@@ -251,6 +207,7 @@ __global__ void __launch_bounds__(WAVE) scan_kernel(const Op op, const int64_t n
             compute(tile * TT - my_shift, std::false_type{});
         else
             compute(tile * TT - my_shift, std::true_type{});
+        op.end_tile(st);
 
         if (NOUT > 0) {
             wave_sync();
@@ -277,38 +234,6 @@ __global__ void __launch_bounds__(WAVE) scan_kernel(const Op op, const int64_t n
 }
 
 // ---------------------------------------------------------------------------------------------
-// per-row helpers
-// ---------------------------------------------------------------------------------------------
-__device__ __forceinline__ float spike_count(float v, float theta, unsigned cap)
-{
-    // count = v >= theta ? min(unsigned(v / theta), cap) : 0      (IEEE division, truncation)
-    if (v >= theta) {
-        const unsigned k = static_cast<unsigned>(__fdiv_rn(v, theta));
-        return static_cast<float>(k < cap ? k : cap);
-    }
-    return 0.f;
-}
-
-template <int KIND>
-__device__ __forceinline__ float surrogate(float v, float theta, float p0, float p1, float row_a, float row_b)
-{
-    // row_a / row_b are per-row constants prepared in init()
-    if (KIND == EXODUS_SURR_SINGLE_EXP) {
-        // p1/(theta*p0) * exp(-|v - theta| / (theta*p0));  row_a = theta*p0, row_b = p1/(theta*p0)
-        return row_b * expf(-fabsf(v - theta) / row_a);
-    } else if (KIND == EXODUS_SURR_PERIODIC_EXP) {
-        // row_a = theta/2, row_b = p1/theta is NOT used so that the operation order stays
-        // p1 * (exp(.) / theta)
-        float u = v - row_a;
-        if (v >= theta) u = fmodf(u, theta);                 // u > 0 here, so fmod == floor-mod
-        return p1 * (expf(-fabsf(u - row_a) / p0) / theta);
-    } else {
-        // Heaviside window: row_a = theta - p0, row_b = 1/theta
-        return v >= row_a ? row_b : 0.f;
-    }
-}
-
-// ---------------------------------------------------------------------------------------------
 // Ops
 // ---------------------------------------------------------------------------------------------
 struct LeakyFwdOp {
@@ -329,6 +254,7 @@ struct LeakyFwdOp {
         s.v = __fadd_rn(__fmul_rn(s.v, s.a), x[0]);
         y[0] = s.v;
     }
+    __device__ __forceinline__ void end_tile(State &) const {}
     __device__ __forceinline__ void finish(State &, int64_t) const {}
 };
 
@@ -342,25 +268,27 @@ struct LeakyBwdOp {
     float *out[1];
     const float *v_init, *alpha;
     float *alpha_grad, *init_grad;
-    struct State { float g, a; double acc; };
+    struct State { float g, a; TileSum acc; };
     __device__ __forceinline__ void init(State &s, int64_t row, bool) const
     {
         s.g = 0.f;
         s.a = alpha[row];
-        s.acc = 0.0;
+        s.acc.clear();
     }
     __device__ __forceinline__ void step(State &s, const float *x, float *y) const
     {
-        if (ALPHA) s.acc += static_cast<double>(s.g) * static_cast<double>(x[1]);   // g_{u+1} * out_u
+        if (ALPHA) s.acc.add(s.g, x[1]);                          // g_{u+1} * out_u
         s.g = __fadd_rn(__fmul_rn(s.g, s.a), x[0]);
         if (WRITE_GI) y[0] = s.g;
     }
+    __device__ __forceinline__ void end_tile(State &s) const { if (ALPHA) s.acc.fold(); }
     __device__ __forceinline__ void finish(State &s, int64_t row) const
     {
         if (init_grad) init_grad[row] = __fmul_rn(s.a, s.g);
         if (ALPHA) {
-            s.acc += static_cast<double>(s.g) * static_cast<double>(v_init[row]);
-            alpha_grad[row] = static_cast<float>(s.acc);
+            s.acc.add(s.g, v_init[row]);
+            s.acc.fold();
+            alpha_grad[row] = static_cast<float>(s.acc.total);
         }
     }
 };
@@ -404,6 +332,7 @@ struct LifFwdOp {
         s.v = v;
         y[0] = v;
     }
+    __device__ __forceinline__ void end_tile(State &) const {}
     __device__ __forceinline__ void finish(State &, int64_t) const {}
 };
 
@@ -450,6 +379,7 @@ struct SynLifFwdOp {
         y[0] = v;
         y[1] = s.i;
     }
+    __device__ __forceinline__ void end_tile(State &) const {}
     __device__ __forceinline__ void finish(State &, int64_t) const {}
 };
 
@@ -468,8 +398,8 @@ struct LifBwdOp {
     float *alpha_grad, *init_grad;
     int apply_low;
     unsigned cap;
-    float p0, p1;
-    struct State { float lam, a, ac, c, th, lo, ra, rb; double acc; };
+    float p0, p1, inv_p0;
+    struct State { float lam, a, ac, c, th, lo; SurrConst k; TileSum acc; };
     __device__ __forceinline__ void init(State &s, int64_t row, bool) const
     {
         s.lam = 0.f;
@@ -478,41 +408,34 @@ struct LifBwdOp {
         s.ac = __fmul_rn(s.a, s.c);
         s.th = theta[row];
         s.lo = apply_low ? theta_low[row] : 0.f;
-        s.acc = 0.0;
-        if (KIND == EXODUS_SURR_SINGLE_EXP) {
-            s.ra = __fmul_rn(s.th, p0);
-            s.rb = __fdiv_rn(p1, s.ra);
-        } else if (KIND == EXODUS_SURR_PERIODIC_EXP) {
-            s.ra = __fmul_rn(s.th, 0.5f);
-            s.rb = 0.f;
-        } else {
-            s.ra = __fsub_rn(s.th, p0);
-            s.rb = __fdiv_rn(1.f, s.th);
-        }
+        s.acc.clear();
+        if constexpr (KIND != EXODUS_SURR_TENSOR) s.k = surrogate_consts<KIND>(s.th, p0, p1);
     }
     __device__ __forceinline__ void step(State &s, const float *x, float *y) const
     {
         const float v = x[1];
         float sg;
         if constexpr (KIND == EXODUS_SURR_TENSOR) sg = x[SURR_SLOT];
-        else sg = surrogate<KIND>(v, s.th, p0, p1, s.ra, s.rb);
+        else sg = surrogate<KIND>(v, s.th, inv_p0, s.k);
         float g = __fmul_rn(sg, x[0]);
         if constexpr (HAS_GV) g = __fadd_rn(g, x[GV_SLOT]);
         if (ALPHA) {
             const float vpost = __fsub_rn(v, __fmul_rn(s.c, spike_count(v, s.th, cap)));
-            s.acc += static_cast<double>(s.lam) * static_cast<double>(vpost);       // lambda_{u+1} * vpost_u
+            s.acc.add(s.lam, vpost);                              // lambda_{u+1} * vpost_u
         }
         const float f = __fsub_rn(s.a, __fmul_rn(s.ac, sg));
         const float lam = __fadd_rn(g, __fmul_rn(f, s.lam));
         s.lam = (apply_low && !(v > s.lo)) ? 0.f : lam;
         y[0] = s.lam;
     }
+    __device__ __forceinline__ void end_tile(State &s) const { if (ALPHA) s.acc.fold(); }
     __device__ __forceinline__ void finish(State &s, int64_t row) const
     {
         if (init_grad) init_grad[row] = __fmul_rn(s.a, s.lam);
         if (ALPHA) {
-            s.acc += static_cast<double>(s.lam) * static_cast<double>(v_init[row]);
-            alpha_grad[row] = static_cast<float>(s.acc);
+            s.acc.add(s.lam, v_init[row]);
+            s.acc.fold();
+            alpha_grad[row] = static_cast<float>(s.acc.total);
         }
     }
 };
@@ -538,8 +461,8 @@ struct SynLifBwdOp {
     float *alpha_mem_grad, *alpha_syn_grad, *v_init_grad, *i_init_grad;
     int apply_low, decay_early, norm_input;
     unsigned cap;
-    float p0, p1;
-    struct State { float lam, mu, am, as, amc, k, c, th, lo, ra, rb; double acc_m, acc_s; };
+    float p0, p1, inv_p0;
+    struct State { float lam, mu, am, as, amc, k, c, th, lo; SurrConst sk; TileSum acc_m, acc_s; };
     __device__ __forceinline__ void init(State &s, int64_t row, bool) const
     {
         s.lam = 0.f;
@@ -551,52 +474,51 @@ struct SynLifBwdOp {
         s.k = norm_input ? __fsub_rn(1.0f, s.am) : 1.0f;
         s.th = theta[row];
         s.lo = apply_low ? theta_low[row] : 0.f;
-        s.acc_m = 0.0;
-        s.acc_s = 0.0;
-        if (KIND == EXODUS_SURR_SINGLE_EXP) {
-            s.ra = __fmul_rn(s.th, p0);
-            s.rb = __fdiv_rn(p1, s.ra);
-        } else if (KIND == EXODUS_SURR_PERIODIC_EXP) {
-            s.ra = __fmul_rn(s.th, 0.5f);
-            s.rb = 0.f;
-        } else {
-            s.ra = __fsub_rn(s.th, p0);
-            s.rb = __fdiv_rn(1.f, s.th);
-        }
+        s.acc_m.clear();
+        s.acc_s.clear();
+        s.sk = surrogate_consts<KIND>(s.th, p0, p1);
     }
     __device__ __forceinline__ void step(State &s, const float *x, float *y) const
     {
         const float v = x[1], i = x[2];
-        const float sg = surrogate<KIND>(v, s.th, p0, p1, s.ra, s.rb);
+        const float sg = surrogate<KIND>(v, s.th, inv_p0, s.sk);
         float g = __fmul_rn(sg, x[0]);
         if constexpr (EXTRA) g = __fadd_rn(g, x[3]);
         const float vpost = __fsub_rn(v, __fmul_rn(s.c, spike_count(v, s.th, cap)));
-        s.acc_m += static_cast<double>(s.lam) * static_cast<double>(vpost);         // lambda_{u+1} * vpost_u
-        if (!decay_early) s.acc_s += static_cast<double>(s.mu) * static_cast<double>(i);   // mu_{u+1} * i_u
+        s.acc_m.add(s.lam, vpost);                                // lambda_{u+1} * vpost_u
+        if (!decay_early) s.acc_s.add(s.mu, i);                   // mu_{u+1} * i_u
         const float f = __fsub_rn(s.am, __fmul_rn(s.amc, sg));
         const float lam = __fadd_rn(g, __fmul_rn(f, s.lam));
         s.lam = (apply_low && !(v > s.lo)) ? 0.f : lam;
-        if (norm_input) s.acc_m -= static_cast<double>(s.lam) * static_cast<double>(i);
+        if (norm_input) s.acc_m.sub(s.lam, i);
         float du = __fmul_rn(s.lam, s.k);
         if constexpr (EXTRA) du = __fadd_rn(du, x[4]);
         s.mu = __fadd_rn(__fmul_rn(s.mu, s.as), du);
-        if (decay_early) s.acc_s += static_cast<double>(s.mu) * static_cast<double>(i);    // mu_u * i_u
+        if (decay_early) s.acc_s.add(s.mu, i);                    // mu_u * i_u
         y[0] = decay_early ? __fmul_rn(s.mu, s.as) : s.mu;
+    }
+    __device__ __forceinline__ void end_tile(State &s) const
+    {
+        s.acc_m.fold();
+        s.acc_s.fold();
     }
     __device__ __forceinline__ void finish(State &s, int64_t row) const
     {
         if (v_init_grad) v_init_grad[row] = __fmul_rn(s.am, s.lam);
         if (i_init_grad) i_init_grad[row] = __fmul_rn(s.as, s.mu);
         if (alpha_mem_grad) {
-            s.acc_m += static_cast<double>(s.lam) * static_cast<double>(v_init[row]);
-            alpha_mem_grad[row] = static_cast<float>(s.acc_m);
+            s.acc_m.add(s.lam, v_init[row]);
+            s.acc_m.fold();
+            alpha_mem_grad[row] = static_cast<float>(s.acc_m.total);
         }
         if (alpha_syn_grad) {
-            if (decay_early)
-                s.acc_s = s.acc_s / static_cast<double>(s.as);
-            else
-                s.acc_s += static_cast<double>(s.mu) * static_cast<double>(i_init[row]);
-            alpha_syn_grad[row] = static_cast<float>(s.acc_s);
+            if (decay_early) {
+                s.acc_s.total = s.acc_s.total / static_cast<double>(s.as);
+            } else {
+                s.acc_s.add(s.mu, i_init[row]);
+                s.acc_s.fold();
+            }
+            alpha_syn_grad[row] = static_cast<float>(s.acc_s.total);
         }
     }
 };
@@ -622,6 +544,7 @@ struct LifBwdTensorsOp {
         s.lam = __fmul_rn(x[2], __fadd_rn(x[0], __fmul_rn(f, s.lam)));
         y[0] = s.lam;
     }
+    __device__ __forceinline__ void end_tile(State &) const {}
     __device__ __forceinline__ void finish(State &, int64_t) const {}
 };
 
@@ -666,13 +589,13 @@ struct LifBwdAlphaTensorsOp {
         s.s_prev = x[1];
         s.vp_prev = x[3];
     }
+    __device__ __forceinline__ void end_tile(State &) const {}
     __device__ __forceinline__ void finish(State &s, int64_t row) const { alpha_grad[row] = static_cast<float>(s.acc); }
 };
 
 // ---------------------------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------------------------
-inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 template <class Op, int TT>
 int launch(const Op &op, int64_t n, int64_t t, void *stream)
@@ -729,6 +652,7 @@ int launch_lif_bwd(float *input_grad, float *alpha_grad, float *init_grad, const
     op.cap = static_cast<unsigned>(max_spikes);
     op.p0 = p0;
     op.p1 = p1;
+    op.inv_p0 = p0 != 0.f ? 1.f / p0 : 0.f;
     if constexpr (Op::NIN <= 2) return launch<Op, EXODUS_TT_1>(op, n, t, stream);
     else return launch<Op, EXODUS_TT_3>(op, n, t, stream);
 }
@@ -788,6 +712,7 @@ int launch_synlif_bwd(float *grad_input, float *alpha_mem_grad, float *alpha_syn
     op.cap = static_cast<unsigned>(max_spikes);
     op.p0 = p0;
     op.p1 = p1;
+    op.inv_p0 = p0 != 0.f ? 1.f / p0 : 0.f;
     return launch<Op, EXODUS_TT_3>(op, n, t, stream);
 }
 

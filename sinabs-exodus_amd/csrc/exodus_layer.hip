@@ -1,0 +1,429 @@
+// Layer-layout kernels of libexodus_hip.so: the spiking layer computed directly on the layer's own
+// (batch, time, neurons) tensors, neurons contiguous.
+//
+// In this layout the time recurrence of a neuron walks memory with stride `neurons`, and
+// adjacent lanes hold adjacent neurons: every wave-wide load or store is one contiguous segment,
+// so nothing has to be transposed (neither by torch before the kernel, as the (rows, time)
+// Functions need, nor through LDS).  One lane owns NPL adjacent neurons of one batch element.
+//
+// The forward pass writes only what the layer hands out -- the spike raster and the final
+// states -- plus one checkpoint of (post-reset potential, synaptic current) every CKPT steps.
+// The backward pass reads the input again, rebuilds each CKPT-step chunk of membrane potential
+// and synaptic current in registers from its checkpoint (same operations, same order, hence the
+// same bits as the forward pass produced) and then walks the chunk in reverse.  Per
+// neuron-timestep this moves 8 B forward (x in, spikes out) and 12 B backward (grad_spikes and x
+// in, grad_x out) plus 16 B per 32 steps of checkpoints, instead of the 32 B of a forward that
+// stores v_mem and i_syn for the backward to read.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "exodus_common.hpp"
+
+namespace {
+
+constexpr int CKPT = 32;      // steps between checkpoints = length of a backward chunk
+constexpr int FWD_UNROLL = 8; // forward steps per software-pipeline stage (divides CKPT)
+constexpr int BLOCK = 256;
+
+struct LayerConsts {
+    const float *v_init, *i_init, *alpha_mem, *alpha_syn, *c, *theta, *theta_low;
+    int apply_low, decay_early, norm_input;
+    unsigned cap;
+};
+
+template <int NPL> struct Vec;
+template <> struct Vec<1> { typedef float type; };
+template <> struct Vec<4> { typedef f32x4 type; };
+
+template <int NPL> __device__ __forceinline__ float lane_get(const typename Vec<NPL>::type &v, int e);
+template <> __device__ __forceinline__ float lane_get<1>(const float &v, int) { return v; }
+template <> __device__ __forceinline__ float lane_get<4>(const f32x4 &v, int e) { return v[e]; }
+template <int NPL> __device__ __forceinline__ void lane_put(typename Vec<NPL>::type &v, int e, float x);
+template <> __device__ __forceinline__ void lane_put<1>(float &v, int, float x) { v = x; }
+template <> __device__ __forceinline__ void lane_put<4>(f32x4 &v, int e, float x) { v[e] = x; }
+
+// per-neuron constants and running state of the forward recurrence
+struct Neuron {
+    float am, as, k, c, th, lo;     // decay factors, 1 - alpha_mem, subtract value, threshold, lower bound
+    float vpost, i;                 // potential after the reset of the previous step, synaptic current
+};
+
+template <bool SYN>
+__device__ __forceinline__ void neuron_load(Neuron &n, const LayerConsts &p, int64_t row)
+{
+    n.am = p.alpha_mem[row];
+    n.as = SYN ? p.alpha_syn[row] : 0.f;
+    n.k = __fsub_rn(1.0f, n.am);
+    n.c = p.c[row];
+    n.th = p.theta[row];
+    n.lo = p.apply_low ? p.theta_low[row] : 0.f;
+}
+
+// One step of the layer's forward arithmetic, in the order the composed layer performs it
+// (input scaling, synapse, input normalisation, membrane, clamp, threshold):
+//   xin = decay_early ? x * a_syn : x;  i = i * a_syn + xin   (SYN; otherwise i = x)
+//   u = norm_input ? (1 - a_mem) * i : i;   v = vpost * a_mem + u;   clamp;   count from v
+// Returns the pre-reset potential v; `count` is the spike count; n.vpost / n.i are advanced.
+template <bool SYN>
+__device__ __forceinline__ float neuron_step(Neuron &n, const LayerConsts &p, float x, float &count)
+{
+    if (SYN) {
+        const float xin = p.decay_early ? __fmul_rn(x, n.as) : x;
+        n.i = __fadd_rn(__fmul_rn(n.i, n.as), xin);
+    } else {
+        n.i = x;
+    }
+    const float u = p.norm_input ? __fmul_rn(n.k, n.i) : n.i;
+    float v = __fadd_rn(__fmul_rn(n.vpost, n.am), u);
+    if (p.apply_low && v < n.lo) v = n.lo;
+    count = spike_count(v, n.th, p.cap);
+    n.vpost = __fsub_rn(v, __fmul_rn(count, n.c));
+    return v;
+}
+
+// ---------------------------------------------------------------------------------------------
+// forward
+// ---------------------------------------------------------------------------------------------
+template <bool SYN, int NPL>
+__global__ void __launch_bounds__(BLOCK) layer_lif_forward(
+    float *__restrict__ spikes, float *__restrict__ v_rec, float *__restrict__ i_rec, float *__restrict__ ckpt_v,
+    float *__restrict__ ckpt_i, float *__restrict__ v_last, float *__restrict__ i_last, double *spike_sum,
+    const float *__restrict__ x, const LayerConsts p, const int64_t blocks_per_batch, const int64_t T,
+    const int64_t M)
+{
+    typedef typename Vec<NPL>::type V;
+    // A block works inside one batch element: block-uniform base pointers plus a small lane offset,
+    // so that addresses cost scalar registers only.
+    const int64_t b = blockIdx.x / blocks_per_batch;
+    const int64_t m0 = static_cast<int64_t>(blockIdx.x - b * blocks_per_batch) * (BLOCK * NPL);
+    const unsigned lane_off = threadIdx.x * NPL;
+    const int64_t first = b * M + m0 + lane_off;              // first neuron (row) of this lane
+    double my_spikes = 0.0;
+    if (m0 + lane_off < M) {
+        const int64_t n_ck = (T + CKPT - 1) / CKPT;
+        const float *xp = x + (b * T) * M + m0;
+        float *sp = spikes + (b * T) * M + m0;
+        float *vrp = v_rec ? v_rec + (b * T) * M + m0 : nullptr;
+        float *irp = i_rec ? i_rec + (b * T) * M + m0 : nullptr;
+        float *cvp = ckpt_v ? ckpt_v + (b * n_ck) * M + m0 : nullptr;
+        float *cip = (SYN && ckpt_i) ? ckpt_i + (b * n_ck) * M + m0 : nullptr;
+
+        Neuron nr[NPL];
+#pragma unroll
+        for (int e = 0; e < NPL; ++e) {
+            neuron_load<SYN>(nr[e], p, first + e);
+            nr[e].vpost = p.v_init[first + e];
+            nr[e].i = SYN ? p.i_init[first + e] : 0.f;
+        }
+
+        V cur[FWD_UNROLL], nxt[FWD_UNROLL];
+        auto fetch = [&](V(&dst)[FWD_UNROLL], int64_t t0) {
+#pragma unroll
+            for (int u = 0; u < FWD_UNROLL; ++u)
+                if (t0 + u < T) dst[u] = ld_stream(reinterpret_cast<const V *>(xp + (t0 + u) * M + lane_off));
+        };
+        fetch(cur, 0);
+        float part = 0.f;                                     // spike count of the current chunk (exact in fp32)
+        for (int64_t t0 = 0; t0 < T; t0 += FWD_UNROLL) {
+            if (t0 + FWD_UNROLL < T) fetch(nxt, t0 + FWD_UNROLL);
+            if ((t0 % CKPT) == 0) {
+                if (cvp) {
+                    V cv, ci;
+#pragma unroll
+                    for (int e = 0; e < NPL; ++e) {
+                        lane_put<NPL>(cv, e, nr[e].vpost);
+                        lane_put<NPL>(ci, e, nr[e].i);
+                    }
+                    st_stream(cv, reinterpret_cast<V *>(cvp + (t0 / CKPT) * M + lane_off));
+                    if (cip) st_stream(ci, reinterpret_cast<V *>(cip + (t0 / CKPT) * M + lane_off));
+                }
+                my_spikes += static_cast<double>(part);
+                part = 0.f;
+            }
+#pragma unroll
+            for (int u = 0; u < FWD_UNROLL; ++u) {
+                const int64_t t = t0 + u;
+                if (t < T) {
+                    V s, vr, ir;
+#pragma unroll
+                    for (int e = 0; e < NPL; ++e) {
+                        float count;
+                        neuron_step<SYN>(nr[e], p, lane_get<NPL>(cur[u], e), count);
+                        lane_put<NPL>(s, e, count);
+                        lane_put<NPL>(vr, e, nr[e].vpost);
+                        lane_put<NPL>(ir, e, nr[e].i);
+                        part += count;
+                    }
+                    st_stream(s, reinterpret_cast<V *>(sp + t * M + lane_off));
+                    if (vrp) st_stream(vr, reinterpret_cast<V *>(vrp + t * M + lane_off));
+                    if (irp) st_stream(ir, reinterpret_cast<V *>(irp + t * M + lane_off));
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < FWD_UNROLL; ++u) cur[u] = nxt[u];
+        }
+        my_spikes += static_cast<double>(part);
+#pragma unroll
+        for (int e = 0; e < NPL; ++e) {
+            v_last[first + e] = nr[e].vpost;
+            if (SYN && i_last) i_last[first + e] = nr[e].i;
+        }
+    }
+    if (spike_sum) {
+        // wave reduction, then one atomic per wave
+#pragma unroll
+        for (int off = WAVE / 2; off > 0; off >>= 1) my_spikes += __shfl_xor(my_spikes, off, WAVE);
+        if ((threadIdx.x & (WAVE - 1)) == 0 && my_spikes != 0.0) atomicAdd(spike_sum, my_spikes);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// backward
+// ---------------------------------------------------------------------------------------------
+// With lambda_t = dL/du_t (membrane adjoint) and mu_t = dL/di_t (synapse adjoint):
+//   g_t      = s_t * grad_spikes_t              (at the last step the gradients of the final states
+//                                                join in: see below)
+//   lambda_t = nc_t (g_t + (a_mem - a_mem c s_t) lambda_{t+1})
+//   mu_t     = a_syn mu_{t+1} + k lambda_t,     k = norm_input ? 1 - a_mem : 1
+//   grad_x_t = decay_early ? a_syn mu_t : mu_t  (no synapse: grad_x_t = k lambda_t)
+//   grad_alpha_mem = sum_t lambda_t vpost_{t-1} - (norm_input ? sum_t lambda_t i_t : 0)
+//   grad_alpha_syn = decay_early ? (sum_t mu_t i_t) / a_syn : sum_t mu_t i_{t-1}
+//   grad_v_init = a_mem lambda_0,  grad_i_init = a_syn mu_0
+// The final potential handed out by the forward is vpost_{T-1} = v_{T-1} - c count_{T-1}; a gradient
+// gv on it reaches v_{T-1} directly and the spike count with weight -c, a gradient on the final
+// synaptic current adds to mu_{T-1}.
+template <bool SYN, int KIND>
+__global__ void __launch_bounds__(BLOCK) layer_lif_backward(
+    float *__restrict__ grad_x, float *__restrict__ alpha_mem_grad, float *__restrict__ alpha_syn_grad,
+    float *__restrict__ v_init_grad, float *__restrict__ i_init_grad, const float *__restrict__ grad_spikes,
+    const float *__restrict__ grad_v_last, const float *__restrict__ grad_i_last, const float *__restrict__ x,
+    const float *__restrict__ ckpt_v, const float *__restrict__ ckpt_i, const LayerConsts p, const float p0,
+    const float p1, const float inv_p0, const int64_t blocks_per_batch, const int64_t T, const int64_t M)
+{
+    const int64_t b = blockIdx.x / blocks_per_batch;
+    const int64_t m0 = static_cast<int64_t>(blockIdx.x - b * blocks_per_batch) * BLOCK;
+    const unsigned lane_off = threadIdx.x;
+    if (m0 + lane_off >= M) return;
+    const int64_t row = b * M + m0 + lane_off;
+    const int64_t n_ck = (T + CKPT - 1) / CKPT;
+    // block-uniform bases; the lane offset is added at each access
+    const float *xp = x + (b * T) * M + m0;
+    const float *gp = grad_spikes + (b * T) * M + m0;
+    float *op = grad_x + (b * T) * M + m0;
+    const float *cvp = ckpt_v + (b * n_ck) * M + m0;
+    const float *cip = SYN ? ckpt_i + (b * n_ck) * M + m0 : nullptr;
+
+    Neuron nr;
+    neuron_load<SYN>(nr, p, row);
+    const float amc = __fmul_rn(nr.am, nr.c);
+    const float kk = p.norm_input ? nr.k : 1.0f;
+    const SurrConst sk = surrogate_consts<KIND>(nr.th, p0, p1);
+    const float gvl = grad_v_last ? grad_v_last[row] : 0.f;
+    const float gil = (SYN && grad_i_last) ? grad_i_last[row] : 0.f;
+
+    float lam = 0.f, mu = 0.f;
+    TileSum acc_m, acc_s;
+    acc_m.clear();
+    acc_s.clear();
+
+    for (int64_t j = n_ck - 1; j >= 0; --j) {
+        const int64_t t0 = j * CKPT;
+        const int len = (T - t0) < CKPT ? static_cast<int>(T - t0) : CKPT;
+        float xr[CKPT], gr[CKPT], vr[CKPT];
+#pragma unroll
+        for (int k = 0; k < CKPT; ++k)
+            if (k < len) {
+                xr[k] = ld_stream(xp + (t0 + k) * M + lane_off);
+                gr[k] = ld_stream(gp + (t0 + k) * M + lane_off);
+            }
+        nr.vpost = ld_stream(cvp + j * M + lane_off);
+        nr.i = SYN ? ld_stream(cip + j * M + lane_off) : 0.f;
+
+        // rebuild the chunk: vr[k] = pre-reset potential, xr[k] = synaptic current (the value that
+        // was normalised and fed to the membrane; without synapse that is the input itself)
+#pragma unroll
+        for (int k = 0; k < CKPT; ++k)
+            if (k < len) {
+                float count;
+                vr[k] = neuron_step<SYN>(nr, p, xr[k], count);
+                xr[k] = nr.i;
+            }
+
+        // reverse walk
+#pragma unroll
+        for (int kq = 0; kq < CKPT; ++kq) {
+            const int k = CKPT - 1 - kq;
+            if (k < len) {
+                const float v = vr[k], cur_i = xr[k];
+                const float sg = surrogate<KIND>(v, nr.th, inv_p0, sk);
+                float g;
+                if (t0 + k == T - 1 && grad_v_last) {
+                    g = __fadd_rn(__fmul_rn(sg, __fsub_rn(gr[k], __fmul_rn(nr.c, gvl))), gvl);
+                } else {
+                    g = __fmul_rn(sg, gr[k]);
+                }
+                const float vpost = __fsub_rn(v, __fmul_rn(nr.c, spike_count(v, nr.th, p.cap)));
+                acc_m.add(lam, vpost);                          // lambda_{t+1} * vpost_t
+                if (SYN && !p.decay_early) acc_s.add(mu, cur_i);   // mu_{t+1} * i_t
+                const float f = __fsub_rn(nr.am, __fmul_rn(amc, sg));
+                const float l = __fadd_rn(g, __fmul_rn(f, lam));
+                lam = (p.apply_low && !(v > nr.lo)) ? 0.f : l;
+                if (p.norm_input) acc_m.sub(lam, cur_i);
+                float du = __fmul_rn(lam, kk);
+                if (SYN) {
+                    if (t0 + k == T - 1) du = __fadd_rn(du, gil);
+                    mu = __fadd_rn(__fmul_rn(mu, nr.as), du);
+                    if (p.decay_early) acc_s.add(mu, cur_i);    // mu_t * i_t
+                    gr[k] = p.decay_early ? __fmul_rn(mu, nr.as) : mu;
+                } else {
+                    gr[k] = du;
+                }
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < CKPT; ++k)
+            if (k < len) st_stream(gr[k], op + (t0 + k) * M + lane_off);
+        acc_m.fold();
+        acc_s.fold();
+    }
+
+    if (v_init_grad) v_init_grad[row] = __fmul_rn(nr.am, lam);
+    if (SYN && i_init_grad) i_init_grad[row] = __fmul_rn(nr.as, mu);
+    if (alpha_mem_grad) {
+        acc_m.add(lam, p.v_init[row]);
+        acc_m.fold();
+        alpha_mem_grad[row] = static_cast<float>(acc_m.total);
+    }
+    if (SYN && alpha_syn_grad) {
+        if (p.decay_early) {
+            acc_s.total = acc_s.total / static_cast<double>(nr.as);
+        } else {
+            acc_s.add(mu, p.i_init[row]);
+            acc_s.fold();
+        }
+        alpha_syn_grad[row] = static_cast<float>(acc_s.total);
+    }
+}
+
+inline bool bad3(int64_t b, int64_t t, int64_t m)
+{
+    if (b < 0 || t < 0 || m < 0) return true;
+    if (b == 0 || t == 0 || m == 0) return false;
+    if (b > INT64_MAX / t) return true;
+    return (b * t) > INT64_MAX / m;
+}
+
+template <bool SYN, int KIND>
+int launch_bwd(float *grad_x, float *am_g, float *as_g, float *v0_g, float *i0_g, const float *grad_spikes,
+               const float *gvl, const float *gil, const float *x, const float *ckpt_v, const float *ckpt_i,
+               const LayerConsts &p, float p0, float p1, int64_t B, int64_t T, int64_t M, hipStream_t s)
+{
+    const int64_t blocks_per_batch = (M + BLOCK - 1) / BLOCK;
+    if (blocks_per_batch > 0x7fffffffLL / B) return hipErrorInvalidValue;
+    const int64_t blocks = blocks_per_batch * B;
+    hipLaunchKernelGGL((layer_lif_backward<SYN, KIND>), dim3(static_cast<unsigned>(blocks)), dim3(BLOCK), 0, s, grad_x,
+                       am_g, as_g, v0_g, i0_g, grad_spikes, gvl, gil, x, ckpt_v, ckpt_i, p, p0, p1,
+                       p0 != 0.f ? 1.f / p0 : 0.f, blocks_per_batch, T, M);
+    return static_cast<int>(hipGetLastError());
+}
+
+}  // namespace
+
+extern "C" {
+
+#define EXODUS_API __attribute__((visibility("default")))
+
+EXODUS_API int exodus_layer_checkpoint_interval(void) { return CKPT; }
+
+EXODUS_API int exodus_layer_lif_forward(float *out_spikes, float *out_vmem_rec, float *out_isyn_rec, float *ckpt_v,
+                                        float *ckpt_i, float *v_last, float *i_last, double *spike_sum,
+                                        const float *input, const float *vmem_post_initial,
+                                        const float *isyn_initial, const float *alpha_mem, const float *alpha_syn,
+                                        const float *membr_subtract, const float *theta, const float *theta_low,
+                                        int apply_theta_low, int max_num_spikes, int decay_early, int norm_input,
+                                        int64_t batch, int64_t t, int64_t neurons, void *stream)
+{
+    if (bad3(batch, t, neurons)) return hipErrorInvalidValue;
+    if (batch == 0 || t == 0 || neurons == 0) return hipSuccess;
+    const bool syn = alpha_syn != nullptr;
+    if (!out_spikes || !v_last || !input || !vmem_post_initial || !alpha_mem || !membr_subtract || !theta ||
+        (apply_theta_low && !theta_low) || (syn && !isyn_initial) || (syn && ckpt_v && !ckpt_i))
+        return hipErrorInvalidValue;
+    LayerConsts p;
+    p.v_init = vmem_post_initial;
+    p.i_init = isyn_initial;
+    p.alpha_mem = alpha_mem;
+    p.alpha_syn = alpha_syn;
+    p.c = membr_subtract;
+    p.theta = theta;
+    p.theta_low = theta_low;
+    p.apply_low = apply_theta_low ? 1 : 0;
+    p.decay_early = decay_early ? 1 : 0;
+    p.norm_input = norm_input ? 1 : 0;
+    p.cap = static_cast<unsigned>(max_num_spikes);
+    // four neurons per lane need 16-byte aligned rows of every (batch, time, neurons) tensor
+    bool vec = (neurons % 4) == 0 && aligned16(input) && aligned16(out_spikes) && aligned16(out_vmem_rec) &&
+               aligned16(out_isyn_rec) && aligned16(ckpt_v) && aligned16(ckpt_i);
+    const int npl = vec ? 4 : 1;
+    const int64_t blocks_per_batch = (neurons + BLOCK * npl - 1) / (BLOCK * npl);
+    if (blocks_per_batch > 0x7fffffffLL / batch) return hipErrorInvalidValue;
+    const int64_t blocks = blocks_per_batch * batch;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const dim3 grid(static_cast<unsigned>(blocks)), block(BLOCK);
+#define EXODUS_FWD(SYN, NPL)                                                                                     \
+    hipLaunchKernelGGL((layer_lif_forward<SYN, NPL>), grid, block, 0, s, out_spikes, out_vmem_rec, out_isyn_rec, \
+                       ckpt_v, ckpt_i, v_last, i_last, spike_sum, input, p, blocks_per_batch, t, neurons)
+    if (syn) {
+        if (vec) EXODUS_FWD(true, 4); else EXODUS_FWD(true, 1);
+    } else {
+        if (vec) EXODUS_FWD(false, 4); else EXODUS_FWD(false, 1);
+    }
+#undef EXODUS_FWD
+    return static_cast<int>(hipGetLastError());
+}
+
+EXODUS_API int exodus_layer_lif_backward(float *grad_input, float *alpha_mem_grad, float *alpha_syn_grad,
+                                         float *vmem_init_grad, float *isyn_init_grad, const float *grad_spikes,
+                                         const float *grad_v_last, const float *grad_i_last, const float *input,
+                                         const float *ckpt_v, const float *ckpt_i, const float *vmem_post_initial,
+                                         const float *isyn_initial, const float *alpha_mem, const float *alpha_syn,
+                                         const float *membr_subtract, const float *theta, const float *theta_low,
+                                         int apply_theta_low, int max_num_spikes, int decay_early, int norm_input,
+                                         int surrogate_kind, float surr_p0, float surr_p1, int64_t batch, int64_t t,
+                                         int64_t neurons, void *stream)
+{
+    if (bad3(batch, t, neurons)) return hipErrorInvalidValue;
+    if (batch == 0 || t == 0 || neurons == 0) return hipSuccess;
+    const bool syn = alpha_syn != nullptr;
+    if (!grad_input || !grad_spikes || !input || !ckpt_v || !alpha_mem || !membr_subtract || !theta ||
+        (apply_theta_low && !theta_low) || (syn && !ckpt_i))
+        return hipErrorInvalidValue;
+    if (alpha_mem_grad && !vmem_post_initial) return hipErrorInvalidValue;
+    if (syn && alpha_syn_grad && !decay_early && !isyn_initial) return hipErrorInvalidValue;
+    LayerConsts p;
+    p.v_init = vmem_post_initial;
+    p.i_init = isyn_initial;
+    p.alpha_mem = alpha_mem;
+    p.alpha_syn = alpha_syn;
+    p.c = membr_subtract;
+    p.theta = theta;
+    p.theta_low = theta_low;
+    p.apply_low = apply_theta_low ? 1 : 0;
+    p.decay_early = decay_early ? 1 : 0;
+    p.norm_input = norm_input ? 1 : 0;
+    p.cap = static_cast<unsigned>(max_num_spikes);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+#define EXODUS_BWD(SYN, K)                                                                                        \
+    return launch_bwd<SYN, K>(grad_input, alpha_mem_grad, alpha_syn_grad, vmem_init_grad, isyn_init_grad,         \
+                              grad_spikes, grad_v_last, grad_i_last, input, ckpt_v, ckpt_i, p, surr_p0, surr_p1, \
+                              batch, t, neurons, s)
+    switch (surrogate_kind) {
+        case EXODUS_SURR_SINGLE_EXP: if (syn) EXODUS_BWD(true, EXODUS_SURR_SINGLE_EXP); EXODUS_BWD(false, EXODUS_SURR_SINGLE_EXP);
+        case EXODUS_SURR_PERIODIC_EXP: if (syn) EXODUS_BWD(true, EXODUS_SURR_PERIODIC_EXP); EXODUS_BWD(false, EXODUS_SURR_PERIODIC_EXP);
+        case EXODUS_SURR_HEAVISIDE: if (syn) EXODUS_BWD(true, EXODUS_SURR_HEAVISIDE); EXODUS_BWD(false, EXODUS_SURR_HEAVISIDE);
+        default: return hipErrorInvalidValue;
+    }
+#undef EXODUS_BWD
+}
+
+}  // extern "C"

@@ -10,6 +10,7 @@ import of this module fails with an ``ImportError`` that says how to build it.
 from __future__ import annotations
 
 import ctypes
+import math
 import os
 from typing import Optional
 
@@ -40,6 +41,9 @@ _SIGNATURES = {
     "exodus_lif_backward_fused": ([_p] * 12 + [_int, _int, _int, _f, _f, _i64, _i64, _p], _int),
     "exodus_synlif_forward": ([_p] * 11 + [_int, _int, _int, _int, _i64, _i64, _p], _int),
     "exodus_synlif_backward": ([_p] * 17 + [_int, _int, _int, _int, _int, _f, _f, _i64, _i64, _p], _int),
+    "exodus_layer_checkpoint_interval": ([], _int),
+    "exodus_layer_lif_forward": ([_p] * 16 + [_int, _int, _int, _int, _i64, _i64, _i64, _p], _int),
+    "exodus_layer_lif_backward": ([_p] * 18 + [_int, _int, _int, _int, _int, _f, _f, _i64, _i64, _i64, _p], _int),
 }
 
 
@@ -357,3 +361,108 @@ def synLifBackward(gradSpikes, gradVmem, gradIsyn, vmem, isyn, vmemPostInitial, 
                                           int(bool(normInput)), int(surrogateKind), float(surrP0), float(surrP1),
                                           n, t, _stream(vmem)), "exodus_synlif_backward")
     return (inputGrad, *per_row)
+
+
+# ------------------------------------------------------------------------------------------
+# layer-layout kernels: (batch, time, neurons) tensors, no transposition
+# ------------------------------------------------------------------------------------------
+
+def checkpointInterval() -> int:
+    return int(lib.exodus_layer_checkpoint_interval())
+
+
+def _btm(x: torch.Tensor, name: str, like: Optional[torch.Tensor] = None):
+    _dev(x, name, like)
+    if x.ndim != 3:
+        raise RuntimeError(f"{name} must be 3-D (batch, time, neurons)")
+    return x
+
+
+def layerLifForward(input, vmemPostInitial, isynInitial, alphaMem, alphaSyn, membrSubtract, theta, thetaLow,
+                    applyThetaLow: bool, maxNumSpikes: int, decayEarly: bool, normInput: bool,
+                    wantCheckpoints: bool = True, wantRecords: bool = False, wantSpikeSum: bool = True,
+                    outSpikes: Optional[torch.Tensor] = None, stateShape: Optional[tuple] = None):
+    """Returns dict(spikes, v_last, i_last, ckpt_v, ckpt_i, v_rec, i_rec, spike_sum); absent items are None.
+    ``stateShape`` (product = batch*neurons) gives v_last / i_last that shape instead of a flat vector."""
+    _btm(input, "input")
+    b, t, m = input.shape
+    n = b * m
+    syn = alphaSyn is not None
+    rows = [("vmemPostInitial", vmemPostInitial), ("alphaMem", alphaMem), ("membrSubtract", membrSubtract),
+            ("theta", theta)]
+    if syn:
+        rows += [("isynInitial", isynInitial), ("alphaSyn", alphaSyn)]
+    for nm, x in rows:
+        _rows(_dev(x, nm, input), nm, n)
+    if applyThetaLow:
+        _rows(_dev(thetaLow, "thetaLow", input), "thetaLow", n)
+    else:
+        thetaLow = None
+    spikes = torch.empty_like(input) if outSpikes is None else outSpikes
+    if spikes.shape != input.shape:
+        raise RuntimeError("outSpikes must have the shape of input")
+    _dev(spikes, "outSpikes", input)
+    new = lambda *shape: torch.empty(shape, dtype=torch.float32, device=input.device)
+    n_ck = (t + checkpointInterval() - 1) // checkpointInterval()
+    state_shape = (n,) if stateShape is None else tuple(stateShape)
+    if math.prod(state_shape) != n:
+        raise RuntimeError(f"stateShape {state_shape} does not hold {n} neurons")
+    res = dict(spikes=spikes, v_last=new(*state_shape), i_last=new(*state_shape) if syn else None,
+               ckpt_v=new(b, n_ck, m) if wantCheckpoints else None,
+               ckpt_i=new(b, n_ck, m) if (wantCheckpoints and syn) else None,
+               v_rec=new(b, t, m) if wantRecords else None, i_rec=new(b, t, m) if (wantRecords and syn) else None,
+               spike_sum=torch.zeros((), dtype=torch.float64, device=input.device) if wantSpikeSum else None)
+    with torch.cuda.device(input.device):
+        _check(lib.exodus_layer_lif_forward(
+            _ptr(spikes), _ptr(res["v_rec"]), _ptr(res["i_rec"]), _ptr(res["ckpt_v"]), _ptr(res["ckpt_i"]),
+            _ptr(res["v_last"]), _ptr(res["i_last"]), _ptr(res["spike_sum"]), _ptr(input), _ptr(vmemPostInitial),
+            _ptr(isynInitial) if syn else None, _ptr(alphaMem), _ptr(alphaSyn) if syn else None, _ptr(membrSubtract),
+            _ptr(theta), _ptr(thetaLow), int(bool(applyThetaLow)), int(maxNumSpikes), int(bool(decayEarly)),
+            int(bool(normInput)), b, t, m, _stream(input)), "exodus_layer_lif_forward")
+    return res
+
+
+def layerLifBackward(gradSpikes, gradVLast, gradILast, input, ckptV, ckptI, vmemPostInitial, isynInitial, alphaMem,
+                     alphaSyn, membrSubtract, theta, thetaLow, applyThetaLow: bool, maxNumSpikes: int,
+                     decayEarly: bool, normInput: bool, surrogateKind: int, surrP0: float, surrP1: float,
+                     gradInput: Optional[torch.Tensor] = None):
+    """Returns (gradInput, alphaMemGrad, alphaSynGrad | None, vInitGrad, iInitGrad | None)."""
+    _btm(input, "input")
+    b, t, m = input.shape
+    n = b * m
+    syn = alphaSyn is not None
+    if _btm(gradSpikes, "gradSpikes", input).shape != input.shape:
+        raise RuntimeError("gradSpikes must have the shape of input")
+    n_ck = (t + checkpointInterval() - 1) // checkpointInterval()
+    for nm, x in (("ckptV", ckptV),) + ((("ckptI", ckptI),) if syn else ()):
+        if _btm(x, nm, input).shape != (b, n_ck, m):
+            raise RuntimeError(f"{nm} must have shape ({b}, {n_ck}, {m})")
+    rows = [("vmemPostInitial", vmemPostInitial), ("alphaMem", alphaMem), ("membrSubtract", membrSubtract),
+            ("theta", theta)]
+    if syn:
+        rows += [("isynInitial", isynInitial), ("alphaSyn", alphaSyn)]
+    for nm, x in rows:
+        _rows(_dev(x, nm, input), nm, n)
+    for nm, x in (("gradVLast", gradVLast), ("gradILast", gradILast if syn else None)):
+        if x is not None and _dev(x, nm, input).numel() != n:
+            raise RuntimeError(f"{nm} must hold {n} values")
+    if applyThetaLow:
+        _rows(_dev(thetaLow, "thetaLow", input), "thetaLow", n)
+    else:
+        thetaLow = None
+    if gradInput is None:
+        gradInput = torch.empty_like(input)
+    elif _btm(gradInput, "gradInput", input).shape != input.shape:
+        raise RuntimeError("gradInput must have the shape of input")
+    z = lambda: torch.zeros(n, dtype=torch.float32, device=input.device)
+    am_g, v0_g = z(), z()
+    as_g, i0_g = (z(), z()) if syn else (None, None)
+    with torch.cuda.device(input.device):
+        _check(lib.exodus_layer_lif_backward(
+            _ptr(gradInput), _ptr(am_g), _ptr(as_g), _ptr(v0_g), _ptr(i0_g), _ptr(gradSpikes), _ptr(gradVLast),
+            _ptr(gradILast) if syn else None, _ptr(input), _ptr(ckptV), _ptr(ckptI) if syn else None,
+            _ptr(vmemPostInitial), _ptr(isynInitial) if syn else None, _ptr(alphaMem), _ptr(alphaSyn) if syn else None,
+            _ptr(membrSubtract), _ptr(theta), _ptr(thetaLow), int(bool(applyThetaLow)), int(maxNumSpikes),
+            int(bool(decayEarly)), int(bool(normInput)), int(surrogateKind), float(surrP0), float(surrP1), b, t, m,
+            _stream(input)), "exodus_layer_lif_backward")
+    return gradInput, am_g, as_g, v0_g, i0_g

@@ -1,0 +1,103 @@
+"""``SpikingLayerFunction``: a whole LIF/IAF layer pass on the layer's own (batch, time, neurons)
+layout, one kernel per direction.
+
+What the reference layer does with two transposing copies, up to two autograd Functions and
+several elementwise passes (reference sinabs/exodus/layers/lif.py:152-307) happens here inside
+the kernels: synaptic current, input normalisation, membrane update, clamp, threshold, reset,
+final states and the spike total for ``firing_rate``.  The forward keeps only checkpoints; the
+backward re-reads the input and rebuilds membrane potential and synaptic current chunk by chunk,
+so neither is ever written to memory in full.
+"""
+from typing import Callable, Optional
+
+import torch
+
+from . import _hip
+from .spike import classify_surrogate
+
+
+class SpikingLayerFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(
+        ctx,
+        inp: torch.Tensor,                      # (batch, time, neurons), contiguous
+        alpha_mem: torch.Tensor,                # (batch*neurons,)
+        alpha_syn: Optional[torch.Tensor],      # (batch*neurons,) or None: no synaptic current
+        v_mem_init: torch.Tensor,               # (batch*neurons,) potential after reset
+        i_syn_init: Optional[torch.Tensor],     # (batch*neurons,) or None
+        threshold: torch.Tensor,
+        membrane_subtract: Optional[torch.Tensor],
+        min_v_mem: Optional[torch.Tensor],
+        surrogate_grad_fn: Callable,
+        max_num_spikes_per_bin: Optional[int],
+        decay_early: bool,
+        norm_input: bool,
+        state_shape: Optional[tuple] = None,
+    ):
+        """Returns ``(spikes (batch,time,neurons), v_mem_last, i_syn_last | None, spike_total)``;
+        ``v_mem_last`` is the potential after the last reset, ``spike_total`` a float64 scalar
+        (not differentiable).  The final states come as flat vectors, or in ``state_shape`` if given."""
+        kind, p0, p1 = classify_surrogate(surrogate_grad_fn)
+        if kind == _hip.SURR_TENSOR:
+            raise ValueError("surrogate_grad_fn is not one the layer kernel can evaluate")
+        if inp.ndim != 3:
+            raise ValueError("'inp' must be 3D, (batch, time, neurons)")
+        if not inp.is_contiguous():
+            raise ValueError("'inp' has to be contiguous.")
+        if membrane_subtract is None:
+            membrane_subtract = threshold
+        syn = alpha_syn is not None
+        apply_min = min_v_mem is not None
+        checks = [((alpha_mem < 0) | (alpha_mem > 1)).any()]
+        if syn:
+            checks.append(((alpha_syn < 0) | (alpha_syn > 1)).any())
+        if apply_min:
+            checks.append((threshold <= min_v_mem).any())
+        flags = torch.stack(checks).tolist()
+        if flags[0] or (syn and flags[1]):
+            raise ValueError("'alpha' must be between 0 and 1.")
+        if apply_min and flags[-1]:
+            raise ValueError("`threshold` must be greater than `min_v_mem`.")
+
+        max_spikes = -1 if max_num_spikes_per_bin is None else int(max_num_spikes_per_bin)
+        need_grad = any(ctx.needs_input_grad)
+        res = _hip.layerLifForward(
+            inp, v_mem_init, i_syn_init, alpha_mem, alpha_syn, membrane_subtract, threshold, min_v_mem, apply_min,
+            max_spikes, decay_early, norm_input, wantCheckpoints=need_grad, stateShape=state_shape,
+        )
+        ctx.cfg = (syn, apply_min, max_spikes, bool(decay_early), bool(norm_input), kind, p0, p1)
+        ctx.set_materialize_grads(False)
+        if need_grad:
+            saved = [inp, res["ckpt_v"], v_mem_init, alpha_mem, membrane_subtract, threshold]
+            if syn:
+                saved += [res["ckpt_i"], i_syn_init, alpha_syn]
+            if apply_min:
+                saved.append(min_v_mem)
+            ctx.save_for_backward(*saved)
+        ctx.mark_non_differentiable(res["spike_sum"])
+        if syn:
+            return res["spikes"], res["v_last"], res["i_last"], res["spike_sum"]
+        return res["spikes"], res["v_last"], None, res["spike_sum"]
+
+    @staticmethod
+    def backward(ctx, grad_spikes, grad_v_last, grad_i_last, _grad_total):
+        syn, apply_min, max_spikes, decay_early, norm_input, kind, p0, p1 = ctx.cfg
+        saved = list(ctx.saved_tensors)
+        inp, ckpt_v, v_mem_init, alpha_mem, membrane_subtract, threshold = saved[:6]
+        rest = saved[6:]
+        ckpt_i = i_syn_init = alpha_syn = None
+        if syn:
+            ckpt_i, i_syn_init, alpha_syn = rest[:3]
+            rest = rest[3:]
+        min_v_mem = rest[0] if apply_min else None
+        if grad_spikes is None and grad_v_last is None and grad_i_last is None:
+            return (None,) * 13
+        if grad_spikes is None:
+            grad_spikes = torch.zeros_like(inp)
+        cont = lambda x: None if x is None else x.contiguous()
+        grad_input, g_am, g_as, g_v0, g_i0 = _hip.layerLifBackward(
+            cont(grad_spikes), cont(grad_v_last), cont(grad_i_last) if syn else None, inp, ckpt_v, ckpt_i,
+            v_mem_init, i_syn_init, alpha_mem, alpha_syn, membrane_subtract, threshold, min_v_mem, apply_min,
+            max_spikes, decay_early, norm_input, kind, p0, p1,
+        )
+        return (grad_input, g_am, g_as, g_v0, g_i0, None, None, None, None, None, None, None, None)

@@ -6,6 +6,7 @@ import torch
 from .._compat import (LIFBase, MaxSpike, MembraneSubtract, MultiSpike, SingleExponential, SingleSpike,
                        SqueezeMixin)
 from ..leaky import LeakyIntegrator
+from ..layer_function import SpikingLayerFunction
 from ..spike import IntegrateAndFire
 from ..synaptic import SynapticIntegrateAndFire, fusable
 
@@ -84,6 +85,10 @@ class LIF(LIFBase):
         # layers with synapses run synapse and membrane in one kernel when the surrogate gradient
         # is one the kernels can evaluate; set to False to force the two separate Functions
         self.fuse_synapse = True
+        # spiking layers that do not record states run one kernel per direction on the input's own
+        # (batch, time, neurons) layout (no transposing copies, no stored v_mem / i_syn); set to False
+        # to force the (rows, time) Functions
+        self.native_layout = True
 
     def _parse_activation_fn(self, spike_fn, reset_fn):
         """Translate the spike mechanism into a per-step spike cap (reference lif.py:130-150)."""
@@ -194,8 +199,54 @@ class LIF(LIFBase):
         v_mem_2d = v_mem_2d - membrane_subtract.unsqueeze(1) * output_2d
         return output_2d, v_mem_2d, i_syn_2d
 
+    def _use_native_layout(self, input_data: torch.Tensor) -> bool:
+        return (self.native_layout and self.spike_fn is not None and not self.record_states
+                and input_data.is_cuda and input_data.dtype == torch.float32 and input_data.ndim >= 2
+                and fusable(self.surrogate_grad_fn))
+
+    def _forward_native(self, input_data: torch.Tensor) -> torch.Tensor:
+        """Whole layer in one kernel on (batch, time, neurons); same values as the other path."""
+        batch_size, time_steps, *trailing_dim = input_data.shape
+        state_shape = (batch_size, *trailing_dim)
+        if not self.is_state_initialised() or not self.state_has_shape(state_shape):
+            self.init_state_with_shape(state_shape)
+        dev = self.v_mem.device
+        has_syn = self.tau_syn_calculated is not None
+        alpha_mem = expand_to_1d_contiguous(self.alpha_mem_calculated, state_shape, dev)
+        alpha_syn = expand_to_1d_contiguous(self.alpha_syn_calculated, state_shape, dev) if has_syn else None
+        spike_threshold = expand_to_1d_contiguous(self.spike_threshold, state_shape, dev)
+        min_v_mem = None if self.min_v_mem is None else expand_to_1d_contiguous(self.min_v_mem, state_shape, dev)
+        membrane_subtract = self.reset_fn.subtract_value
+        if membrane_subtract is None:
+            membrane_subtract = spike_threshold
+        else:
+            membrane_subtract = expand_to_1d_contiguous(membrane_subtract, state_shape, dev)
+        spikes, v_last, i_last, spike_total = SpikingLayerFunction.apply(
+            input_data.reshape(batch_size, time_steps, -1).contiguous(),
+            alpha_mem,
+            alpha_syn,
+            self.v_mem.flatten().contiguous(),
+            self.i_syn.flatten().contiguous() if has_syn else None,
+            spike_threshold,
+            membrane_subtract,
+            min_v_mem,
+            self.surrogate_grad_fn,
+            self.max_num_spikes_per_bin,
+            self.decay_early,
+            self.norm_input,
+            state_shape,
+        )
+        self.recordings = dict()
+        self.v_mem = v_last
+        if has_syn:
+            self.i_syn = i_last
+        self.firing_rate = (spike_total / max(spikes.numel(), 1)).float()
+        return spikes.reshape(input_data.shape)
+
     def forward(self, input_data: torch.Tensor) -> torch.Tensor:
         """Process ``input_data`` of shape (batch, time, ...); returns a tensor of the same shape."""
+        if self._use_native_layout(input_data):
+            return self._forward_native(input_data)
         input_2d, (batch_size, time_steps, *trailing_dim) = self._prepare_input(input_data)
         self.recordings = dict()
 

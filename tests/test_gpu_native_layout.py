@@ -1,0 +1,99 @@
+"""The layer-layout kernels (whole layer on (batch, time, neurons), recompute-in-backward) against
+the (rows, time) path of the same layer and against the CPU oracle."""
+from itertools import product
+
+import pytest
+import torch
+
+from _util import assert_close, gen
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def L():
+    assert torch.cuda.is_available()
+    import sinabs.exodus.layers as el
+    from sinabs.exodus import _hip
+    from sinabs.exodus._compat import activation as act
+    return el, act, _hip
+
+
+def pair(el, cls, **kw):
+    a = cls(**kw).cuda(); b = cls(**kw).cuda()
+    b.native_layout = False
+    return a, b
+
+
+SHAPES = [(1, 1, (1,)), (2, 7, (3,)), (3, 33, (5, 4)), (2, 100, (2, 7, 7)), (4, 64, (256,)), (2, 300, (260,)),
+          (3, 97, (1024,))]
+
+
+@pytest.mark.parametrize("batch,steps,trailing", SHAPES)
+@pytest.mark.parametrize("tau_syn,decay_early,norm_input", [(None, True, True), (None, True, False), (6.0, True, True),
+                                                             (6.0, False, False)])
+@pytest.mark.parametrize("spike,lo,surr", [("multi", None, "single"), ("max2", -0.7, "periodic"), ("single", -0.3, "heaviside")])
+def test_native_equals_rows_path(L, batch, steps, trailing, tau_syn, decay_early, norm_input, spike, lo, surr):
+    el, act, _ = L
+    m = 1
+    for d in trailing:
+        m *= d
+    fn = {"multi": act.MultiSpike, "single": act.SingleSpike, "max2": act.MaxSpike(2)}[spike]
+    sg = {"single": act.SingleExponential(), "periodic": act.PeriodicExponential(0.4, 0.8), "heaviside": act.Heaviside(0.7)}[surr]
+    g = gen(batch * 1000 + steps + m)
+    kw = dict(tau_mem=10.0 + 20.0 * torch.rand(trailing, generator=g), tau_syn=tau_syn, spike_fn=fn, min_v_mem=lo,
+              surrogate_grad_fn=sg, train_alphas=True, norm_input=norm_input, decay_early=decay_early)
+    native, rows = pair(el, el.LIF, **kw)
+    scale = (8.0 if norm_input else 0.8) * (1.0 if tau_syn is None else 0.4)
+    data = (torch.rand((2, batch, steps) + trailing, generator=g) * scale * 2 - 0.3 * scale).cuda()
+    xa = data.clone().requires_grad_(True); xb = data.clone().requires_grad_(True)
+    for k in range(2):                                   # second call starts from the first call's states
+        a = native(xa[k]); b = rows(xb[k])
+        assert a.shape == b.shape == xa[k].shape
+        assert torch.equal(a, b)
+        assert torch.equal(native.v_mem, rows.v_mem)
+        if tau_syn is not None:
+            assert torch.equal(native.i_syn, rows.i_syn)
+        assert torch.allclose(native.firing_rate, rows.firing_rate, rtol=1e-6, atol=0)
+    w = torch.rand(a.shape, generator=g).cuda()
+    (a * w).sum().backward(); (b * w).sum().backward()
+    assert_close(xa.grad, xb.grad, "grad input")
+    for (k, p), (_, q) in zip(native.named_parameters(), rows.named_parameters()):
+        if q.grad is not None:
+            assert_close(p.grad, q.grad, f"grad {k}", rtol=1e-4, atol=1e-5 * max(1.0, (batch * steps) ** 0.5))
+
+
+def test_native_iaf_squeeze_and_unknown_surrogate_fallback(L):
+    el, act, _ = L
+    x = torch.rand(6 * 50, 2, 5, 5, generator=gen(3)).cuda()
+    native, rows = pair(el, el.IAFSqueeze, batch_size=6, min_v_mem=-1.0)
+    assert torch.equal(native(x), rows(x)) and native(x).is_contiguous()
+    custom = el.IAF(surrogate_grad_fn=lambda v, th: 1.0 / (1.0 + (v - th) ** 2)).cuda()
+    assert not custom._use_native_layout(x.reshape(6, 50, 2, 5, 5))
+    rec = el.IAF(record_states=True).cuda()
+    assert not rec._use_native_layout(x.reshape(6, 50, 2, 5, 5))
+    out = custom(x.reshape(6, 50, 2, 5, 5)); assert out.shape == (6, 50, 2, 5, 5)
+
+
+def test_native_forward_against_cpu_oracle(L):
+    """Bit-exact spikes and final states against the C restatement of the reference kernel."""
+    el, act, hip = L
+    from oracle import exodus_ref as ref
+    from oracle import sinabs_cpu as sc
+    b, t, m = 3, 130, 40
+    g = gen(11)
+    x = torch.randn(b, t, m, generator=g) * 0.6 + 0.2
+    alpha = torch.rand(b * m, generator=g); v0 = torch.randn(b * m, generator=g) * 0.3
+    th = 0.5 + torch.rand(b * m, generator=g); c = 0.3 + 0.5 * torch.rand(b * m, generator=g); lo = -0.5 * torch.ones(b * m)
+    ws, wv = ref.lif_forward(sc.bt_to_rows(x), v0, alpha, c, th, lo, True, 2)
+    D = lambda z: z.cuda()
+    res = hip.layerLifForward(D(x), D(v0), None, D(alpha), None, D(c), D(th), D(lo), True, 2, True, False,
+                              wantRecords=True)
+    assert torch.equal(res["spikes"].cpu(), sc.rows_to_bt(ws, b))
+    vpost = wv - c[:, None] * ws
+    assert torch.equal(res["v_rec"].cpu(), sc.rows_to_bt(vpost, b))
+    assert torch.equal(res["v_last"].cpu(), vpost[:, -1])
+    assert float(res["spike_sum"]) == float(ws.sum())
+    ck = hip.checkpointInterval()
+    want_ck = torch.stack([v0] + [vpost[:, k * ck - 1] for k in range(1, (t + ck - 1) // ck)], 1)   # (rows, n_ck)
+    assert torch.equal(res["ckpt_v"].cpu(), sc.rows_to_bt(want_ck, b))
