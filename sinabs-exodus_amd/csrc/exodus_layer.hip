@@ -21,9 +21,18 @@
 
 namespace {
 
-constexpr int CKPT = 32;      // steps between checkpoints = length of a backward chunk
-constexpr int FWD_UNROLL = 8; // forward steps per software-pipeline stage (divides CKPT)
-constexpr int BLOCK = 256;
+#ifndef EXODUS_LAYER_FWD_UNROLL
+#define EXODUS_LAYER_FWD_UNROLL 8
+#endif
+#ifndef EXODUS_LAYER_BLOCK
+#define EXODUS_LAYER_BLOCK 256
+#endif
+#ifndef EXODUS_LAYER_BWD_WAVES
+#define EXODUS_LAYER_BWD_WAVES 3      // resident waves per SIMD the backward kernel is compiled for
+#endif
+constexpr int CKPT = 32;                             // steps between checkpoints = length of a backward chunk
+constexpr int FWD_UNROLL = EXODUS_LAYER_FWD_UNROLL;  // forward steps per software-pipeline stage (divides CKPT)
+constexpr int BLOCK = EXODUS_LAYER_BLOCK;
 
 struct LayerConsts {
     const float *v_init, *i_init, *alpha_mem, *alpha_syn, *c, *theta, *theta_low;
@@ -193,7 +202,8 @@ __global__ void __launch_bounds__(BLOCK) layer_lif_forward(
 // gv on it reaches v_{T-1} directly and the spike count with weight -c, a gradient on the final
 // synaptic current adds to mu_{T-1}.
 template <bool SYN, int KIND>
-__global__ void __launch_bounds__(BLOCK) layer_lif_backward(
+__global__ void __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(EXODUS_LAYER_BWD_WAVES, EXODUS_LAYER_BWD_WAVES)))
+layer_lif_backward(
     float *__restrict__ grad_x, float *__restrict__ alpha_mem_grad, float *__restrict__ alpha_syn_grad,
     float *__restrict__ v_init_grad, float *__restrict__ i_init_grad, const float *__restrict__ grad_spikes,
     const float *__restrict__ grad_v_last, const float *__restrict__ grad_i_last, const float *__restrict__ x,
