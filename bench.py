@@ -78,7 +78,21 @@ def build_layer_workload(key, torch, hip, act, dev):
     elif key == "c1":
         cfg = dict(a_mem=ones, a_syn=None, lo=None, cap=-1, norm=False)
     else:
-        raise SystemExit("the layer-layout path covers the spiking workloads (c5, c2, c1)")
+        # C3: ExpLeak with trainable per-channel alpha; forward 8 B (x in, out out), backward 12 B
+        # (grad_out and saved out in, grad_x out)
+        tau = 5.0 + 45.0 * torch.rand(M, generator=g, device=dev)
+        a_mem = rows(torch.exp(-1.0 / tau))
+        holder = {}
+
+        def fwd():
+            holder["out"] = hip.layerLeakyForward(x, zeros, a_mem, False, False)[0]
+
+        def bwd():
+            r = hip.layerLeakyBackward(go, None, holder["out"], x, zeros, a_mem, False, False, True)
+            return r[1].view(B, M).sum(0)
+
+        return dict(fwd=fwd, bwd=bwd, N=N, T=T, fwd_name="exodus_layer_leaky_forward",
+                    bwd_name="exodus_layer_leaky_backward", bytes=(8, 12))
     syn = cfg["a_syn"] is not None
     holder = {}
 
@@ -238,7 +252,7 @@ def main():
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    if args.path == "layer" and args.workload != "c3":
+    if args.path == "layer":
         wl = build_layer_workload(args.workload, torch, hip, act, dev)
     else:
         args.path = "rows"

@@ -201,6 +201,23 @@ int exodus_layer_lif_backward(float *grad_input, float *alpha_mem_grad, float *a
                               int surrogate_kind, float surr_p0, float surr_p1, int64_t batch, int64_t t,
                               int64_t neurons, void *stream);
 
+/* Forward of the non-spiking leaky-integrator layer (ExpLeak) on (batch,t,neurons): per neuron
+ *   xin = norm_input ? (1 - alpha) * input : input;  xin = decay_early ? xin * alpha : xin;
+ *   out_t = alpha * out_{t-1} + xin_t,  out_{-1} = vmem_initial
+ * (reference sinabs/exodus/layers/lif.py:206-223).  v_last (batch*neurons) receives out[:, -1]. */
+int exodus_layer_leaky_forward(float *out, float *v_last, const float *input, const float *vmem_initial,
+                               const float *alpha, int decay_early, int norm_input, int64_t batch,
+                               int64_t t, int64_t neurons, void *stream);
+
+/* Backward of the above: grad_input (batch,t,neurons); optional per-neuron alpha_grad (needs `out`
+ * and `vmem_initial`, and `input` when one of the input scalings is on) and vmem_init_grad;
+ * grad_v_last (batch*neurons, optional) is a gradient arriving at the final state. */
+int exodus_layer_leaky_backward(float *grad_input, float *alpha_grad, float *vmem_init_grad,
+                                const float *grad_out, const float *grad_v_last, const float *out,
+                                const float *input, const float *vmem_initial, const float *alpha,
+                                int decay_early, int norm_input, int64_t batch, int64_t t,
+                                int64_t neurons, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -315,6 +315,149 @@ layer_lif_backward(
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// non-spiking leaky integrator layer (ExpLeak) on the layer layout
+// ---------------------------------------------------------------------------------------------
+struct LeakyConsts {
+    const float *v_init, *alpha;
+    int decay_early, norm_input;
+};
+
+constexpr int LEAKY_UNROLL = 8;
+
+// xin = norm_input ? (1 - alpha) * x : x;  xin = decay_early ? xin * alpha : xin;  v = v * alpha + xin
+template <int NPL>
+__global__ void __launch_bounds__(BLOCK) layer_leaky_forward(float *__restrict__ out, float *__restrict__ v_last,
+                                                             const float *__restrict__ x, const LeakyConsts p,
+                                                             const int64_t blocks_per_batch, const int64_t T,
+                                                             const int64_t M)
+{
+    typedef typename Vec<NPL>::type V;
+    const int64_t b = blockIdx.x / blocks_per_batch;
+    const int64_t m0 = static_cast<int64_t>(blockIdx.x - b * blocks_per_batch) * (BLOCK * NPL);
+    const unsigned lane_off = threadIdx.x * NPL;
+    if (m0 + lane_off >= M) return;
+    const int64_t first = b * M + m0 + lane_off;
+    const float *xp = x + (b * T) * M + m0;
+    float *op = out + (b * T) * M + m0;
+    float a[NPL], k[NPL], v[NPL];
+#pragma unroll
+    for (int e = 0; e < NPL; ++e) {
+        a[e] = p.alpha[first + e];
+        k[e] = __fsub_rn(1.0f, a[e]);
+        v[e] = p.v_init[first + e];
+    }
+    V cur[LEAKY_UNROLL], nxt[LEAKY_UNROLL];
+    auto fetch = [&](V(&dst)[LEAKY_UNROLL], int64_t t0) {
+#pragma unroll
+        for (int u = 0; u < LEAKY_UNROLL; ++u)
+            if (t0 + u < T) dst[u] = ld_stream(reinterpret_cast<const V *>(xp + (t0 + u) * M + lane_off));
+    };
+    fetch(cur, 0);
+    for (int64_t t0 = 0; t0 < T; t0 += LEAKY_UNROLL) {
+        if (t0 + LEAKY_UNROLL < T) fetch(nxt, t0 + LEAKY_UNROLL);
+#pragma unroll
+        for (int u = 0; u < LEAKY_UNROLL; ++u) {
+            if (t0 + u < T) {
+                V o;
+#pragma unroll
+                for (int e = 0; e < NPL; ++e) {
+                    float xin = lane_get<NPL>(cur[u], e);
+                    if (p.norm_input) xin = __fmul_rn(k[e], xin);
+                    if (p.decay_early) xin = __fmul_rn(xin, a[e]);
+                    v[e] = __fadd_rn(__fmul_rn(v[e], a[e]), xin);
+                    lane_put<NPL>(o, e, v[e]);
+                }
+                st_stream(o, reinterpret_cast<V *>(op + (t0 + u) * M + lane_off));
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < LEAKY_UNROLL; ++u) cur[u] = nxt[u];
+    }
+#pragma unroll
+    for (int e = 0; e < NPL; ++e) v_last[first + e] = v[e];
+}
+
+// g_t = alpha g_{t+1} + grad_out_t (+ grad_v_last at the last step)
+// grad_x_t = ((decay_early ? g_t alpha : g_t) * (norm_input ? 1 - alpha : 1))
+// grad_alpha = sum_t g_t out_{t-1}  +  (decay_early ? sum_t g_t (k x_t) : 0)  -  (norm_input ? sum_t (g_t [alpha]) x_t : 0)
+// `x` is only read when WITH_X (alpha gradient wanted and one of the input scalings is on).
+template <int NPL, bool ALPHA, bool WITH_X>
+__global__ void __launch_bounds__(BLOCK) layer_leaky_backward(
+    float *__restrict__ grad_x, float *__restrict__ alpha_grad, float *__restrict__ v_init_grad,
+    const float *__restrict__ grad_out, const float *__restrict__ grad_v_last, const float *__restrict__ out,
+    const float *__restrict__ x, const LeakyConsts p, const int64_t blocks_per_batch, const int64_t T, const int64_t M)
+{
+    typedef typename Vec<NPL>::type V;
+    const int64_t b = blockIdx.x / blocks_per_batch;
+    const int64_t m0 = static_cast<int64_t>(blockIdx.x - b * blocks_per_batch) * (BLOCK * NPL);
+    const unsigned lane_off = threadIdx.x * NPL;
+    if (m0 + lane_off >= M) return;
+    const int64_t first = b * M + m0 + lane_off;
+    const float *gp = grad_out + (b * T) * M + m0;
+    const float *outp = ALPHA ? out + (b * T) * M + m0 : nullptr;
+    const float *xp = WITH_X ? x + (b * T) * M + m0 : nullptr;
+    float *op = grad_x + (b * T) * M + m0;
+    float a[NPL], k[NPL], g[NPL];
+    TileSum acc[NPL];
+#pragma unroll
+    for (int e = 0; e < NPL; ++e) {
+        a[e] = p.alpha[first + e];
+        k[e] = __fsub_rn(1.0f, a[e]);
+        g[e] = grad_v_last ? grad_v_last[first + e] : 0.f;     // joins grad_out at the last step
+        acc[e].clear();
+    }
+    // step t needs out_{t-1}: walk t = T-1 .. 0 in groups, newest first
+    for (int64_t t_hi = T; t_hi > 0; t_hi -= LEAKY_UNROLL) {
+        V gv[LEAKY_UNROLL], ov[LEAKY_UNROLL], xv[LEAKY_UNROLL];
+#pragma unroll
+        for (int u = 0; u < LEAKY_UNROLL; ++u) {
+            const int64_t t = t_hi - 1 - u;
+            if (t >= 0) {
+                gv[u] = ld_stream(reinterpret_cast<const V *>(gp + t * M + lane_off));
+                if (WITH_X) xv[u] = ld_stream(reinterpret_cast<const V *>(xp + t * M + lane_off));
+                if (ALPHA && t >= 1) ov[u] = ld_stream(reinterpret_cast<const V *>(outp + (t - 1) * M + lane_off));
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < LEAKY_UNROLL; ++u) {
+            const int64_t t = t_hi - 1 - u;
+            if (t >= 0) {
+                V o;
+#pragma unroll
+                for (int e = 0; e < NPL; ++e) {
+                    // first processed step (t = T-1): g holds grad_v_last and there is no later step to decay
+                    const float carried = (t == T - 1) ? g[e] : __fmul_rn(g[e], a[e]);
+                    g[e] = __fadd_rn(carried, lane_get<NPL>(gv[u], e));
+                    float gx = g[e];
+                    if (p.decay_early) gx = __fmul_rn(gx, a[e]);
+                    if (ALPHA) {
+                        const float prev = t >= 1 ? lane_get<NPL>(ov[u], e) : p.v_init[first + e];
+                        acc[e].add(g[e], prev);
+                        if (WITH_X) {
+                            const float xe = lane_get<NPL>(xv[u], e);
+                            if (p.decay_early) acc[e].add(g[e], p.norm_input ? __fmul_rn(k[e], xe) : xe);
+                            if (p.norm_input) acc[e].sub(gx, xe);
+                        }
+                    }
+                    if (p.norm_input) gx = __fmul_rn(gx, k[e]);
+                    lane_put<NPL>(o, e, gx);
+                }
+                st_stream(o, reinterpret_cast<V *>(op + t * M + lane_off));
+            }
+        }
+        if (ALPHA) {
+#pragma unroll
+            for (int e = 0; e < NPL; ++e) acc[e].fold();
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < NPL; ++e) {
+        if (v_init_grad) v_init_grad[first + e] = __fmul_rn(a[e], g[e]);
+        if (ALPHA) alpha_grad[first + e] = static_cast<float>(acc[e].total);
+    }
+}
+
 inline bool bad3(int64_t b, int64_t t, int64_t m)
 {
     if (b < 0 || t < 0 || m < 0) return true;
@@ -434,6 +577,68 @@ EXODUS_API int exodus_layer_lif_backward(float *grad_input, float *alpha_mem_gra
         default: return hipErrorInvalidValue;
     }
 #undef EXODUS_BWD
+}
+
+EXODUS_API int exodus_layer_leaky_forward(float *out, float *v_last, const float *input, const float *vmem_initial,
+                                          const float *alpha, int decay_early, int norm_input, int64_t batch,
+                                          int64_t t, int64_t neurons, void *stream)
+{
+    if (bad3(batch, t, neurons)) return hipErrorInvalidValue;
+    if (batch == 0 || t == 0 || neurons == 0) return hipSuccess;
+    if (!out || !v_last || !input || !vmem_initial || !alpha) return hipErrorInvalidValue;
+    LeakyConsts p;
+    p.v_init = vmem_initial;
+    p.alpha = alpha;
+    p.decay_early = decay_early ? 1 : 0;
+    p.norm_input = norm_input ? 1 : 0;
+    const bool vec = (neurons % 4) == 0 && aligned16(input) && aligned16(out);
+    const int npl = vec ? 4 : 1;
+    const int64_t blocks_per_batch = (neurons + BLOCK * npl - 1) / (BLOCK * npl);
+    if (blocks_per_batch > 0x7fffffffLL / batch) return hipErrorInvalidValue;
+    const dim3 grid(static_cast<unsigned>(blocks_per_batch * batch)), block(BLOCK);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (vec)
+        hipLaunchKernelGGL((layer_leaky_forward<4>), grid, block, 0, s, out, v_last, input, p, blocks_per_batch, t, neurons);
+    else
+        hipLaunchKernelGGL((layer_leaky_forward<1>), grid, block, 0, s, out, v_last, input, p, blocks_per_batch, t, neurons);
+    return static_cast<int>(hipGetLastError());
+}
+
+EXODUS_API int exodus_layer_leaky_backward(float *grad_input, float *alpha_grad, float *vmem_init_grad,
+                                           const float *grad_out, const float *grad_v_last, const float *out,
+                                           const float *input, const float *vmem_initial, const float *alpha,
+                                           int decay_early, int norm_input, int64_t batch, int64_t t,
+                                           int64_t neurons, void *stream)
+{
+    if (bad3(batch, t, neurons)) return hipErrorInvalidValue;
+    if (batch == 0 || t == 0 || neurons == 0) return hipSuccess;
+    if (!grad_input || !grad_out || !alpha) return hipErrorInvalidValue;
+    const bool want_alpha = alpha_grad != nullptr;
+    const bool with_x = want_alpha && (decay_early || norm_input);
+    if (want_alpha && (!out || !vmem_initial)) return hipErrorInvalidValue;
+    if (with_x && !input) return hipErrorInvalidValue;
+    LeakyConsts p;
+    p.v_init = vmem_initial;
+    p.alpha = alpha;
+    p.decay_early = decay_early ? 1 : 0;
+    p.norm_input = norm_input ? 1 : 0;
+    const bool vec = (neurons % 4) == 0 && aligned16(grad_input) && aligned16(grad_out) && aligned16(out) &&
+                     aligned16(input);
+    const int npl = vec ? 4 : 1;
+    const int64_t blocks_per_batch = (neurons + BLOCK * npl - 1) / (BLOCK * npl);
+    if (blocks_per_batch > 0x7fffffffLL / batch) return hipErrorInvalidValue;
+    const dim3 grid(static_cast<unsigned>(blocks_per_batch * batch)), block(BLOCK);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+#define EXODUS_LK(NPL, AL, WX)                                                                                 \
+    hipLaunchKernelGGL((layer_leaky_backward<NPL, AL, WX>), grid, block, 0, s, grad_input, alpha_grad,        \
+                       vmem_init_grad, grad_out, grad_v_last, out, input, p, blocks_per_batch, t, neurons)
+    if (vec) {
+        if (with_x) EXODUS_LK(4, true, true); else if (want_alpha) EXODUS_LK(4, true, false); else EXODUS_LK(4, false, false);
+    } else {
+        if (with_x) EXODUS_LK(1, true, true); else if (want_alpha) EXODUS_LK(1, true, false); else EXODUS_LK(1, false, false);
+    }
+#undef EXODUS_LK
+    return static_cast<int>(hipGetLastError());
 }
 
 }  // extern "C"

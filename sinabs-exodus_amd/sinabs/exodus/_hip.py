@@ -44,6 +44,8 @@ _SIGNATURES = {
     "exodus_layer_checkpoint_interval": ([], _int),
     "exodus_layer_lif_forward": ([_p] * 16 + [_int, _int, _int, _int, _i64, _i64, _i64, _p], _int),
     "exodus_layer_lif_backward": ([_p] * 18 + [_int, _int, _int, _int, _int, _f, _f, _i64, _i64, _i64, _p], _int),
+    "exodus_layer_leaky_forward": ([_p] * 5 + [_int, _int, _i64, _i64, _i64, _p], _int),
+    "exodus_layer_leaky_backward": ([_p] * 9 + [_int, _int, _i64, _i64, _i64, _p], _int),
 }
 
 
@@ -466,3 +468,55 @@ def layerLifBackward(gradSpikes, gradVLast, gradILast, input, ckptV, ckptI, vmem
             int(bool(decayEarly)), int(bool(normInput)), int(surrogateKind), float(surrP0), float(surrP1), b, t, m,
             _stream(input)), "exodus_layer_lif_backward")
     return gradInput, am_g, as_g, v0_g, i0_g
+
+
+def layerLeakyForward(input, vmemInitial, alpha, decayEarly: bool, normInput: bool,
+                      stateShape: Optional[tuple] = None):
+    """Leaky-integrator layer on (batch, time, neurons): returns (out, v_last)."""
+    _btm(input, "input")
+    b, t, m = input.shape
+    n = b * m
+    _rows(_dev(vmemInitial, "vmemInitial", input), "vmemInitial", n)
+    _rows(_dev(alpha, "alpha", input), "alpha", n)
+    state_shape = (n,) if stateShape is None else tuple(stateShape)
+    if math.prod(state_shape) != n:
+        raise RuntimeError(f"stateShape {state_shape} does not hold {n} neurons")
+    out = torch.empty_like(input)
+    v_last = torch.empty(state_shape, dtype=torch.float32, device=input.device)
+    if t == 0:
+        v_last.copy_(vmemInitial.reshape(state_shape))
+    with torch.cuda.device(input.device):
+        _check(lib.exodus_layer_leaky_forward(_ptr(out), _ptr(v_last), _ptr(input), _ptr(vmemInitial), _ptr(alpha),
+                                              int(bool(decayEarly)), int(bool(normInput)), b, t, m, _stream(input)),
+               "exodus_layer_leaky_forward")
+    return out, v_last
+
+
+def layerLeakyBackward(gradOut, gradVLast, out, input, vmemInitial, alpha, decayEarly: bool, normInput: bool,
+                       needAlphaGrad: bool):
+    """Returns (gradInput, alphaGrad | None, vInitGrad)."""
+    _btm(gradOut, "gradOut")
+    b, t, m = gradOut.shape
+    n = b * m
+    _rows(_dev(alpha, "alpha", gradOut), "alpha", n)
+    if gradVLast is not None and _dev(gradVLast, "gradVLast", gradOut).numel() != n:
+        raise RuntimeError(f"gradVLast must hold {n} values")
+    need_x = needAlphaGrad and (decayEarly or normInput)
+    if needAlphaGrad:
+        if _btm(out, "out", gradOut).shape != gradOut.shape:
+            raise RuntimeError("out must have the shape of gradOut")
+        _rows(_dev(vmemInitial, "vmemInitial", gradOut), "vmemInitial", n)
+    if need_x and _btm(input, "input", gradOut).shape != gradOut.shape:
+        raise RuntimeError("input must have the shape of gradOut")
+    grad_input = torch.empty_like(gradOut)
+    alpha_grad = torch.zeros(n, dtype=torch.float32, device=gradOut.device) if needAlphaGrad else None
+    v_init_grad = torch.zeros(n, dtype=torch.float32, device=gradOut.device)
+    if t == 0 and gradVLast is not None:
+        v_init_grad.copy_(gradVLast.reshape(-1))
+    with torch.cuda.device(gradOut.device):
+        _check(lib.exodus_layer_leaky_backward(
+            _ptr(grad_input), _ptr(alpha_grad), _ptr(v_init_grad), _ptr(gradOut), _ptr(gradVLast),
+            _ptr(out) if needAlphaGrad else None, _ptr(input) if need_x else None,
+            _ptr(vmemInitial) if needAlphaGrad else None, _ptr(alpha), int(bool(decayEarly)), int(bool(normInput)),
+            b, t, m, _stream(gradOut)), "exodus_layer_leaky_backward")
+    return grad_input, alpha_grad, v_init_grad

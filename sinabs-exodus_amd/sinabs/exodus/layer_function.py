@@ -101,3 +101,45 @@ class SpikingLayerFunction(torch.autograd.Function):
             max_spikes, decay_early, norm_input, kind, p0, p1,
         )
         return (grad_input, g_am, g_as, g_v0, g_i0, None, None, None, None, None, None, None, None)
+
+
+class LeakyLayerFunction(torch.autograd.Function):
+    """The non-spiking leaky-integrator layer (ExpLeak) on (batch, time, neurons): input scalings and
+    the integrator in one kernel per direction (reference sinabs/exodus/layers/lif.py:206-223)."""
+
+    @staticmethod
+    def forward(ctx, inp, alpha, v_mem_init, decay_early: bool, norm_input: bool, state_shape=None):
+        """Returns ``(out (batch,time,neurons), v_mem_last)``."""
+        if inp.ndim != 3:
+            raise ValueError("'inp' must be 3D, (batch, time, neurons)")
+        if not inp.is_contiguous():
+            raise ValueError("'inp' has to be contiguous.")
+        out, v_last = _hip.layerLeakyForward(inp, v_mem_init, alpha, decay_early, norm_input, stateShape=state_shape)
+        ctx.cfg = (bool(decay_early), bool(norm_input), alpha.requires_grad)
+        ctx.set_materialize_grads(False)
+        if alpha.requires_grad:
+            need_x = decay_early or norm_input
+            ctx.save_for_backward(alpha, v_mem_init, out, inp if need_x else None)
+        else:
+            ctx.save_for_backward(alpha)
+        return out, v_last
+
+    @staticmethod
+    def backward(ctx, grad_out, grad_v_last):
+        decay_early, norm_input, need_alpha = ctx.cfg
+        if need_alpha:
+            alpha, v_mem_init, out, inp = ctx.saved_tensors
+        else:
+            (alpha,) = ctx.saved_tensors
+            v_mem_init = out = inp = None
+        if grad_out is None and grad_v_last is None:
+            return (None,) * 6
+        if grad_out is None:
+            shape = out.shape if out is not None else None
+            if shape is None:
+                raise RuntimeError("gradient of the final state alone needs the output's shape")
+            grad_out = torch.zeros(shape, dtype=torch.float32, device=alpha.device)
+        cont = lambda x: None if x is None else x.contiguous()
+        grad_input, grad_alpha, grad_init = _hip.layerLeakyBackward(
+            cont(grad_out), cont(grad_v_last), out, inp, v_mem_init, alpha, decay_early, norm_input, need_alpha)
+        return grad_input, grad_alpha, grad_init, None, None, None

@@ -6,7 +6,7 @@ import torch
 from .._compat import (LIFBase, MaxSpike, MembraneSubtract, MultiSpike, SingleExponential, SingleSpike,
                        SqueezeMixin)
 from ..leaky import LeakyIntegrator
-from ..layer_function import SpikingLayerFunction
+from ..layer_function import LeakyLayerFunction, SpikingLayerFunction
 from ..spike import IntegrateAndFire
 from ..synaptic import SynapticIntegrateAndFire, fusable
 
@@ -200,9 +200,32 @@ class LIF(LIFBase):
         return output_2d, v_mem_2d, i_syn_2d
 
     def _use_native_layout(self, input_data: torch.Tensor) -> bool:
-        return (self.native_layout and self.spike_fn is not None and not self.record_states
-                and input_data.is_cuda and input_data.dtype == torch.float32 and input_data.ndim >= 2
-                and fusable(self.surrogate_grad_fn))
+        if not (self.native_layout and input_data.is_cuda and input_data.dtype == torch.float32
+                and input_data.ndim >= 2):
+            return False
+        if self.spike_fn is None:                      # leaky integrator: the output is the state record
+            return self.tau_syn_calculated is None
+        return not self.record_states and fusable(self.surrogate_grad_fn)
+
+    def _forward_native_leaky(self, input_data: torch.Tensor) -> torch.Tensor:
+        batch_size, time_steps, *trailing_dim = input_data.shape
+        state_shape = (batch_size, *trailing_dim)
+        if not self.is_state_initialised() or not self.state_has_shape(state_shape):
+            self.init_state_with_shape(state_shape)
+        alpha_mem = expand_to_1d_contiguous(self.alpha_mem_calculated, state_shape, self.v_mem.device)
+        out, v_last = LeakyLayerFunction.apply(
+            input_data.reshape(batch_size, time_steps, -1).contiguous(),
+            alpha_mem,
+            self.v_mem.flatten().contiguous(),
+            self.decay_early,
+            self.norm_input,
+            state_shape,
+        )
+        out = out.reshape(input_data.shape)
+        self.recordings = {"v_mem": out} if self.record_states else dict()
+        self.v_mem = v_last
+        self.firing_rate = out.sum() / max(out.numel(), 1)
+        return out
 
     def _forward_native(self, input_data: torch.Tensor) -> torch.Tensor:
         """Whole layer in one kernel on (batch, time, neurons); same values as the other path."""
@@ -246,6 +269,8 @@ class LIF(LIFBase):
     def forward(self, input_data: torch.Tensor) -> torch.Tensor:
         """Process ``input_data`` of shape (batch, time, ...); returns a tensor of the same shape."""
         if self._use_native_layout(input_data):
+            if self.spike_fn is None:
+                return self._forward_native_leaky(input_data)
             return self._forward_native(input_data)
         input_2d, (batch_size, time_steps, *trailing_dim) = self._prepare_input(input_data)
         self.recordings = dict()

@@ -97,3 +97,32 @@ def test_native_forward_against_cpu_oracle(L):
     ck = hip.checkpointInterval()
     want_ck = torch.stack([v0] + [vpost[:, k * ck - 1] for k in range(1, (t + ck - 1) // ck)], 1)   # (rows, n_ck)
     assert torch.equal(res["ckpt_v"].cpu(), sc.rows_to_bt(want_ck, b))
+
+
+@pytest.mark.parametrize("batch,steps,trailing", [(1, 1, (1,)), (2, 7, (3,)), (3, 33, (5, 4)), (4, 64, (256,)), (2, 300, (260,))])
+@pytest.mark.parametrize("decay_early,norm_input,train_alphas", list(product((True, False), (True, False), (True, False))))
+def test_native_expleak_equals_rows_path(L, batch, steps, trailing, decay_early, norm_input, train_alphas):
+    el, _, _ = L
+    g = gen(batch * 100 + steps)
+    kw = dict(tau_mem=5.0 + 40.0 * torch.rand(trailing, generator=g), train_alphas=train_alphas, norm_input=norm_input,
+              decay_early=decay_early)
+    native, rows = pair(el, el.ExpLeak, **kw)
+    data = torch.randn((2, batch, steps) + trailing, generator=g).cuda()
+    xa = data.clone().requires_grad_(True); xb = data.clone().requires_grad_(True)
+    for k in range(2):
+        a = native(xa[k]); b = rows(xb[k])
+        assert torch.equal(a, b) and torch.equal(native.v_mem, rows.v_mem)
+    w = torch.randn(a.shape, generator=g).cuda()
+    (a * w).sum().backward(); (b * w).sum().backward()
+    assert_close(xa.grad, xb.grad, "grad input")
+    for (k, p), (_, q) in zip(native.named_parameters(), rows.named_parameters()):
+        if q.grad is not None:
+            assert_close(p.grad, q.grad, f"grad {k}", rtol=1e-4, atol=1e-5 * max(1.0, (batch * steps) ** 0.5))
+
+
+def test_native_expleak_records_and_squeeze(L):
+    el, _, _ = L
+    x = torch.rand(5 * 40, 3, 4, 4, generator=gen(5)).cuda()
+    native, rows = pair(el, el.ExpLeakSqueeze, tau_mem=12.0, batch_size=5, record_states=True)
+    a = native(x); b = rows(x)
+    assert torch.equal(a, b) and torch.equal(native.recordings["v_mem"], rows.recordings["v_mem"])
