@@ -17,6 +17,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <initializer_list>
+
 #include "exodus_common.hpp"
 
 namespace {
@@ -41,14 +43,18 @@ struct LayerConsts {
 };
 
 template <int NPL> struct Vec;
+typedef float f32x2 __attribute__((ext_vector_type(2)));
 template <> struct Vec<1> { typedef float type; };
+template <> struct Vec<2> { typedef f32x2 type; };
 template <> struct Vec<4> { typedef f32x4 type; };
 
 template <int NPL> __device__ __forceinline__ float lane_get(const typename Vec<NPL>::type &v, int e);
 template <> __device__ __forceinline__ float lane_get<1>(const float &v, int) { return v; }
+template <> __device__ __forceinline__ float lane_get<2>(const f32x2 &v, int e) { return v[e]; }
 template <> __device__ __forceinline__ float lane_get<4>(const f32x4 &v, int e) { return v[e]; }
 template <int NPL> __device__ __forceinline__ void lane_put(typename Vec<NPL>::type &v, int e, float x);
 template <> __device__ __forceinline__ void lane_put<1>(float &v, int, float x) { v = x; }
+template <> __device__ __forceinline__ void lane_put<2>(f32x2 &v, int e, float x) { v[e] = x; }
 template <> __device__ __forceinline__ void lane_put<4>(f32x4 &v, int e, float x) { v[e] = x; }
 
 // per-neuron constants and running state of the forward recurrence
@@ -458,6 +464,30 @@ __global__ void __launch_bounds__(BLOCK) layer_leaky_backward(
     }
 }
 
+// Neurons per lane of the forward kernels.  Wider lanes mean wider memory accesses but fewer
+// lanes: stay at the widest width that still gives every SIMD about four waves, so that small
+// layers are not starved of parallelism.  `align` is the common alignment (bytes) of all
+// (batch, time, neurons) pointers involved.
+inline int pick_neurons_per_lane(int64_t batch, int64_t neurons, unsigned align)
+{
+    int cus = 0, dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+        cus = 256;
+    const int64_t wanted_lanes = static_cast<int64_t>(cus) * 16 * WAVE;
+    const int64_t n = batch * neurons;
+    if ((neurons % 4) == 0 && (align % 16) == 0 && n / 4 >= wanted_lanes) return 4;
+    if ((neurons % 2) == 0 && (align % 8) == 0 && n / 2 >= wanted_lanes) return 2;
+    return 1;
+}
+
+inline unsigned common_alignment(std::initializer_list<const void *> ptrs)
+{
+    uintptr_t bits = 0;
+    for (const void *q : ptrs) bits |= reinterpret_cast<uintptr_t>(q);   // null pointers do not constrain
+    return static_cast<unsigned>(bits & 15u) == 0 ? 16u : ((bits & 7u) == 0 ? 8u : 4u);
+}
+
 inline bool bad3(int64_t b, int64_t t, int64_t m)
 {
     if (b < 0 || t < 0 || m < 0) return true;
@@ -514,10 +544,8 @@ EXODUS_API int exodus_layer_lif_forward(float *out_spikes, float *out_vmem_rec, 
     p.decay_early = decay_early ? 1 : 0;
     p.norm_input = norm_input ? 1 : 0;
     p.cap = static_cast<unsigned>(max_num_spikes);
-    // four neurons per lane need 16-byte aligned rows of every (batch, time, neurons) tensor
-    bool vec = (neurons % 4) == 0 && aligned16(input) && aligned16(out_spikes) && aligned16(out_vmem_rec) &&
-               aligned16(out_isyn_rec) && aligned16(ckpt_v) && aligned16(ckpt_i);
-    const int npl = vec ? 4 : 1;
+    const int npl = pick_neurons_per_lane(
+        batch, neurons, common_alignment({input, out_spikes, out_vmem_rec, out_isyn_rec, ckpt_v, ckpt_i}));
     const int64_t blocks_per_batch = (neurons + BLOCK * npl - 1) / (BLOCK * npl);
     if (blocks_per_batch > 0x7fffffffLL / batch) return hipErrorInvalidValue;
     const int64_t blocks = blocks_per_batch * batch;
@@ -527,9 +555,9 @@ EXODUS_API int exodus_layer_lif_forward(float *out_spikes, float *out_vmem_rec, 
     hipLaunchKernelGGL((layer_lif_forward<SYN, NPL>), grid, block, 0, s, out_spikes, out_vmem_rec, out_isyn_rec, \
                        ckpt_v, ckpt_i, v_last, i_last, spike_sum, input, p, blocks_per_batch, t, neurons)
     if (syn) {
-        if (vec) EXODUS_FWD(true, 4); else EXODUS_FWD(true, 1);
+        if (npl == 4) EXODUS_FWD(true, 4); else if (npl == 2) EXODUS_FWD(true, 2); else EXODUS_FWD(true, 1);
     } else {
-        if (vec) EXODUS_FWD(false, 4); else EXODUS_FWD(false, 1);
+        if (npl == 4) EXODUS_FWD(false, 4); else if (npl == 2) EXODUS_FWD(false, 2); else EXODUS_FWD(false, 1);
     }
 #undef EXODUS_FWD
     return static_cast<int>(hipGetLastError());
@@ -591,14 +619,15 @@ EXODUS_API int exodus_layer_leaky_forward(float *out, float *v_last, const float
     p.alpha = alpha;
     p.decay_early = decay_early ? 1 : 0;
     p.norm_input = norm_input ? 1 : 0;
-    const bool vec = (neurons % 4) == 0 && aligned16(input) && aligned16(out);
-    const int npl = vec ? 4 : 1;
+    const int npl = pick_neurons_per_lane(batch, neurons, common_alignment({input, out}));
     const int64_t blocks_per_batch = (neurons + BLOCK * npl - 1) / (BLOCK * npl);
     if (blocks_per_batch > 0x7fffffffLL / batch) return hipErrorInvalidValue;
     const dim3 grid(static_cast<unsigned>(blocks_per_batch * batch)), block(BLOCK);
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (vec)
+    if (npl == 4)
         hipLaunchKernelGGL((layer_leaky_forward<4>), grid, block, 0, s, out, v_last, input, p, blocks_per_batch, t, neurons);
+    else if (npl == 2)
+        hipLaunchKernelGGL((layer_leaky_forward<2>), grid, block, 0, s, out, v_last, input, p, blocks_per_batch, t, neurons);
     else
         hipLaunchKernelGGL((layer_leaky_forward<1>), grid, block, 0, s, out, v_last, input, p, blocks_per_batch, t, neurons);
     return static_cast<int>(hipGetLastError());
@@ -622,9 +651,7 @@ EXODUS_API int exodus_layer_leaky_backward(float *grad_input, float *alpha_grad,
     p.alpha = alpha;
     p.decay_early = decay_early ? 1 : 0;
     p.norm_input = norm_input ? 1 : 0;
-    const bool vec = (neurons % 4) == 0 && aligned16(grad_input) && aligned16(grad_out) && aligned16(out) &&
-                     aligned16(input);
-    const int npl = vec ? 4 : 1;
+    const int npl = pick_neurons_per_lane(batch, neurons, common_alignment({grad_input, grad_out, out, input}));
     const int64_t blocks_per_batch = (neurons + BLOCK * npl - 1) / (BLOCK * npl);
     if (blocks_per_batch > 0x7fffffffLL / batch) return hipErrorInvalidValue;
     const dim3 grid(static_cast<unsigned>(blocks_per_batch * batch)), block(BLOCK);
@@ -632,8 +659,10 @@ EXODUS_API int exodus_layer_leaky_backward(float *grad_input, float *alpha_grad,
 #define EXODUS_LK(NPL, AL, WX)                                                                                 \
     hipLaunchKernelGGL((layer_leaky_backward<NPL, AL, WX>), grid, block, 0, s, grad_input, alpha_grad,        \
                        vmem_init_grad, grad_out, grad_v_last, out, input, p, blocks_per_batch, t, neurons)
-    if (vec) {
+    if (npl == 4) {
         if (with_x) EXODUS_LK(4, true, true); else if (want_alpha) EXODUS_LK(4, true, false); else EXODUS_LK(4, false, false);
+    } else if (npl == 2) {
+        if (with_x) EXODUS_LK(2, true, true); else if (want_alpha) EXODUS_LK(2, true, false); else EXODUS_LK(2, false, false);
     } else {
         if (with_x) EXODUS_LK(1, true, true); else if (want_alpha) EXODUS_LK(1, true, false); else EXODUS_LK(1, false, false);
     }

@@ -1,0 +1,147 @@
+"""The benchmark configurations at their full sizes.  A CPU comparison of 2e9 neuron-timesteps is
+out of reach, so these tests check (a) a random sample of neurons against the CPU oracle, bit for bit
+in the forward direction and within rtol 1e-4 / atol 1e-5 for gradients, and (b) size-independent
+properties: integer spike counts within the cap, the fused spike total, the lower bound, linearity
+of the backward pass in the incoming gradient."""
+import math
+
+import pytest
+import torch
+
+from _util import assert_close, gen
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def mods():
+    assert torch.cuda.is_available()
+    from oracle import exodus_ref as ref
+    from sinabs.exodus import _hip as hip
+    return hip, ref
+
+
+def need_gib(gib):
+    free, _ = torch.cuda.mem_get_info()
+    if free < gib * 2 ** 30:
+        pytest.skip(f"needs {gib} GiB of free device memory")
+
+
+def sample_columns(x, idx_b, idx_m):
+    """(B,T,M) device tensor -> (n_sample, T) CPU rows for the sampled (batch, neuron) pairs."""
+    return x[idx_b, :, idx_m].contiguous().cpu()
+
+
+def test_c5_synaptic_lif_full_size(mods):
+    hip, ref = mods
+    need_gib(60)
+    B, T, M = 16, 2000, 65536
+    N = B * M
+    dev = "cuda"
+    g = torch.Generator(device=dev).manual_seed(4)
+    x = torch.randn(B, T, M, generator=g, device=dev) * 0.5 + 0.05
+    am, asyn = math.exp(-1 / 20.0), math.exp(-1 / 5.0)
+    full = lambda v: torch.full((N,), v, device=dev)
+    a_mem, a_syn, lo, one, zero = full(am), full(asyn), full(-1.0), full(1.0), full(0.0)
+    res = hip.layerLifForward(x, zero, zero, a_mem, a_syn, one, one, lo, True, 2, True, True)
+    spikes = res["spikes"]
+
+    # properties
+    assert float(res["spike_sum"]) == float(spikes.sum(dtype=torch.float64))
+    assert bool(((spikes == 0) | (spikes == 1) | (spikes == 2)).all())
+    assert float(res["v_last"].min()) >= -1.0 - 2.0                     # post-reset: clamp minus at most 2 resets
+    assert 0 < float(res["spike_sum"]) < N * T
+
+    # sampled neurons against the oracle (composition of its pieces, as the reference layer composes them)
+    cg = gen(5)
+    n_s = 1024
+    ib = torch.randint(0, B, (n_s,), generator=cg); im = torch.randint(0, M, (n_s,), generator=cg)
+    xs = sample_columns(x, ib.to(dev), im.to(dev))
+    r = lambda v: torch.full((n_s,), v)
+    i_rows = ref.leaky_forward((xs * r(asyn)[:, None]).contiguous(), r(0.0), r(asyn))
+    ws, wv = ref.integrate_and_fire_forward(((1.0 - r(am)[:, None]) * i_rows).contiguous(), r(am), r(0.0), r(1.0), None,
+                                            r(-1.0), 2)
+    assert torch.equal(sample_columns(spikes, ib.to(dev), im.to(dev)), ws)
+    flat = (ib * M + im)
+    assert torch.equal(res["v_last"].cpu()[flat], (wv - ws)[:, -1])
+    assert torch.equal(res["i_last"].cpu()[flat], i_rows[:, -1])
+
+    # backward: sampled neurons against the oracle's chained backward, and linearity in grad_spikes
+    go1 = torch.randn(B, T, M, generator=g, device=dev)
+    bw = lambda go: hip.layerLifBackward(go, None, None, x, res["ckpt_v"], res["ckpt_i"], zero, zero, a_mem, a_syn, one,
+                                         one, lo, True, 2, True, True, hip.SURR_SINGLE_EXP, 0.5, 1.0)
+    gi1, gam1, gas1, _, _ = bw(go1)
+    gos = sample_columns(go1, ib.to(dev), im.to(dev))
+    g_u, g_am_lif, _ = ref.integrate_and_fire_backward(gos, None, wv, ws, r(0.0), r(am), r(1.0), r(1.0), r(-1.0),
+                                                       ref.SingleExponential(), True, gate_initial=True)
+    g_i = ((1.0 - r(am)[:, None]) * g_u).contiguous()
+    g_xin, g_as_leaky, _ = ref.leaky_integrator_backward(g_i, i_rows, r(0.0), r(asyn), True)
+    want_gx = g_xin * r(asyn)[:, None]
+    assert_close(sample_columns(gi1, ib.to(dev), im.to(dev)), want_gx, "grad_x of sampled neurons")
+    want_gam = g_am_lif - (g_u * i_rows).sum(1)
+    want_gas = g_as_leaky + (g_xin * xs).sum(1)
+    assert_close(gam1.cpu()[flat], want_gam, "grad alpha_mem of sampled neurons", rtol=1e-4, atol=1e-5 * T ** 0.5)
+    assert_close(gas1.cpu()[flat], want_gas, "grad alpha_syn of sampled neurons", rtol=1e-4, atol=1e-5 * T ** 0.5)
+    del go1
+    gi2, _, _, _, _ = bw(gi1 * 0 + 1.0)                                   # grad = ones
+    gi3, _, _, _, _ = bw(gi1 * 0 + 3.0)
+    assert_close(gi3[:2, :, :4096], 3.0 * gi2[:2, :, :4096], "backward is linear in grad_spikes")
+
+
+def test_c2_lif_full_size(mods):
+    hip, ref = mods
+    need_gib(30)
+    B, T, M = 32, 300, 128 * 32 * 32
+    N = B * M
+    dev = "cuda"
+    g = torch.Generator(device=dev).manual_seed(1)
+    x = torch.randn(B, T, M, generator=g, device=dev) * 0.3 + 0.1
+    am = math.exp(-1 / 20.0)
+    full = lambda v: torch.full((N,), v, device=dev)
+    a_mem, one, zero = full(am), full(1.0), full(0.0)
+    res = hip.layerLifForward(x, zero, None, a_mem, None, one, one, None, False, 1, True, True)
+    spikes = res["spikes"]
+    assert float(res["spike_sum"]) == float(spikes.sum(dtype=torch.float64))
+    assert bool(((spikes == 0) | (spikes == 1)).all())
+    cg = gen(6); n_s = 2048
+    ib = torch.randint(0, B, (n_s,), generator=cg); im = torch.randint(0, M, (n_s,), generator=cg)
+    xs = sample_columns(x, ib.to(dev), im.to(dev))
+    r = lambda v: torch.full((n_s,), v)
+    ws, wv = ref.integrate_and_fire_forward(((1.0 - r(am)[:, None]) * xs).contiguous(), r(am), r(0.0), r(1.0), None, None, 1)
+    assert torch.equal(sample_columns(spikes, ib.to(dev), im.to(dev)), ws)
+    go = torch.ones(B, T, M, device=dev)
+    gi, gam, _, gv0, _ = hip.layerLifBackward(go, None, None, x, res["ckpt_v"], None, zero, None, a_mem, None, one, one,
+                                              None, False, 1, True, True, hip.SURR_SINGLE_EXP, 0.5, 1.0)
+    g_u, g_am_lif, g_v0 = ref.integrate_and_fire_backward(torch.ones(n_s, T), None, wv, ws, r(0.0), r(am), r(1.0), r(1.0),
+                                                          None, ref.SingleExponential(), True, gate_initial=True)
+    assert_close(sample_columns(gi, ib.to(dev), im.to(dev)), (1.0 - r(am)[:, None]) * g_u, "grad_x of sampled neurons")
+    flat = ib * M + im
+    assert_close(gv0.cpu()[flat], g_v0, "grad v_init of sampled neurons")
+    assert_close(gam.cpu()[flat], g_am_lif - (g_u * xs).sum(1), "grad alpha of sampled neurons", rtol=1e-4,
+                 atol=1e-5 * T ** 0.5)
+
+
+def test_c5_rows_kernels_full_size_sampled(mods):
+    """The (rows, time) kernels at 1 048 576 x 2000 (offsets beyond 2^31): sampled rows against the oracle."""
+    hip, ref = mods
+    need_gib(45)
+    n, t = 1 << 20, 2000
+    dev = "cuda"
+    g = torch.Generator(device=dev).manual_seed(7)
+    x = torch.randn(n, t, generator=g, device=dev) * 0.5 + 0.05
+    alpha = torch.rand(n, generator=g, device=dev); th = torch.rand(n, generator=g, device=dev) + 0.5
+    zero = torch.zeros(n, device=dev); lo = -torch.ones(n, device=dev)
+    s = torch.empty_like(x); v = torch.empty_like(x)
+    hip.lifForward(s, v, x, zero, alpha, th, th, lo, True, 2)
+    idx = torch.cat([torch.tensor([0, 1, n - 2, n - 1, (1 << 20) - 64 * 3 - 1]), torch.randint(0, n, (507,), generator=gen(8))])
+    c = lambda z: z[idx.to(dev)].contiguous().cpu()
+    ws, wv = ref.lif_forward(c(x), c(zero), c(alpha), c(th), c(th), c(lo), True, 2)
+    assert torch.equal(c(s), ws) and torch.equal(c(v), wv)
+    go = torch.randn(n, t, generator=g, device=dev)
+    gi, ga, ginit = hip.lifBackwardFused(go, None, v, zero, alpha, th, th, lo, True, 2, hip.SURR_SINGLE_EXP, 0.5, 1.0,
+                                         needAlphaGrad=True)
+    wgi, wga, wginit = ref.integrate_and_fire_backward(c(go), None, wv, ws, c(zero), c(alpha), c(th), c(th), c(lo),
+                                                       ref.SingleExponential(), True, gate_initial=True)
+    assert_close(c(gi), wgi, "grad_input of sampled rows")
+    assert_close(c(ginit), wginit, "grad_init of sampled rows")
+    assert_close(c(ga), wga, "grad_alpha of sampled rows", rtol=1e-4, atol=1e-5 * t ** 0.5)
