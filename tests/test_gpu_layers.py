@@ -357,3 +357,41 @@ def test_expleak_equal_output_and_grads(L, train_alphas, norm_input):
     assert_close(xb.grad, xa.grad, "grad input", rtol=1e-4, atol=1e-5)
     for (k, p), (_, q) in zip(plain.named_parameters(), fast.named_parameters()):
         assert_close(q.grad, p.grad, f"grad {k}", rtol=1e-3, atol=1e-4)
+
+
+# ------------------------------------------------------------------------------------------ conv SNN
+def conv_snn(layers_mod, batch_size):
+    """The convolutional configuration of the benchmark description: conv / pooling work on
+    (batch*time, C, H, W), the neuron layers are the Squeeze variants in between."""
+    return nn.Sequential(
+        nn.Conv2d(2, 32, 3), layers_mod.IAFSqueeze(batch_size=batch_size), nn.AvgPool2d(2),
+        nn.Conv2d(32, 64, 3), layers_mod.IAFSqueeze(batch_size=batch_size), nn.Flatten(),
+        nn.Linear(64 * 14 * 14, 10), layers_mod.IAFSqueeze(batch_size=batch_size),
+    )
+
+
+def test_conv_snn_end_to_end(L):
+    el, sl, _ = L
+    torch.manual_seed(4)
+    batch, steps = 3, 40
+    fast = conv_snn(el, batch).cuda(); plain = conv_snn(sl, batch).cuda()
+    for i in (0, 3, 6):
+        with torch.no_grad():
+            fast[i].weight.mul_(3.0)
+        plain[i].load_state_dict(fast[i].state_dict())
+    x = (torch.rand(batch, steps, 2, 34, 34, generator=gen(30)) < 0.02).float().cuda()
+    labels = torch.randint(0, 10, (batch,), generator=gen(31)).cuda()
+
+    def run(model):
+        out = model(x.flatten(0, 1)).reshape(batch, steps, 10)
+        loss = nn.functional.cross_entropy(out.sum(1), labels)
+        loss.backward()
+        return out, loss
+
+    out_f, loss_f = run(fast); out_p, loss_p = run(plain)
+    assert out_p.sum() > 0 and torch.equal(out_f, out_p)
+    assert torch.equal(fast[1].v_mem, plain[1].v_mem)
+    assert_close(loss_f, loss_p, "loss", rtol=1e-6, atol=1e-7)
+    for (k, p), (_, q) in zip(plain.named_parameters(), fast.named_parameters()):
+        if p.grad is not None:
+            assert_close(q.grad, p.grad, f"grad {k}", rtol=1e-4, atol=1e-5)
