@@ -24,7 +24,7 @@
 namespace {
 
 #ifndef EXODUS_LAYER_FWD_UNROLL
-#define EXODUS_LAYER_FWD_UNROLL 8
+#define EXODUS_LAYER_FWD_UNROLL 16
 #endif
 #ifndef EXODUS_LAYER_BLOCK
 #define EXODUS_LAYER_BLOCK 256

@@ -1,5 +1,4 @@
-from .lif import LIF, LIFSqueeze
-from .iaf import IAF, IAFSqueeze
-from .exp_leak import ExpLeak, ExpLeakSqueeze
+"""``sinabs.exodus.layers``: LIF, IAF, ExpLeak and their Squeeze variants."""
+from .neurons import ExpLeak, ExpLeakSqueeze, IAF, IAFSqueeze, LIF, LIFSqueeze  # noqa: F401
 
 __all__ = ["LIF", "LIFSqueeze", "IAF", "IAFSqueeze", "ExpLeak", "ExpLeakSqueeze"]

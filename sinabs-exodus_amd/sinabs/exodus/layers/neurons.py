@@ -1,0 +1,411 @@
+"""The EXODUS neuron layers on the gfx950 kernels: ``LIF`` and its two specialisations ``IAF`` (no leak,
+no input normalisation) and ``ExpLeak`` (no spikes), plus the ``*Squeeze`` variants for 4-D
+(batch*time, channel, height, width) tensors.
+
+Public names, constructor arguments, parameters, states and outputs are those of the reference
+layers (reference sinabs/exodus/layers/lif.py, iaf.py, exp_leak.py); the modules ``lif``, ``iaf`` and
+``exp_leak`` next to this one re-export them under the reference's import paths.
+"""
+from typing import Callable, Optional, Tuple, Union
+
+import numpy as np
+import torch
+
+from .._compat import (LIFBase, MaxSpike, MembraneSubtract, MultiSpike, SingleExponential, SingleSpike,
+                       SqueezeMixin)
+from ..leaky import LeakyIntegrator
+from ..layer_function import LeakyLayerFunction, SpikingLayerFunction
+from ..spike import IntegrateAndFire
+from ..synaptic import SynapticIntegrateAndFire, fusable
+
+__all__ = ["LIF", "LIFSqueeze", "IAF", "IAFSqueeze", "ExpLeak", "ExpLeakSqueeze", "expand_to_1d_contiguous"]
+
+
+def expand_to_1d_contiguous(value: Union[float, torch.Tensor], shape: Tuple[int], device=None) -> torch.Tensor:
+    """Broadcast ``value`` to ``shape`` (so per-channel tensors line up with the batch dimension),
+    then flatten to a contiguous float32 vector with one entry per row of the (N, T) matrices
+    (reference sinabs/exodus/layers/lif.py:20-44).  ``device`` moves plain numbers and stray CPU
+    tensors next to the states."""
+    return torch.as_tensor(value, device=device).expand(shape).float().flatten().contiguous()
+
+
+class LIF(LIFBase):
+    """
+    Leaky integrate-and-fire layer whose dynamics and gradients run in HIP kernels.
+
+    Neuron dynamics in discrete time:
+
+    .. math ::
+        V_{mem}(t+1) = \\alpha V_{mem}(t) + (1-\\alpha)\\sum z(t)
+
+        \\text{if } V_{mem}(t) >= V_{th} \\text{, then } V_{mem} \\rightarrow V_{mem} - V_{sub}
+
+    with :math:`\\alpha = e^{-1/\\tau_{mem}}`.
+
+    Parameters
+    ----------
+    tau_mem: membrane time constant.
+    tau_syn: synaptic time constant; None (default) means no synaptic dynamics.
+    spike_threshold: spikes are emitted when v_mem reaches this value. Default 1.0.
+    spike_fn: ``MultiSpike`` / ``SingleSpike`` (pass the class) or a ``MaxSpike(k)`` instance.
+    reset_fn: a ``MembraneSubtract`` instance (the only supported reset).
+    surrogate_grad_fn: callable ``(v_mem, threshold) -> d spikes / d v_mem``.
+    min_v_mem: lower bound of v_mem, applied at every step; None = unbounded.
+    train_alphas: train the decay factors exp(-1/tau) instead of the time constants.
+    shape: optionally initialise the state with this shape; otherwise inferred from the input.
+    norm_input: scale the input current by (1 - alpha_mem).
+    record_states: keep v_mem / i_syn of every step in ``self.recordings``.
+    decay_early: apply the synaptic decay to an input already in the step it arrives, so that a
+        unit pulse gives a synaptic current of alpha rather than one (same as sinabs). Only
+        affects synaptic currents. Default True.
+    """
+
+    def __init__(
+        self,
+        tau_mem: Union[float, torch.Tensor],
+        tau_syn: Optional[Union[float, torch.Tensor]] = None,
+        spike_threshold: Optional[Union[float, torch.Tensor]] = 1.0,
+        spike_fn: Callable = MultiSpike,
+        reset_fn: Callable = MembraneSubtract(),
+        surrogate_grad_fn: Callable = SingleExponential(),
+        min_v_mem: Optional[Union[float, torch.Tensor]] = None,
+        train_alphas: bool = False,
+        shape: Optional[torch.Size] = None,
+        norm_input: bool = True,
+        record_states: bool = False,
+        decay_early: bool = True,
+    ):
+        self._parse_activation_fn(spike_fn, reset_fn)
+        super().__init__(
+            tau_mem=tau_mem,
+            tau_syn=tau_syn,
+            spike_threshold=spike_threshold,
+            spike_fn=spike_fn,
+            reset_fn=reset_fn,
+            surrogate_grad_fn=surrogate_grad_fn,
+            min_v_mem=min_v_mem,
+            train_alphas=train_alphas,
+            shape=shape,
+            norm_input=norm_input,
+            record_states=record_states,
+        )
+        self.decay_early = decay_early
+        # layers with synapses run synapse and membrane in one kernel when the surrogate gradient
+        # is one the kernels can evaluate; set to False to force the two separate Functions
+        self.fuse_synapse = True
+        # spiking layers that do not record states run one kernel per direction on the input's own
+        # (batch, time, neurons) layout (no transposing copies, no stored v_mem / i_syn); set to False
+        # to force the (rows, time) Functions
+        self.native_layout = True
+
+    def _parse_activation_fn(self, spike_fn, reset_fn):
+        """Translate the spike mechanism into a per-step spike cap (reference lif.py:130-150)."""
+        if spike_fn is None:
+            return  # non-spiking
+        supported_spike = spike_fn in (MultiSpike, SingleSpike) or isinstance(spike_fn, MaxSpike)
+        if not supported_spike or not isinstance(reset_fn, MembraneSubtract):
+            raise NotImplementedError(
+                "Spike mechanism config not supported. "
+                "Use MultiSpike/SingleSpike/MaxSpike and MembraneSubtract functions."
+            )
+        if isinstance(spike_fn, MaxSpike):
+            self.max_num_spikes_per_bin = spike_fn.max_num_spikes_per_bin
+        elif spike_fn == MultiSpike:
+            self.max_num_spikes_per_bin = None
+        else:
+            self.max_num_spikes_per_bin = 1
+
+    # ------------------------------------------------------------------ layout
+    def _prepare_input(self, input_data: torch.Tensor):
+        """(batch, time, *trailing) -> contiguous (batch*prod(trailing), time); (re)initialise the
+        states when their shape does not fit (reference lif.py:152-183)."""
+        batch_size, time_steps, *trailing_dim = input_data.shape
+        state_shape = (batch_size, *trailing_dim)
+        if not self.is_state_initialised() or not self.state_has_shape(state_shape):
+            self.init_state_with_shape(state_shape)
+        input_2d = input_data.movedim(1, -1).reshape(-1, time_steps)
+        return input_2d, (batch_size, time_steps, *trailing_dim)
+
+    @staticmethod
+    def _rows_to_full(x_2d: torch.Tensor, batch_size: int, trailing_dim) -> torch.Tensor:
+        return x_2d.reshape(batch_size, *trailing_dim, -1).movedim(-1, 1)
+
+    # ------------------------------------------------------------------ dynamics
+    def _forward_synaptic(self, input_2d: torch.Tensor) -> torch.Tensor:
+        """Exponential synapse i_t = alpha_syn * i_{t-1} + x_t (x pre-scaled by alpha_syn when
+        ``decay_early``) -- reference lif.py:185-198."""
+        alpha_syn = expand_to_1d_contiguous(self.alpha_syn_calculated, self.v_mem.shape, self.v_mem.device)
+        if self.decay_early:
+            input_2d = input_2d * alpha_syn.unsqueeze(1)
+        return LeakyIntegrator.apply(input_2d.contiguous(), alpha_syn, self.i_syn.flatten().contiguous())
+
+    def _forward_membrane(self, i_syn_2d: torch.Tensor):
+        """Membrane stage: returns (output, post-reset v_mem), both (N, T) -- reference lif.py:200-258."""
+        state_shape = self.v_mem.shape
+        dev = self.v_mem.device
+        alpha_mem = expand_to_1d_contiguous(self.alpha_mem_calculated, state_shape, dev)
+
+        if self.norm_input:
+            i_syn_2d = (1.0 - alpha_mem.unsqueeze(1)) * i_syn_2d
+
+        if self.spike_fn is None:
+            # leaky integrator without spikes: output and state are the same tensor
+            if self.decay_early:
+                i_syn_2d = i_syn_2d * alpha_mem.unsqueeze(1)
+            v_mem = LeakyIntegrator.apply(i_syn_2d.contiguous(), alpha_mem, self.v_mem.flatten().contiguous())
+            return v_mem, v_mem
+
+        spike_threshold = expand_to_1d_contiguous(self.spike_threshold, state_shape, dev)
+        min_v_mem = None if self.min_v_mem is None else expand_to_1d_contiguous(self.min_v_mem, state_shape, dev)
+        membrane_subtract = self.reset_fn.subtract_value
+        if membrane_subtract is None:
+            membrane_subtract = spike_threshold
+        else:
+            membrane_subtract = expand_to_1d_contiguous(membrane_subtract, state_shape, dev)
+
+        output_2d, v_mem_2d = IntegrateAndFire.apply(
+            i_syn_2d.contiguous(),
+            alpha_mem,
+            self.v_mem.flatten().contiguous(),
+            spike_threshold,
+            membrane_subtract,
+            min_v_mem,
+            self.surrogate_grad_fn,
+            self.max_num_spikes_per_bin,
+        )
+        # the Function returns the potential before reset; the layer state is after reset
+        v_mem_2d = v_mem_2d - membrane_subtract.unsqueeze(1) * output_2d
+        return output_2d, v_mem_2d
+
+    def _forward_synaptic_membrane(self, input_2d: torch.Tensor):
+        """Same values as ``_forward_synaptic`` followed by ``_forward_membrane`` (same operations
+        in the same order), computed by the fused kernels: returns (output, post-reset v_mem, i_syn)."""
+        state_shape, dev = self.v_mem.shape, self.v_mem.device
+        alpha_syn = expand_to_1d_contiguous(self.alpha_syn_calculated, state_shape, dev)
+        alpha_mem = expand_to_1d_contiguous(self.alpha_mem_calculated, state_shape, dev)
+        spike_threshold = expand_to_1d_contiguous(self.spike_threshold, state_shape, dev)
+        min_v_mem = None if self.min_v_mem is None else expand_to_1d_contiguous(self.min_v_mem, state_shape, dev)
+        membrane_subtract = self.reset_fn.subtract_value
+        if membrane_subtract is None:
+            membrane_subtract = spike_threshold
+        else:
+            membrane_subtract = expand_to_1d_contiguous(membrane_subtract, state_shape, dev)
+        output_2d, v_mem_2d, i_syn_2d = SynapticIntegrateAndFire.apply(
+            input_2d.contiguous(),
+            alpha_syn,
+            alpha_mem,
+            self.i_syn.flatten().contiguous(),
+            self.v_mem.flatten().contiguous(),
+            spike_threshold,
+            membrane_subtract,
+            min_v_mem,
+            self.surrogate_grad_fn,
+            self.max_num_spikes_per_bin,
+            self.decay_early,
+            self.norm_input,
+        )
+        v_mem_2d = v_mem_2d - membrane_subtract.unsqueeze(1) * output_2d
+        return output_2d, v_mem_2d, i_syn_2d
+
+    def _use_native_layout(self, input_data: torch.Tensor) -> bool:
+        if not (self.native_layout and input_data.is_cuda and input_data.dtype == torch.float32
+                and input_data.ndim >= 2):
+            return False
+        if self.spike_fn is None:                      # leaky integrator: the output is the state record
+            return self.tau_syn_calculated is None
+        return not self.record_states and fusable(self.surrogate_grad_fn)
+
+    def _forward_native_leaky(self, input_data: torch.Tensor) -> torch.Tensor:
+        batch_size, time_steps, *trailing_dim = input_data.shape
+        state_shape = (batch_size, *trailing_dim)
+        if not self.is_state_initialised() or not self.state_has_shape(state_shape):
+            self.init_state_with_shape(state_shape)
+        alpha_mem = expand_to_1d_contiguous(self.alpha_mem_calculated, state_shape, self.v_mem.device)
+        out, v_last = LeakyLayerFunction.apply(
+            input_data.reshape(batch_size, time_steps, -1).contiguous(),
+            alpha_mem,
+            self.v_mem.flatten().contiguous(),
+            self.decay_early,
+            self.norm_input,
+            state_shape,
+        )
+        out = out.reshape(input_data.shape)
+        self.recordings = {"v_mem": out} if self.record_states else dict()
+        self.v_mem = v_last
+        self.firing_rate = out.sum() / max(out.numel(), 1)
+        return out
+
+    def _forward_native(self, input_data: torch.Tensor) -> torch.Tensor:
+        """Whole layer in one kernel on (batch, time, neurons); same values as the other path."""
+        batch_size, time_steps, *trailing_dim = input_data.shape
+        state_shape = (batch_size, *trailing_dim)
+        if not self.is_state_initialised() or not self.state_has_shape(state_shape):
+            self.init_state_with_shape(state_shape)
+        dev = self.v_mem.device
+        has_syn = self.tau_syn_calculated is not None
+        alpha_mem = expand_to_1d_contiguous(self.alpha_mem_calculated, state_shape, dev)
+        alpha_syn = expand_to_1d_contiguous(self.alpha_syn_calculated, state_shape, dev) if has_syn else None
+        spike_threshold = expand_to_1d_contiguous(self.spike_threshold, state_shape, dev)
+        min_v_mem = None if self.min_v_mem is None else expand_to_1d_contiguous(self.min_v_mem, state_shape, dev)
+        membrane_subtract = self.reset_fn.subtract_value
+        if membrane_subtract is None:
+            membrane_subtract = spike_threshold
+        else:
+            membrane_subtract = expand_to_1d_contiguous(membrane_subtract, state_shape, dev)
+        spikes, v_last, i_last, spike_total = SpikingLayerFunction.apply(
+            input_data.reshape(batch_size, time_steps, -1).contiguous(),
+            alpha_mem,
+            alpha_syn,
+            self.v_mem.flatten().contiguous(),
+            self.i_syn.flatten().contiguous() if has_syn else None,
+            spike_threshold,
+            membrane_subtract,
+            min_v_mem,
+            self.surrogate_grad_fn,
+            self.max_num_spikes_per_bin,
+            self.decay_early,
+            self.norm_input,
+            state_shape,
+        )
+        self.recordings = dict()
+        self.v_mem = v_last
+        if has_syn:
+            self.i_syn = i_last
+        self.firing_rate = (spike_total / max(spikes.numel(), 1)).float()
+        return spikes.reshape(input_data.shape)
+
+    def forward(self, input_data: torch.Tensor) -> torch.Tensor:
+        """Process ``input_data`` of shape (batch, time, ...); returns a tensor of the same shape."""
+        if self._use_native_layout(input_data):
+            if self.spike_fn is None:
+                return self._forward_native_leaky(input_data)
+            return self._forward_native(input_data)
+        input_2d, (batch_size, time_steps, *trailing_dim) = self._prepare_input(input_data)
+        self.recordings = dict()
+
+        if self.tau_syn_calculated is None:
+            output_2d, v_mem_2d = self._forward_membrane(input_2d)
+        else:
+            if self.spike_fn is not None and self.fuse_synapse and fusable(self.surrogate_grad_fn):
+                # synapse and membrane in one kernel per direction
+                output_2d, v_mem_2d, i_syn_2d = self._forward_synaptic_membrane(input_2d)
+            else:
+                i_syn_2d = self._forward_synaptic(input_2d)
+                output_2d, v_mem_2d = self._forward_membrane(i_syn_2d)
+            i_syn_full = self._rows_to_full(i_syn_2d, batch_size, trailing_dim)
+            self.i_syn = i_syn_full[:, -1].clone()
+            if self.record_states:
+                self.recordings["i_syn"] = i_syn_full
+
+        v_mem_full = self._rows_to_full(v_mem_2d, batch_size, trailing_dim)
+        output_full = self._rows_to_full(output_2d, batch_size, trailing_dim)
+
+        if self.record_states:
+            self.recordings["v_mem"] = v_mem_full
+        self.v_mem = v_mem_full[:, -1].clone()
+        self.firing_rate = output_full.sum() / output_full.numel()
+        return output_full
+
+    def __repr__(self):
+        return "EXODUS " + super().__repr__()
+
+
+class IAF(LIF):
+    """
+    Integrate-and-fire layer: a ``LIF`` whose membrane does not leak (alpha = 1) and whose input is
+    not normalised.
+
+    .. math ::
+        V_{mem}(t+1) = V_{mem}(t) + \\sum z(t)
+
+        \\text{if } V_{mem}(t) >= V_{th} \\text{, then } V_{mem} \\rightarrow V_{mem} - V_{sub}
+
+    Takes the arguments of ``LIF`` except ``tau_mem``, ``train_alphas`` and ``norm_input``.
+    """
+
+    _dropped_args = ("tau_mem", "train_alphas", "norm_input")
+
+    def __init__(
+        self,
+        spike_threshold: Optional[Union[float, torch.Tensor]] = 1.0,
+        spike_fn: Callable = MultiSpike,
+        reset_fn: Callable = MembraneSubtract(),
+        surrogate_grad_fn: Callable = SingleExponential(),
+        tau_syn: Optional[Union[float, torch.Tensor]] = None,
+        min_v_mem: Optional[Union[float, torch.Tensor]] = None,
+        shape: Optional[torch.Size] = None,
+        record_states: bool = False,
+        decay_early: bool = True,
+    ):
+        LIF.__init__(self, np.inf, tau_syn, spike_threshold, spike_fn, reset_fn, surrogate_grad_fn, min_v_mem,
+                     train_alphas=False, shape=shape, norm_input=False, record_states=record_states,
+                     decay_early=decay_early)
+        self.tau_mem = None                      # an IAF neuron has no membrane time constant
+
+    @property
+    def alpha_mem_calculated(self):
+        return torch.tensor(1.0).to(self.v_mem.device)
+
+    @property
+    def _param_dict(self) -> dict:
+        return {k: v for k, v in super()._param_dict.items() if k not in self._dropped_args}
+
+
+class ExpLeak(LIF):
+    """
+    Leaky integrator without spikes: the output is the membrane potential.
+
+    .. math ::
+        V_{mem}(t+1) = \\alpha V_{mem}(t) + (1-\\alpha)\\sum z(t)
+
+    ``tau_mem``, ``shape``, ``train_alphas``, ``min_v_mem``, ``norm_input`` (default False here) and
+    ``record_states`` as for ``LIF``.  ``decay_early`` applies the decay to an input already in the step
+    it arrives, so that a unit pulse gives alpha rather than one; False (default) is the sinabs behaviour.
+    """
+
+    _dropped_args = ("tau_syn", "spike_fn", "reset_fn", "surrogate_grad_fn", "spike_threshold")
+
+    def __init__(
+        self,
+        tau_mem: Union[float, torch.Tensor],
+        shape: Optional[torch.Size] = None,
+        train_alphas: bool = False,
+        min_v_mem: Optional[float] = None,
+        norm_input: bool = False,
+        record_states: bool = False,
+        decay_early: bool = False,
+    ):
+        LIF.__init__(self, tau_mem, None, None, None, None, None, min_v_mem, train_alphas, shape, norm_input,
+                     record_states, decay_early)
+
+    @property
+    def _param_dict(self) -> dict:
+        return {k: v for k, v in super()._param_dict.items() if k not in self._dropped_args}
+
+
+def _squeezed(layer_cls: type, name: str) -> type:
+    """The variant of ``layer_cls`` for squeezed 4-D input (batch*time, channel, height, width), as
+    produced and consumed by convolution and pooling layers: it inflates the input to
+    (batch, time, ...), runs ``layer_cls`` and flattens the first two dimensions again."""
+
+    class Squeezed(layer_cls, SqueezeMixin):
+        def __init__(self, batch_size=None, num_timesteps=None, **kwargs):
+            layer_cls.__init__(self, **kwargs)
+            self.squeeze_init(batch_size, num_timesteps)
+
+        def forward(self, input_data: torch.Tensor) -> torch.Tensor:
+            return self.squeeze_forward(input_data, super().forward)
+
+        @property
+        def _param_dict(self) -> dict:
+            return self.squeeze_param_dict(super()._param_dict)
+
+    Squeezed.__name__ = Squeezed.__qualname__ = name
+    Squeezed.__module__ = __name__
+    Squeezed.__doc__ = f"``{layer_cls.__name__}`` for squeezed 4-D input (batch*time, channel, height, width)."
+    return Squeezed
+
+
+LIFSqueeze = _squeezed(LIF, "LIFSqueeze")
+IAFSqueeze = _squeezed(IAF, "IAFSqueeze")
+ExpLeakSqueeze = _squeezed(ExpLeak, "ExpLeakSqueeze")

@@ -1,60 +1,33 @@
-"""``LeakyIntegrator`` autograd Function on the gfx950 kernels.
+"""``LeakyIntegrator``: v_t = alpha * v_{t-1} + input_t on (N, Time) matrices, as an autograd Function
+on the gfx950 kernels.
 
-Same signature, checks, saved tensors and returned gradients as the reference Function
-(reference sinabs/exodus/leaky.py:5-76); the backward is a single fused reverse pass that
-yields the input gradient, the initial-state gradient and (when ``alpha`` requires grad) the
-alpha gradient together.
+Drop-in for the reference Function of the same name (reference sinabs/exodus/leaky.py:5-76): same
+arguments ``(inp (N, T), alpha (N,), v_mem_init (N,))``, same checks, same three gradients.  The
+backward is one fused reverse pass: input gradient ``g_t = alpha g_{t+1} + grad_t``, initial-state
+gradient ``alpha g_0`` and, when ``alpha`` requires grad, ``sum_t g_t out_{t-1}`` for alpha.
 """
 import torch
 
 from . import _hip
+from ._checks import check_per_row, check_rows_by_time
 
 
 class LeakyIntegrator(torch.autograd.Function):
     @staticmethod
     def forward(ctx, inp: torch.Tensor, alpha: torch.Tensor, v_mem_init: torch.Tensor):
-        """
-        Evolve a leaky integrator as ``v_t = alpha * v_{t-1} + input_t``.
-
-        Parameters
-        ----------
-        inp: 2D input, shape (N, T_sim); N is anything that can be computed in parallel
-            (batches, neurons...). Has to be contiguous.
-        alpha: 1D, shape (N,). State decay factor exp(-dt/tau). Set 1 for IAF neurons.
-        v_mem_init: 1D, shape (N,). Initial states. Has to be contiguous.
-        """
-        if not inp.ndim == 2:
-            raise ValueError("'inp' must be 2D, (N, Time)")
-        if not inp.is_contiguous():
-            raise ValueError("'inp' has to be contiguous.")
-        if not alpha.ndim == 1:
-            raise ValueError("'alpha' must be 1D, (N,)")
-        if not alpha.is_contiguous():
-            raise ValueError("'alpha' has to be contiguous.")
-        if not v_mem_init.ndim == 1:
-            raise ValueError("'v_mem_init' must be 1D, (N,)")
-        if not v_mem_init.is_contiguous():
-            raise ValueError("'v_mem_init' has to be contiguous.")
-
+        check_rows_by_time("inp", inp)
+        check_per_row(alpha=alpha, v_mem_init=v_mem_init)
         out = _hip.leakyForward(inp, v_mem_init, alpha)
-
         ctx.get_alpha_grads = alpha.requires_grad
-        if alpha.requires_grad:
-            ctx.save_for_backward(out, v_mem_init, alpha)
-        else:
-            ctx.save_for_backward(alpha)
+        # the output is only needed again for the alpha gradient
+        ctx.save_for_backward(alpha, *((out, v_mem_init) if alpha.requires_grad else ()))
         return out
 
     @staticmethod
     def backward(ctx, grad_output):
-        grad_output = grad_output.contiguous()
-        if ctx.get_alpha_grads:
-            out, v_mem_init, alpha = ctx.saved_tensors
-            grad_input, grad_alpha, grad_init = _hip.leakyBackwardFused(
-                grad_output, alpha, output=out, vmemInitial=v_mem_init, needAlphaGrad=True
-            )
-        else:
-            (alpha,) = ctx.saved_tensors
-            grad_input, grad_alpha, grad_init = _hip.leakyBackwardFused(grad_output, alpha)
-        # grad_init is one more decay step back from the first time point: alpha * grad_input[:, 0]
+        alpha, *extra = ctx.saved_tensors
+        out, v_mem_init = extra if ctx.get_alpha_grads else (None, None)
+        grad_input, grad_alpha, grad_init = _hip.leakyBackwardFused(
+            grad_output.contiguous(), alpha, output=out, vmemInitial=v_mem_init, needAlphaGrad=ctx.get_alpha_grads
+        )
         return grad_input, grad_alpha, grad_init

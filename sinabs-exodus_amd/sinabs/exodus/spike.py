@@ -21,6 +21,7 @@ from typing import Callable, Optional, Tuple, Union
 import torch
 
 from . import _hip
+from ._checks import check_per_row, check_rows_by_time
 
 _KNOWN_SURROGATE_MODULES = ("sinabs.activation", "sinabs.exodus._compat")
 
@@ -80,31 +81,9 @@ class IntegrateAndFire(torch.autograd.Function):
             membrane_subtract = torch.ones_like(alpha) * threshold
         apply_min_v_mem = min_v_mem is not None
 
-        if not inp.ndim == 2:
-            raise ValueError("'inp' must be 2D, (N, Time)")
-        if not inp.is_contiguous():
-            raise ValueError("'inp' has to be contiguous.")
-        if not alpha.ndim == 1:
-            raise ValueError("'alpha' must be 1D, (N,)")
-        if not alpha.is_contiguous():
-            raise ValueError("'alpha' has to be contiguous.")
-        if not membrane_subtract.ndim == 1:
-            raise ValueError("'membrane_subtract' must be 1D, (N,)")
-        if not membrane_subtract.is_contiguous():
-            raise ValueError("'membrane_subtract' has to be contiguous.")
-        if not v_mem_init.ndim == 1:
-            raise ValueError("'v_mem_init' must be 1D, (N,)")
-        if not v_mem_init.is_contiguous():
-            raise ValueError("'v_mem_init' has to be contiguous.")
-        if not threshold.ndim == 1:
-            raise ValueError("'threshold' must be 1D, (N,)")
-        if not threshold.is_contiguous():
-            raise ValueError("'threshold' has to be contiguous.")
-        if apply_min_v_mem:
-            if not min_v_mem.ndim == 1:
-                raise ValueError("'min_v_mem' must be 1D, (N,)")
-            if not min_v_mem.is_contiguous():
-                raise ValueError("'min_v_mem' has to be contiguous.")
+        check_rows_by_time("inp", inp)
+        check_per_row(alpha=alpha, membrane_subtract=membrane_subtract, v_mem_init=v_mem_init, threshold=threshold,
+                      min_v_mem=min_v_mem)
 
         # value checks: one device->host transfer for both conditions
         alpha_bad = ((alpha < 0) | (alpha > 1)).any()

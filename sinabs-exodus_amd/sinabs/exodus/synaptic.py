@@ -14,6 +14,7 @@ from typing import Callable, Optional
 import torch
 
 from . import _hip
+from ._checks import check_per_row, check_rows_by_time
 from .spike import classify_surrogate
 
 
@@ -46,19 +47,9 @@ class SynapticIntegrateAndFire(torch.autograd.Function):
         if kind == _hip.SURR_TENSOR:
             raise ValueError("surrogate_grad_fn is not one the fused kernel can evaluate; "
                              "use LeakyIntegrator and IntegrateAndFire instead")
-        if not inp.ndim == 2:
-            raise ValueError("'inp' must be 2D, (N, Time)")
-        if not inp.is_contiguous():
-            raise ValueError("'inp' has to be contiguous.")
-        for name, x in (("alpha_syn", alpha_syn), ("alpha_mem", alpha_mem), ("i_syn_init", i_syn_init),
-                        ("v_mem_init", v_mem_init), ("threshold", threshold),
-                        ("membrane_subtract", membrane_subtract), ("min_v_mem", min_v_mem)):
-            if x is None:
-                continue
-            if not x.ndim == 1:
-                raise ValueError(f"'{name}' must be 1D, (N,)")
-            if not x.is_contiguous():
-                raise ValueError(f"'{name}' has to be contiguous.")
+        check_rows_by_time("inp", inp)
+        check_per_row(alpha_syn=alpha_syn, alpha_mem=alpha_mem, i_syn_init=i_syn_init, v_mem_init=v_mem_init,
+                      threshold=threshold, membrane_subtract=membrane_subtract, min_v_mem=min_v_mem)
         apply_min = min_v_mem is not None
         checks = [((alpha_mem < 0) | (alpha_mem > 1)).any(), ((alpha_syn < 0) | (alpha_syn > 1)).any()]
         if apply_min:
