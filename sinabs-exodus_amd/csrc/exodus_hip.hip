@@ -53,6 +53,10 @@ __device__ __forceinline__ f32x4 load4(const float *__restrict__ base, int64_t r
         const float *p = base + row * n_steps + t;
         if (VEC) {
             if (t >= 0 && t + 3 < n_steps) v = ld_stream(reinterpret_cast<const f32x4 *>(p));
+        } else if (t >= 0 && t + 3 < n_steps && (reinterpret_cast<uintptr_t>(p) & 15u) == 0) {
+            // rows of any length: tiles are aligned to memory, so a chunk that lies inside its row is a
+            // 16-byte aligned vector; only the chunks that straddle a row boundary go element by element
+            v = ld_stream(reinterpret_cast<const f32x4 *>(p));
         } else {
             if (t + 0 >= 0 && t + 0 < n_steps) v.x = ld_stream(p + 0);
             if (t + 1 >= 0 && t + 1 < n_steps) v.y = ld_stream(p + 1);
@@ -71,6 +75,8 @@ __device__ __forceinline__ void store4(float *__restrict__ base, int64_t row, in
         float *p = base + row * n_steps + t;
         if (VEC) {
             if (t >= 0 && t + 3 < n_steps) st_stream(v, reinterpret_cast<f32x4 *>(p));
+        } else if (t >= 0 && t + 3 < n_steps && (reinterpret_cast<uintptr_t>(p) & 15u) == 0) {
+            st_stream(v, reinterpret_cast<f32x4 *>(p));
         } else {
             if (t + 0 >= 0 && t + 0 < n_steps) st_stream(v.x, p + 0);
             if (t + 1 >= 0 && t + 1 < n_steps) st_stream(v.y, p + 1);
