@@ -13,6 +13,7 @@ from typing import Callable, Optional
 import torch
 
 from . import _hip
+from ._validate import check_parameters
 from .spike import classify_surrogate
 
 
@@ -48,16 +49,7 @@ class SpikingLayerFunction(torch.autograd.Function):
             membrane_subtract = threshold
         syn = alpha_syn is not None
         apply_min = min_v_mem is not None
-        checks = [((alpha_mem < 0) | (alpha_mem > 1)).any()]
-        if syn:
-            checks.append(((alpha_syn < 0) | (alpha_syn > 1)).any())
-        if apply_min:
-            checks.append((threshold <= min_v_mem).any())
-        flags = torch.stack(checks).tolist()
-        if flags[0] or (syn and flags[1]):
-            raise ValueError("'alpha' must be between 0 and 1.")
-        if apply_min and flags[-1]:
-            raise ValueError("`threshold` must be greater than `min_v_mem`.")
+        check_parameters([alpha_mem, alpha_syn] if syn else [alpha_mem], threshold, min_v_mem)
 
         max_spikes = -1 if max_num_spikes_per_bin is None else int(max_num_spikes_per_bin)
         need_grad = any(ctx.needs_input_grad)

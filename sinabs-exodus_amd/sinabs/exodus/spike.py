@@ -22,6 +22,7 @@ import torch
 
 from . import _hip
 from ._checks import check_per_row, check_rows_by_time
+from ._validate import check_parameters
 
 _KNOWN_SURROGATE_MODULES = ("sinabs.activation", "sinabs.exodus._compat")
 
@@ -85,16 +86,7 @@ class IntegrateAndFire(torch.autograd.Function):
         check_per_row(alpha=alpha, membrane_subtract=membrane_subtract, v_mem_init=v_mem_init, threshold=threshold,
                       min_v_mem=min_v_mem)
 
-        # value checks: one device->host transfer for both conditions
-        alpha_bad = ((alpha < 0) | (alpha > 1)).any()
-        if apply_min_v_mem and threshold.shape == min_v_mem.shape:
-            flags = torch.stack((alpha_bad, (threshold <= min_v_mem).any())).tolist()
-        else:
-            flags = [bool(alpha_bad), bool((threshold <= min_v_mem).any()) if apply_min_v_mem else False]
-        if flags[0]:
-            raise ValueError("'alpha' must be between 0 and 1.")
-        if flags[1]:
-            raise ValueError("`threshold` must be greater than `min_v_mem`.")
+        check_parameters([alpha], threshold, min_v_mem)      # alpha in [0, 1], threshold > min_v_mem
 
         v_mem = torch.empty_like(inp)
         output_spikes = torch.empty_like(inp)

@@ -15,6 +15,7 @@ import torch
 
 from . import _hip
 from ._checks import check_per_row, check_rows_by_time
+from ._validate import check_parameters
 from .spike import classify_surrogate
 
 
@@ -51,14 +52,7 @@ class SynapticIntegrateAndFire(torch.autograd.Function):
         check_per_row(alpha_syn=alpha_syn, alpha_mem=alpha_mem, i_syn_init=i_syn_init, v_mem_init=v_mem_init,
                       threshold=threshold, membrane_subtract=membrane_subtract, min_v_mem=min_v_mem)
         apply_min = min_v_mem is not None
-        checks = [((alpha_mem < 0) | (alpha_mem > 1)).any(), ((alpha_syn < 0) | (alpha_syn > 1)).any()]
-        if apply_min:
-            checks.append((threshold <= min_v_mem).any())
-        flags = torch.stack(checks).tolist()
-        if flags[0] or flags[1]:
-            raise ValueError("'alpha' must be between 0 and 1.")
-        if apply_min and flags[2]:
-            raise ValueError("`threshold` must be greater than `min_v_mem`.")
+        check_parameters([alpha_mem, alpha_syn], threshold, min_v_mem)
 
         max_spikes = -1 if max_num_spikes_per_bin is None else int(max_num_spikes_per_bin)
         spikes, v_mem, i_syn = _hip.synLifForward(

@@ -252,3 +252,25 @@ def test_compare_leakyintegrator_backward(fns, oracle):
     assert_close(in_x.grad, in_o.grad, "grad input", rtol=1e-5, atol=1e-6)
     assert_close(v0_x.grad, v0_o.grad, "grad v_init", rtol=1e-5, atol=1e-6)
     assert_close(a_x.grad, a_o.grad, "grad alpha", rtol=1e-4, atol=1e-4)
+
+
+def test_deferred_parameter_validation(fns, oracle):
+    """In 'deferred' mode a bad alpha does not stop the call that carries it; the error surfaces at
+    flush() (or at a later call), and good parameters never raise."""
+    IntegrateAndFire, _ = fns
+    ref, _ = oracle
+    from sinabs.exodus import _validate as val
+    x = torch.rand(2, 10).cuda(); one = torch.ones(2).cuda(); zero = torch.zeros(2).cuda()
+    try:
+        val.set_mode("deferred")
+        IntegrateAndFire.apply(x, one * 0.9, zero, one, one, None, ref.Heaviside())
+        val.flush()
+        IntegrateAndFire.apply(x, torch.tensor([0.5, 1.5]).cuda(), zero, one, one, None, ref.Heaviside())
+        with pytest.raises(ValueError, match="between 0 and 1"):
+            val.flush()
+        IntegrateAndFire.apply(x, one * 0.9, zero, one, one, -one * 2, ref.Heaviside())
+        IntegrateAndFire.apply(x, one * 0.9, zero, one, one, one * 2, ref.Heaviside())
+        with pytest.raises(ValueError, match="greater than"):
+            val.flush()
+    finally:
+        val.set_mode("sync")

@@ -164,3 +164,25 @@ def test_conversion_both_ways():
 def test_bench_refuses_more_than_one_gpu():
     out = subprocess.run(["python", os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
     assert out.returncode != 0 and "one GPU" in (out.stderr + out.stdout)
+
+
+def test_parameter_validation_modes():
+    from sinabs.exodus import _validate as val
+    good, bad = torch.tensor([0.0, 0.5, 1.0]), torch.tensor([0.5, 1.5])
+    th, lo_ok, lo_bad = torch.ones(2), torch.tensor([-1.0, 0.0]), torch.tensor([1.2, 0.0])
+    assert val.get_mode() == "sync"
+    val.check_parameters([good], th, lo_ok)
+    with pytest.raises(ValueError, match="between 0 and 1"):
+        val.check_parameters([good, bad])
+    with pytest.raises(ValueError, match="greater than `min_v_mem`"):
+        val.check_parameters([good], th, lo_bad)
+    try:
+        val.set_mode("off")
+        val.check_parameters([bad], th, lo_bad)               # nothing is checked
+        val.set_mode("deferred")
+        with pytest.raises(ValueError):                          # CPU tensors cannot be deferred: raised at once
+            val.check_parameters([bad])
+        with pytest.raises(ValueError):
+            val.set_mode("nonsense")
+    finally:
+        val.set_mode("sync")
