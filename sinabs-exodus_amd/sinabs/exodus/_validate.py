@@ -10,6 +10,9 @@ on every forward call.  Three modes, selected with ``set_mode``:
                         raised by a later call into this module (or by ``flush()``), so the host can
                         keep queueing work;
 ``"off"``               no checks.
+
+While the current stream is capturing a HIP graph no check runs in any mode: the capture cannot wait
+for the device, and a replay has no host code that could raise.
 """
 from typing import List, Optional, Sequence
 
@@ -60,6 +63,8 @@ def check_parameters(alphas: Sequence[torch.Tensor], threshold: Optional[torch.T
     """``alphas``: decay factors that must lie in [0, 1]; ``threshold`` must exceed ``min_v_mem``."""
     if _MODE == "off":
         return
+    if torch.cuda.is_available() and torch.cuda.is_current_stream_capturing():
+        return          # a graph under capture can neither wait for the device nor raise on replay
     if _MODE == "deferred":
         _poll(wait=False)
     flags = [((a < 0) | (a > 1)).any() for a in alphas]

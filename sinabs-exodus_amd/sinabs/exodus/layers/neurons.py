@@ -25,7 +25,10 @@ def expand_to_1d_contiguous(value: Union[float, torch.Tensor], shape: Tuple[int]
     """Broadcast ``value`` to ``shape`` (so per-channel tensors line up with the batch dimension),
     then flatten to a contiguous float32 vector with one entry per row of the (N, T) matrices
     (reference sinabs/exodus/layers/lif.py:20-44).  ``device`` moves plain numbers and stray CPU
-    tensors next to the states."""
+    tensors next to the states; a plain number is written by a fill kernel rather than copied from
+    host memory, which also works while a HIP graph is being captured."""
+    if not isinstance(value, torch.Tensor):
+        return torch.full((int(np.prod(shape)),), float(value), dtype=torch.float32, device=device)
     return torch.as_tensor(value, device=device).expand(shape).float().flatten().contiguous()
 
 
@@ -344,7 +347,7 @@ class IAF(LIF):
 
     @property
     def alpha_mem_calculated(self):
-        return torch.tensor(1.0).to(self.v_mem.device)
+        return torch.ones((), device=self.v_mem.device)
 
     @property
     def _param_dict(self) -> dict:

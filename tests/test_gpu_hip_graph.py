@@ -1,0 +1,87 @@
+"""A whole forward + backward pass of a small spiking network recorded into a HIP graph
+(``torch.cuda.CUDAGraph``) and replayed: every entry point only enqueues kernels on the stream it is
+given, so the recording holds the hand-written kernels themselves and a replay skips the host side.
+
+Each replay is compared with the same step run eagerly; between replays the program does ordinary eager
+work and waits for the device, so that a node that only works on the first replay is caught."""
+import pytest
+import torch
+import torch.nn as nn
+
+from _util import assert_close, gen
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def el():
+    assert torch.cuda.is_available()
+    import sinabs.exodus.layers as layers
+    return layers
+
+
+def small_network(el, tau_syn):
+    from sinabs.exodus._compat import activation as act
+    return nn.Sequential(
+        nn.Linear(24, 96, bias=False),
+        el.LIF(tau_mem=15.0, tau_syn=tau_syn, min_v_mem=-1.0, spike_fn=act.MaxSpike(2), train_alphas=True, norm_input=False),
+        nn.Linear(96, 10, bias=False),
+        el.IAF(),
+    ).cuda()
+
+
+def step(model, x, weight):
+    """One training-style pass from zero states; returns output spikes, leaves gradients in ``.grad``."""
+    for m in model:
+        if hasattr(m, "reset_states"):
+            m.reset_states()
+    out = model(x)
+    (out * weight).sum().backward()
+    return out
+
+
+@pytest.mark.parametrize("tau_syn", [None, 4.0])
+def test_replays_equal_eager_steps(el, tau_syn):
+    torch.manual_seed(11)
+    recorded = small_network(el, tau_syn); eager = small_network(el, tau_syn)
+    with torch.no_grad():
+        recorded[0].weight.mul_(6.0); recorded[2].weight.mul_(4.0)
+    eager.load_state_dict(recorded.state_dict())
+    batch, steps = 4, 50
+    inputs = [(torch.rand(batch, steps, 24, generator=gen(40 + k)) * (1.0 + 0.5 * k)).cuda() for k in range(4)]
+    weight = torch.rand(batch, steps, 10, generator=gen(39)).cuda()
+    x_static = inputs[0].clone()
+
+    # the usual recipe: a few eager passes on a side stream, gradients released, then the capture
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            step(recorded, x_static, weight)
+            recorded.zero_grad(set_to_none=True)
+    torch.cuda.current_stream().wait_stream(side)
+
+    # the recording zeroes and reads the state tensors that exist now; the layers replace them by new ones
+    # during the pass, so the program has to keep these alive for as long as it replays the graph
+    held = [buf for buf in recorded.buffers()]
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out_static = step(recorded, x_static, weight)
+    grads_static = {k: p.grad for k, p in recorded.named_parameters() if p.grad is not None}
+    assert {"0.weight", "1.alpha_mem", "2.weight"} <= set(grads_static)
+
+    active = 0
+    for k in (1, 2, 0, 3, 1):
+        eager.zero_grad(set_to_none=True)
+        want = step(eager, inputs[k], weight)
+        torch.cuda.synchronize()
+        x_static.copy_(inputs[k])
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out_static, want), f"spikes differ on replay with input {k}"
+        assert torch.equal(recorded[1].v_mem, eager[1].v_mem) and torch.equal(recorded[3].v_mem, eager[3].v_mem)
+        for name, p in eager.named_parameters():
+            if p.grad is not None:
+                assert_close(grads_static[name], p.grad, f"grad {name}, input {k}", rtol=1e-5, atol=1e-6)
+        active += int(want.sum().item() > 0)
+    assert active == 5
