@@ -313,6 +313,13 @@ def main():
             "other_kernel": {"kernel": other_name, "kernel_ms": other_ms,
                              "achieved": N * T * other_bytes / (other_ms * 1e-3) / 1e9},
             "fwd_bwd_combined_frac": N * T * (bf + bb) / ((fwd_ms + bwd_ms) * 1e-3) / 1e9 / HBM_PEAK_GBS,
+            # the same durations priced with the bytes of a kernel pair that stores and re-reads the
+            # states (the figure the workload description quotes); "frac" above uses what this
+            # design has to move, which is less because the backward pass recomputes the states
+            "priced_at_stored_state_bytes": {
+                "bytes_per_neuron_timestep": sum(WORKLOADS[args.workload]["bytes"]),
+                "fwd_bwd_combined_frac": N * T * sum(WORKLOADS[args.workload]["bytes"])
+                / ((fwd_ms + bwd_ms) * 1e-3) / 1e9 / HBM_PEAK_GBS},
         },
     }
     if not args.no_cpu_baseline:

@@ -218,6 +218,28 @@ int exodus_layer_leaky_backward(float *grad_input, float *alpha_grad, float *vme
                                 int decay_early, int norm_input, int64_t batch, int64_t t,
                                 int64_t neurons, void *stream);
 
+/* ---- experimental spike generation on a precomputed membrane potential -------------------------
+ * Replaces spikeForward (reference cuda/bindings.cu:262-290, kernel
+ * cuda/experimental_kernels.h:16-65).  vmem (n, t) holds the response to the input and is updated
+ * in place with the effect of resets (each spike lowers every later step by alpha^j *
+ * membr_subtract * count) and of the lower bound (a step below theta_low keeps its value and raises
+ * every later step by alpha^j * (theta_low - u)); out_spikes (n, t) receives
+ * min(trunc(u / theta), max_num_spikes) where u >= theta, else 0 (max_num_spikes < 0: no cap).
+ * Parameters are scalars, as in the reference.  The corrections are accumulated in one running
+ * value per row (O(t) instead of the reference's O(t^2)), so potentials agree with the reference to
+ * float rounding, not bit for bit.  spikeBackwardRefr (cuda/bindings.cu:292-325), which no Python
+ * code of the reference calls, has no counterpart. */
+int exodus_spike_forward(float *out_spikes, float *vmem, float alpha, float membr_subtract, float theta,
+                         float theta_low, int apply_theta_low, int max_num_spikes, int64_t n, int64_t t,
+                         void *stream);
+
+/* Replaces spikeBackward (reference cuda/bindings.cu:327-359, kernel
+ * cuda/experimental_kernels.h:95-141): gradient with respect to the potential handed to
+ * exodus_spike_forward, from surr, output_grad and not_clipped (all (n, t)), as one reverse pass. */
+int exodus_spike_backward(float *input_grad, const float *surr, const float *output_grad,
+                          const float *not_clipped, float alpha, float membr_subtract, int64_t n,
+                          int64_t t, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

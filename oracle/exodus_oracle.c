@@ -2,8 +2,8 @@
  * TEST INFRASTRUCTURE ONLY -- not part of the shipped library.
  *
  * Scalar CPU restatement of the arithmetic of the six production device
- * routines of the EXODUS reference (one row = one neuron, sequential in
- * time).  Each function names the reference lines it follows.  The loops are
+ * routines of the EXODUS reference and of its experimental spike-generation
+ * pair (one row = one neuron, sequential in time).  Each function names the reference lines it follows.  The loops are
  * written row-major over an (n_rows, n_steps) fp32 matrix with 64-bit
  * offsets.  Build with -ffp-contract=off so that every multiply and add is
  * rounded on its own, which is what the HIP kernels are checked against
@@ -199,5 +199,90 @@ EXPORT void oracle_lif_backward_alpha(float *grad_alpha, const float *grad_out,
             acc += d * g[j];
         }
         grad_alpha[r] = acc;
+    }
+}
+
+/* ---------------------------------------------------------------------------
+ * Experimental spike-generation pair of the reference (spikes from a membrane
+ * potential that already contains the response to the input; only the reset
+ * and the lower bound act here).  Scalar parameters, as in the reference.
+ *
+ * What pins these two (tests/test_oracle_pins.py):
+ *   oracle_spike_forward   notebook cells 2/4 known answer on cumsum(input); on a dyadic grid
+ *                          (all arithmetic exact) it equals oracle_lif_forward applied to the
+ *                          input whose leaky integral is the given potential
+ *   oracle_spike_backward  alpha = 1, nothing clipped: its leaky adjoint equals the notebook's
+ *                          cell 4/6 gradients and oracle_lif_backward; for alpha != 1 or clipped
+ *                          steps only the agreement of this O(T^2) sum with an O(T) recurrence in
+ *                          float64 is checked -- parity unpinned there
+ * ------------------------------------------------------------------------- */
+
+/* For each step in turn: a potential at or above theta emits min(trunc(u/theta), cap) spikes and
+ * every later step of the row loses alpha^j * c * count; otherwise, with the lower bound on, a
+ * potential below theta_low leaves its own step untouched and raises every later step by
+ * alpha^j * (theta_low - u).  u is updated in place.
+ *                                        reference cuda/experimental_kernels.h:33-63 */
+EXPORT void oracle_spike_forward(float *spikes, float *u, float alpha, float membr_subtract,
+                                 float theta, float theta_low, int apply_theta_low,
+                                 int max_num_spikes, int64_t n_rows, int64_t n_steps)
+{
+    const unsigned cap = (unsigned)max_num_spikes;
+#pragma omp parallel for num_threads(g_threads) schedule(static)
+    for (int64_t r = 0; r < n_rows; ++r) {
+        float *v = u + r * n_steps;
+        float *s = spikes + r * n_steps;
+        for (int64_t i = 0; i < n_steps; ++i) {
+            s[i] = 0.0f;
+            if (v[i] >= theta) {
+                unsigned k = (unsigned)(v[i] / theta);
+                if (k > cap)
+                    k = cap;
+                s[i] = (float)k;
+                float w = alpha;
+                for (int64_t j = i + 1; j < n_steps; ++j) {
+                    float drop = w * membr_subtract;
+                    drop = drop * (float)k;
+                    v[j] -= drop;
+                    w *= alpha;
+                }
+            } else if (apply_theta_low && v[i] < theta_low) {
+                float lift = theta_low - v[i];
+                for (int64_t j = i + 1; j < n_steps; ++j) {
+                    lift *= alpha;
+                    v[j] += lift;
+                }
+            }
+        }
+    }
+}
+
+/* gi_i = y_i go_i - sum_{j>i} go_j y_j * (y_i c) * prod_{i<k<j} (alpha - c y_k),  y = surr * nc,
+ * summed term by term in float with the running product, stopping once the product is zero.
+ *                                        reference cuda/experimental_kernels.h:118-140 */
+EXPORT void oracle_spike_backward(float *grad_in, const float *grad_out, const float *surr,
+                                  const float *not_clipped, float alpha, float membr_subtract,
+                                  int64_t n_rows, int64_t n_steps)
+{
+#pragma omp parallel for num_threads(g_threads) schedule(static)
+    for (int64_t r = 0; r < n_rows; ++r) {
+        const float *go = grad_out + r * n_steps;
+        const float *s = surr + r * n_steps;
+        const float *nc = not_clipped + r * n_steps;
+        float *gi = grad_in + r * n_steps;
+        for (int64_t i = 0; i < n_steps; ++i) {
+            float acc = s[i] * nc[i];
+            float prod = acc * membr_subtract;
+            acc = acc * go[i];
+            for (int64_t j = i + 1; j < n_steps && prod != 0.0f; ++j) {
+                float term = go[j] * s[j];
+                term = term * nc[j];
+                term = term * prod;
+                acc -= term;
+                float f = membr_subtract * nc[j];
+                f = f * s[j];
+                prod *= alpha - f;
+            }
+            gi[i] = acc;
+        }
     }
 }

@@ -32,7 +32,9 @@ _int = ctypes.c_int
 
 def build(force: bool = False) -> str:
     """Compile the C restatement with the committed Makefile (gcc, seconds)."""
-    if force or not os.path.exists(_LIB_PATH):
+    src = os.path.join(_HERE, "exodus_oracle.c")
+    stale = not os.path.exists(_LIB_PATH) or os.path.getmtime(src) > os.path.getmtime(_LIB_PATH)
+    if force or stale:
         subprocess.check_call(["make", "-s", "-C", _HERE] + (["-B"] if force else []))
     return _LIB_PATH
 
@@ -50,9 +52,11 @@ def lib() -> ctypes.CDLL:
         L.oracle_lif_forward.argtypes = [_f32p] * 8 + [_int, _int, _i64, _i64]
         L.oracle_lif_backward.argtypes = [_f32p] * 6 + [_i64, _i64]
         L.oracle_lif_backward_alpha.argtypes = [_f32p] * 8 + [_int, _i64, _i64]
+        L.oracle_spike_forward.argtypes = [_f32p] * 2 + [ctypes.c_float] * 4 + [_int, _int, _i64, _i64]
+        L.oracle_spike_backward.argtypes = [_f32p] * 4 + [ctypes.c_float] * 2 + [_i64, _i64]
         for name in ("oracle_leaky_forward", "oracle_leaky_backward", "oracle_leaky_backward_alpha",
                      "oracle_lif_forward", "oracle_lif_backward", "oracle_lif_backward_alpha",
-                     "oracle_set_threads"):
+                     "oracle_spike_forward", "oracle_spike_backward", "oracle_set_threads"):
             getattr(L, name).restype = None
         _lib = L
     return _lib
@@ -143,6 +147,26 @@ def lif_backward_alpha(surr, grad_out, v_post, v_post_init, not_clipped, alpha, 
 # --------------------------------------------------------------------------------------
 # Function-level glue (what the reference autograd Functions compute around the kernels)
 # --------------------------------------------------------------------------------------
+
+def spike_forward(v_mem, alpha, membr_subtract, theta, theta_low, apply_theta_low, max_num_spikes):
+    """Experimental spike generation; ``v_mem`` (N, T) is updated in place, returns the spikes."""
+    _chk(v_mem, 2, "v_mem")
+    n, t = v_mem.shape
+    spikes = torch.empty_like(v_mem)
+    lib().oracle_spike_forward(_p(spikes), _p(v_mem), float(alpha), float(membr_subtract), float(theta),
+                               float(theta_low), int(bool(apply_theta_low)), int(max_num_spikes), n, t)
+    return spikes
+
+
+def spike_backward(surr, grad_out, not_clipped, alpha, membr_subtract):
+    for nm, x in (("surr", surr), ("grad_out", grad_out), ("not_clipped", not_clipped)):
+        _chk(x, 2, nm)
+    n, t = surr.shape
+    gi = torch.empty_like(surr)
+    lib().oracle_spike_backward(_p(gi), _p(grad_out), _p(surr), _p(not_clipped), float(alpha),
+                                float(membr_subtract), n, t)
+    return gi
+
 
 def integrate_and_fire_forward(inp, alpha, v_mem_init, threshold, membrane_subtract=None,
                                min_v_mem=None, max_num_spikes_per_bin: Optional[int] = None):

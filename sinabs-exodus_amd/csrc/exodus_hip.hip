@@ -599,6 +599,64 @@ struct LifBwdAlphaTensorsOp {
     __device__ __forceinline__ void finish(State &s, int64_t row) const { alpha_grad[row] = static_cast<float>(s.acc); }
 };
 
+// Spike generation on a membrane potential that already holds the response to the input (the
+// reference's experimental spikeForward): only reset and lower bound act.  The reference subtracts
+// alpha^j * c * count from every later step for each spike, one spike after the other; here the sum
+// of all pending corrections is one running value  adj_t = alpha * (adj_{t-1} + d_{t-1})  with
+// d = -c * count after a spike and d = theta_low - u below the lower bound, which is the same
+// real-number result in O(T) instead of O(T^2) (float rounding differs in the last bits).
+// out[0] = corrected potential, written over the input; spikes are derived from it on the way out.
+struct SpikeFwdOp {
+    static constexpr int NIN = 1, NOUT = 1, NDER = 1, NROWP = 1, DER_SRC = 0;
+    static constexpr bool REVERSE = false;
+    const float *in[1];
+    float *out[1];
+    float *der;
+    float alpha, c, theta, theta_low;
+    int apply_low;
+    unsigned cap;
+    struct State { float adj; };
+    __device__ __forceinline__ void init(State &s, int64_t, bool) const { s.adj = 0.f; }
+    __device__ __forceinline__ void stash(const State &, float *p) const { p[0] = theta; }
+    __device__ __forceinline__ f32x4 derive(const float *p, f32x4 v) const { return spike_count4(v, p[0], cap); }
+    __device__ __forceinline__ void step(State &s, const float *x, float *y) const
+    {
+        const float u = __fadd_rn(x[0], s.adj);
+        y[0] = u;
+        float d = 0.f;
+        if (u >= theta)
+            d = -__fmul_rn(c, spike_count(u, theta, cap));
+        else if (apply_low && u < theta_low)
+            d = __fsub_rn(theta_low, u);
+        s.adj = __fmul_rn(alpha, __fadd_rn(s.adj, d));
+    }
+    __device__ __forceinline__ void end_tile(State &) const {}
+    __device__ __forceinline__ void finish(State &, int64_t) const {}
+};
+
+// Its backward (the reference's experimental spikeBackward), with y = surr * not_clipped:
+//   gi_i = y_i go_i - (y_i c) m_i,   m_i = go_{i+1} y_{i+1} + (alpha - c y_{i+1}) m_{i+1},  m_{T-1} = 0
+// which is the reference's per-element sum over j > i written as one reverse pass.
+struct SpikeBwdOp {
+    static constexpr int NDER = 0, NROWP = 0;
+    static constexpr int NIN = 3, NOUT = 1;                   // in: grad_out, surr, not_clipped
+    static constexpr bool REVERSE = true;
+    const float *in[3];
+    float *out[1];
+    float alpha, c;
+    struct State { float m; };
+    __device__ __forceinline__ void init(State &s, int64_t, bool) const { s.m = 0.f; }
+    __device__ __forceinline__ void step(State &s, const float *x, float *y) const
+    {
+        const float g = __fmul_rn(x[1], x[2]);
+        const float gy = __fmul_rn(g, x[0]);
+        y[0] = __fsub_rn(gy, __fmul_rn(__fmul_rn(g, c), s.m));
+        s.m = __fadd_rn(gy, __fmul_rn(__fsub_rn(alpha, __fmul_rn(c, g)), s.m));
+    }
+    __device__ __forceinline__ void end_tile(State &) const {}
+    __device__ __forceinline__ void finish(State &, int64_t) const {}
+};
+
 // ---------------------------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------------------------
@@ -964,6 +1022,43 @@ EXODUS_API int exodus_synlif_backward(float *grad_input, float *alpha_mem_grad, 
         default: return hipErrorInvalidValue;
     }
 #undef EXODUS_SYN
+}
+
+EXODUS_API int exodus_spike_forward(float *out_spikes, float *vmem, float alpha, float membr_subtract, float theta,
+                                    float theta_low, int apply_theta_low, int max_num_spikes, int64_t n, int64_t t,
+                                    void *stream)
+{
+    if (bad_dims(n, t)) return hipErrorInvalidValue;
+    if (n == 0 || t == 0) return hipSuccess;
+    if (!out_spikes || !vmem) return hipErrorInvalidValue;
+    SpikeFwdOp op;
+    op.in[0] = vmem;
+    op.out[0] = vmem;
+    op.der = out_spikes;
+    op.alpha = alpha;
+    op.c = membr_subtract;
+    op.theta = theta;
+    op.theta_low = theta_low;
+    op.apply_low = apply_theta_low ? 1 : 0;
+    op.cap = static_cast<unsigned>(max_num_spikes);           // negative -> no cap
+    return launch<SpikeFwdOp, EXODUS_TT_1>(op, n, t, stream);
+}
+
+EXODUS_API int exodus_spike_backward(float *input_grad, const float *surr, const float *output_grad,
+                                     const float *not_clipped, float alpha, float membr_subtract, int64_t n,
+                                     int64_t t, void *stream)
+{
+    if (bad_dims(n, t)) return hipErrorInvalidValue;
+    if (n == 0 || t == 0) return hipSuccess;
+    if (!input_grad || !surr || !output_grad || !not_clipped) return hipErrorInvalidValue;
+    SpikeBwdOp op;
+    op.in[0] = output_grad;
+    op.in[1] = surr;
+    op.in[2] = not_clipped;
+    op.out[0] = input_grad;
+    op.alpha = alpha;
+    op.c = membr_subtract;
+    return launch<SpikeBwdOp, EXODUS_TT_3>(op, n, t, stream);
 }
 
 }  // extern "C"

@@ -41,6 +41,8 @@ _SIGNATURES = {
     "exodus_lif_backward_fused": ([_p] * 12 + [_int, _int, _int, _f, _f, _i64, _i64, _p], _int),
     "exodus_synlif_forward": ([_p] * 11 + [_int, _int, _int, _int, _i64, _i64, _p], _int),
     "exodus_synlif_backward": ([_p] * 17 + [_int, _int, _int, _int, _int, _f, _f, _i64, _i64, _p], _int),
+    "exodus_spike_forward": ([_p, _p, _f, _f, _f, _f, _int, _int, _i64, _i64, _p], _int),
+    "exodus_spike_backward": ([_p] * 4 + [_f, _f, _i64, _i64, _p], _int),
     "exodus_layer_checkpoint_interval": ([], _int),
     "exodus_layer_lif_forward": ([_p] * 16 + [_int, _int, _int, _int, _i64, _i64, _i64, _p], _int),
     "exodus_layer_lif_backward": ([_p] * 18 + [_int, _int, _int, _int, _int, _f, _f, _i64, _i64, _i64, _p], _int),
@@ -222,6 +224,38 @@ def leakyBackwardAlpha(outputGrad, output, vmemInitial, alpha) -> torch.Tensor:
                                                _ptr(vmemInitial), _ptr(alpha), n, t, _stream(outputGrad)),
                "exodus_leaky_backward_alpha")
     return alphaGrad
+
+
+def spikeForward(vmem, alpha: float, membrSubtract: float, theta: float, thetaLow: float, applyThetaLow: bool,
+                 maxNumSpikes: int) -> torch.Tensor:
+    """reference cuda/bindings.cu:262-290 (experimental): ``vmem`` (rows, time) is corrected in place
+    for resets and lower bound, the spike raster is returned."""
+    _dev(vmem, "vmem")
+    if vmem.ndim != 2:
+        raise RuntimeError("vmem must be 2-D (rows, time)")
+    n, t = vmem.shape
+    spikes = torch.empty_like(vmem)
+    with torch.cuda.device(vmem.device):
+        _check(lib.exodus_spike_forward(_ptr(spikes), _ptr(vmem), float(alpha), float(membrSubtract), float(theta),
+                                        float(thetaLow), int(bool(applyThetaLow)), int(maxNumSpikes), n, t,
+                                        _stream(vmem)), "exodus_spike_forward")
+    return spikes
+
+
+def spikeBackward(surr, outputGrad, notClipped, alpha: float, membrSubtract: float) -> torch.Tensor:
+    """reference cuda/bindings.cu:327-359 (experimental)."""
+    _dev(surr, "surr")
+    if surr.ndim != 2:
+        raise RuntimeError("surr must be 2-D (rows, time)")
+    n, t = surr.shape
+    _mat(_dev(outputGrad, "outputGrad", surr), "outputGrad", n, t)
+    _mat(_dev(notClipped, "notClipped", surr), "notClipped", n, t)
+    inputGrad = torch.empty_like(surr)
+    with torch.cuda.device(surr.device):
+        _check(lib.exodus_spike_backward(_ptr(inputGrad), _ptr(surr), _ptr(outputGrad), _ptr(notClipped),
+                                         float(alpha), float(membrSubtract), n, t, _stream(surr)),
+               "exodus_spike_backward")
+    return inputGrad
 
 
 # ------------------------------------------------------------------------------------------

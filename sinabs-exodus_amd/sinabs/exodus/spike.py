@@ -142,3 +142,68 @@ class IntegrateAndFire(torch.autograd.Function):
         # grad_init back-propagates one more decay step from the first time point
         # (d v_0 / d v_init = alpha, the reset on v_init is applied by the caller).
         return (grad_input, grad_alpha, grad_init, None, None, None, None, None)
+
+
+class SpikeFunction(torch.autograd.Function):
+    """Experimental: spikes from a membrane potential that already contains the response to the
+    input; resets and lower bound are applied to ``v_mem`` in place
+    (reference sinabs/exodus/spike.py:7-104).  ``IntegrateAndFire`` is the faster option.
+
+    Arguments as in the reference: ``v_mem`` (N, T) contiguous, scalar ``membrane_subtract``,
+    ``alpha``, ``threshold``, optional scalar ``min_v_mem``, optional ``max_num_spikes_per_bin``.
+    Returns ``(spikes, v_mem)``.  One deliberate difference: the reference hands ``threshold``
+    to the kernel where the lower bound belongs (spike.py:63); here ``min_v_mem`` is the bound.
+    """
+
+    @staticmethod
+    def forward(
+        ctx,
+        v_mem: torch.Tensor,
+        membrane_subtract: float,
+        alpha: float,
+        surrogate_grad_fn: Callable,
+        threshold: float,
+        min_v_mem: Optional[float] = None,
+        max_num_spikes_per_bin: Optional[int] = None,
+    ):
+        if not v_mem.is_contiguous():
+            raise ValueError("'v_mem' has to be contiguous.")
+        if not v_mem.ndim == 2:
+            raise ValueError("'v_mem' must be 2D, (N, Time)")
+        scalar = lambda v: float(v.item()) if isinstance(v, torch.Tensor) else float(v)
+        threshold, alpha, membrane_subtract = scalar(threshold), scalar(alpha), scalar(membrane_subtract)
+        min_v_mem = None if min_v_mem is None else scalar(min_v_mem)
+        if min_v_mem is not None and threshold <= min_v_mem:
+            raise ValueError("`threshold` must be greater than `min_v_mem`.")
+
+        spikes = _hip.spikeForward(
+            v_mem, alpha, membrane_subtract, threshold,
+            0.0 if min_v_mem is None else min_v_mem,
+            min_v_mem is not None,
+            -1 if max_num_spikes_per_bin is None else max_num_spikes_per_bin,
+        )
+        ctx.alpha = alpha
+        ctx.threshold = threshold
+        ctx.min_v_mem = min_v_mem
+        ctx.membrane_subtract = membrane_subtract
+        ctx.surrogate_grad_fn = surrogate_grad_fn
+        ctx.save_for_backward(v_mem)
+        return spikes, v_mem
+
+    @staticmethod
+    def backward(ctx, grad_output, grad_v_mem):
+        if grad_v_mem is not None and torch.count_nonzero(grad_v_mem) > 0:
+            raise NotImplementedError(
+                "Direct Backpropagation through membrane potential is currently not supported."
+            )
+        (v_mem,) = ctx.saved_tensors
+        surrogates = ctx.surrogate_grad_fn(v_mem, ctx.threshold)
+        if ctx.min_v_mem is None:
+            not_clipped = torch.ones_like(surrogates)
+        else:
+            not_clipped = (v_mem > ctx.min_v_mem).float()
+        grad_input = _hip.spikeBackward(
+            surrogates.contiguous(), grad_output.contiguous(), not_clipped.contiguous(),
+            ctx.alpha, ctx.membrane_subtract,
+        )
+        return grad_input, None, None, None, None, None, None

@@ -316,3 +316,72 @@ def test_surrogate_closed_values():
     assert torch.allclose(ref.PeriodicExponential()(torch.tensor([[2.0]]), torch.tensor([[1.0]])), torch.tensor([[1.0]]))
     assert torch.allclose(ref.PeriodicExponential()(torch.tensor([[1.5]]), torch.tensor([[1.0]])),
                           ref.PeriodicExponential()(torch.tensor([[0.5]]), torch.tensor([[1.0]])))
+
+
+# ------------------------------------------------------------------ experimental spike generation
+def test_spike_forward_notebook_known_answer(kat):
+    """The notebook's neuron (alpha = 1) seen from the other side: its potential without resets is
+    cumsum(input); spike generation on that must give the notebook's spikes and potentials."""
+    case = kat["cases"][0]
+    u = f32([kat["input"]]).cumsum(1).contiguous()
+    s = ref.spike_forward(u, 1.0, case["membrane_subtract"], kat["threshold"], 0.0, False, -1)
+    assert s[0].tolist() == case["spikes"]
+    np.testing.assert_allclose(u[0].numpy(), case["v_mem_pre_reset"], atol=case["v_mem_abs_tol"])
+
+
+@pytest.mark.parametrize("use_lo,cap", [(False, -1), (True, -1), (True, 2), (False, 1)])
+def test_spike_forward_equals_lif_forward_on_dyadic_grid(use_lo, cap):
+    """alpha = 1/2, inputs on a 1/64 grid, few steps: every product and sum below is exact in
+    float32, so "leaky integral, then spike generation" and the LIF recurrence must agree to the
+    bit although they order the arithmetic differently.  A clamped step keeps its own value in the
+    spike function (only later steps are raised), hence the max()."""
+    g = torch.Generator().manual_seed(17 + cap)
+    n, t, a, th, c, lo = 64, 9, 0.5, 1.0, 0.75, -0.5
+    x = (torch.randint(-96, 192, (n, t), generator=g).float() / 64.0).contiguous()
+    ones = torch.ones(n)
+    u = ref.leaky_forward(x, torch.zeros(n), a * ones)
+    s_exp = ref.spike_forward(u, a, c, th, lo, use_lo, cap)
+    s_lif, v_lif = ref.lif_forward(x, torch.zeros(n), a * ones, c * ones, th * ones, lo * ones, use_lo, cap)
+    assert s_lif.sum() > 50 and (not use_lo or (u < lo).any())
+    assert torch.equal(s_exp, s_lif)
+    assert torch.equal(torch.clamp(u, min=lo) if use_lo else u, v_lif)
+
+
+def test_spike_backward_notebook_known_answers(kat):
+    """alpha = 1, nothing clipped: the gradient with respect to the input current is the leaky
+    adjoint (reverse cumulative sum) of the gradient with respect to the potential."""
+    th = kat["threshold"]
+    for case in kat["cases"]:
+        surr = torch.full((1, 5), 1.0 / th)
+        go = torch.zeros(1, 5); go[0, -1] = 1.0
+        gu = ref.spike_backward(surr, go, torch.ones(1, 5), 1.0, case["membrane_subtract"])
+        gi = ref.leaky_backward(gu, f32([1.0]))
+        np.testing.assert_allclose(gi[0].numpy(), case["grad_of_last_spike_wrt_input"],
+                                   rtol=case["grad_rel_tol"], atol=2e-7)
+
+
+def test_spike_backward_alpha_one_equals_production_backward():
+    surr, gg, _, _, _ = _random_backward_case(5, clip=False)
+    surr = surr * 0.8
+    n, t = surr.shape
+    ones = torch.ones(n)
+    gu = ref.spike_backward(surr, gg, torch.ones(n, t), 1.0, 0.7)
+    got = ref.leaky_backward(gu, ones)
+    want = ref.lif_backward(surr, (surr * gg).contiguous(), torch.ones(n, t), ones, 0.7 * ones)
+    np.testing.assert_allclose(got.numpy(), want.numpy(), rtol=2e-5, atol=2e-6)
+
+
+@pytest.mark.parametrize("alpha", [1.0, 0.8])
+def test_spike_backward_quadratic_sum_equals_reverse_recurrence(alpha):
+    """Two different algorithms for the same vector (the only check for alpha != 1 and for
+    clipped steps, where no known answer of the reference exists)."""
+    surr, gg, nc, _, _ = _random_backward_case(8)
+    c = 0.6
+    got = ref.spike_backward(surr, gg, nc, alpha, c).double()
+    y = (surr * nc).double(); go = gg.double()
+    m = torch.zeros(surr.shape[0], dtype=torch.float64)
+    want = torch.zeros_like(go)
+    for i in range(surr.shape[1] - 1, -1, -1):
+        want[:, i] = y[:, i] * go[:, i] - y[:, i] * c * m
+        m = go[:, i] * y[:, i] + (alpha - c * y[:, i]) * m
+    np.testing.assert_allclose(got.numpy(), want.numpy(), rtol=1e-4, atol=1e-5)
