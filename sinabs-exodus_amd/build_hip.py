@@ -7,6 +7,7 @@ import os
 import shutil
 import subprocess
 import sys
+import tempfile
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 SRCS = [os.path.join(HERE, "csrc", f) for f in ("exodus_hip.hip", "exodus_layer.hip")]
@@ -28,16 +29,29 @@ def build(force: bool = True) -> str:
     if not force and os.path.exists(OUT) and os.path.getmtime(OUT) >= max(os.path.getmtime(d) for d in deps):
         return OUT
     hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
-    cmd = [hipcc] + FLAGS + ["-I", INCLUDE, "-o", OUT + ".tmp"] + SRCS
-    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     # hipcc's host pass does not know the gfx-only target feature and says so; that line is harmless
     noise = "packed-fp32-ops"
-    out = "\n".join(l for l in proc.stdout.splitlines() if noise not in l)
-    if proc.returncode != 0:
-        sys.stderr.write(out + "\n")
-        raise RuntimeError("hipcc failed building libexodus_hip.so")
-    if out.strip():
-        sys.stderr.write(out + "\n")
+    quiet = lambda text: "\n".join(l for l in text.splitlines() if noise not in l)
+    compile_flags = [f for f in FLAGS if f != "-shared"]
+    with tempfile.TemporaryDirectory() as tmp:
+        # one hipcc process per translation unit, side by side, then one link
+        objs = [os.path.join(tmp, os.path.basename(src) + ".o") for src in SRCS]
+        procs = [subprocess.Popen([hipcc] + compile_flags + ["-I", INCLUDE, "-c", src, "-o", obj],
+                                  stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+                 for src, obj in zip(SRCS, objs)]
+        outputs = [proc.communicate()[0] for proc in procs]
+        log = "\n".join(filter(None, (quiet(o).strip() for o in outputs)))
+        if any(proc.returncode != 0 for proc in procs):
+            sys.stderr.write(log + "\n")
+            raise RuntimeError("hipcc failed compiling libexodus_hip.so")
+        link = subprocess.run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", OUT + ".tmp"] + objs,
+                              stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+        log = "\n".join(filter(None, (log, quiet(link.stdout).strip())))
+        if link.returncode != 0:
+            sys.stderr.write(log + "\n")
+            raise RuntimeError("hipcc failed linking libexodus_hip.so")
+    if log.strip():
+        sys.stderr.write(log + "\n")
     os.replace(OUT + ".tmp", OUT)
     return OUT
 

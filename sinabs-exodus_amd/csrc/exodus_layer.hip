@@ -18,6 +18,7 @@
 #include <stdint.h>
 
 #include <initializer_list>
+#include <type_traits>
 
 #include "exodus_common.hpp"
 
@@ -57,58 +58,165 @@ template <> __device__ __forceinline__ void lane_put<1>(float &v, int, float x) 
 template <> __device__ __forceinline__ void lane_put<2>(f32x2 &v, int e, float x) { v[e] = x; }
 template <> __device__ __forceinline__ void lane_put<4>(f32x4 &v, int e, float x) { v[e] = x; }
 
-// per-neuron constants and running state of the forward recurrence
-struct Neuron {
-    float am, as, k, c, th, lo;     // decay factors, 1 - alpha_mem, subtract value, threshold, lower bound
-    float vpost, i;                 // potential after the reset of the previous step, synaptic current
+// ---------------------------------------------------------------------------------------------
+// memory access: raw buffer instructions
+// ---------------------------------------------------------------------------------------------
+// Every (batch, time, neurons) access of a block has the form
+//     block-uniform base (SGPR pair inside a buffer resource)  +  step * neurons * 4 (SGPR)
+//                                                              +  lane offset (one VGPR, loop-invariant)
+// which is exactly what a buffer instruction adds up by itself, so no access needs vector
+// arithmetic or 64-bit address registers.  num_records is set to the maximum: every access is
+// guarded by the code, not by the hardware range check.
+typedef __amdgpu_buffer_rsrc_t Rsrc;
+constexpr int AUX_LOAD = EXODUS_NT_LOAD ? 2 : 0;     // bit 1 = non-temporal
+constexpr int AUX_STORE = EXODUS_NT_STORE ? 2 : 0;
+
+__device__ __forceinline__ Rsrc make_rsrc(const float *base)
+{
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(base), 0, -1, 0x00020000);
+}
+
+typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+
+template <int NPL> struct BufIO;
+template <> struct BufIO<1> {
+    static __device__ __forceinline__ float load(Rsrc r, unsigned voff, unsigned soff)
+    {
+        return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, AUX_LOAD));
+    }
+    static __device__ __forceinline__ void store(float v, Rsrc r, unsigned voff, unsigned soff)
+    {
+        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), r, voff, soff, AUX_STORE);
+    }
+};
+template <> struct BufIO<2> {
+    static __device__ __forceinline__ f32x2 load(Rsrc r, unsigned voff, unsigned soff)
+    {
+        return __builtin_bit_cast(f32x2, __builtin_amdgcn_raw_buffer_load_b64(r, voff, soff, AUX_LOAD));
+    }
+    static __device__ __forceinline__ void store(f32x2 v, Rsrc r, unsigned voff, unsigned soff)
+    {
+        __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(u32x2, v), r, voff, soff, AUX_STORE);
+    }
+};
+template <> struct BufIO<4> {
+    static __device__ __forceinline__ f32x4 load(Rsrc r, unsigned voff, unsigned soff)
+    {
+        return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, AUX_LOAD));
+    }
+    static __device__ __forceinline__ void store(f32x4 v, Rsrc r, unsigned voff, unsigned soff)
+    {
+        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), r, voff, soff, AUX_STORE);
+    }
 };
 
-template <bool SYN>
+// ---------------------------------------------------------------------------------------------
+// one neuron
+// ---------------------------------------------------------------------------------------------
+// Per-neuron constants and running state.  The layer's options are folded into the constants so
+// that the step itself has no option-dependent code: a factor that an option switches off is 1
+// (multiplying by 1 is exact), a bound that is switched off is an infinity.
+struct Neuron {
+    float am, as;       // decay factors of membrane and synapse
+    float k;            // factor on the current entering the membrane: 1 - alpha_mem (norm_input) or 1
+    float xs;           // factor on the input entering the synapse: alpha_syn (decay_early) or 1
+    float c, th;        // subtract value, threshold
+    float th2;          // 2 * threshold: from here on a second spike (+inf where th <= 0)
+    float thd;          // from here on the spike count needs the quotient v / th (+inf if never)
+    float lo;           // lower bound of the potential, -inf without one
+    float vpost, i;     // potential after the reset of the previous step, synaptic current
+};
+
+// spike-count cap as the kernels use it (block-uniform)
+struct Cap {
+    float one, two;     // min(cap, 1), min(cap, 2)
+    unsigned cap;
+};
+
+// CAPK: 1 = at most one spike per step, 2 = at most two, 0 = any other cap (none, 0, >= 3)
+template <bool SYN, int CAPK>
 __device__ __forceinline__ void neuron_load(Neuron &n, const LayerConsts &p, int64_t row)
 {
     n.am = p.alpha_mem[row];
     n.as = SYN ? p.alpha_syn[row] : 0.f;
-    n.k = __fsub_rn(1.0f, n.am);
+    n.k = p.norm_input ? __fsub_rn(1.0f, n.am) : 1.0f;
+    n.xs = (SYN && p.decay_early) ? n.as : 1.0f;
     n.c = p.c[row];
     n.th = p.theta[row];
-    n.lo = p.apply_low ? p.theta_low[row] : 0.f;
+    // For th > 0:  v >= th <=> RN(v/th) >= 1  and  v >= 2 th <=> RN(v/th) >= 2  (2 th is exact and no
+    // float lies between its predecessor and the rounding boundary of the quotient), so counts up to
+    // 2 need no division.  Everything else -- more than two spikes, or a threshold that is not
+    // positive -- takes the quotient.
+    const bool plain = n.th > 0.f;
+    n.th2 = plain ? __fadd_rn(n.th, n.th) : __builtin_inff();
+    n.thd = plain ? (CAPK == 0 ? n.th2 : __builtin_inff()) : n.th;
+    n.lo = p.apply_low ? p.theta_low[row] : -__builtin_inff();
 }
 
-// One step of the layer's forward arithmetic, in the order the composed layer performs it
-// (input scaling, synapse, input normalisation, membrane, clamp, threshold):
-//   xin = decay_early ? x * a_syn : x;  i = i * a_syn + xin   (SYN; otherwise i = x)
-//   u = norm_input ? (1 - a_mem) * i : i;   v = vpost * a_mem + u;   clamp;   count from v
-// Returns the pre-reset potential v; `count` is the spike count; n.vpost / n.i are advanced.
+// Advance synapse and membrane by one step, in the order the composed layer does it
+// (input scaling, synapse, input normalisation, membrane, clamp):
+//   xin = x * xs;  i = i * a_syn + xin   (SYN; otherwise i = x)
+//   u = k * i;   v = vpost * a_mem + u;   v = max(v, lo)
+// Returns the pre-reset potential v; n.i is advanced, n.vpost is left to the caller (it needs the
+// spike count).
 template <bool SYN>
-__device__ __forceinline__ float neuron_step(Neuron &n, const LayerConsts &p, float x, float &count)
+__device__ __forceinline__ float neuron_advance(Neuron &n, float x)
 {
     if (SYN) {
-        const float xin = p.decay_early ? __fmul_rn(x, n.as) : x;
+        const float xin = __fmul_rn(x, n.xs);
         n.i = __fadd_rn(__fmul_rn(n.i, n.as), xin);
     } else {
         n.i = x;
     }
-    const float u = p.norm_input ? __fmul_rn(n.k, n.i) : n.i;
-    float v = __fadd_rn(__fmul_rn(n.vpost, n.am), u);
-    if (p.apply_low && v < n.lo) v = n.lo;
-    count = spike_count(v, n.th, p.cap);
-    n.vpost = __fsub_rn(v, __fmul_rn(count, n.c));
-    return v;
+    const float u = __fmul_rn(n.k, n.i);
+    const float v = __fadd_rn(__fmul_rn(n.vpost, n.am), u);
+    return v < n.lo ? n.lo : v;
+}
+
+// count = v >= th ? min(unsigned(v / th), cap) : 0   (IEEE division, truncation), in two parts:
+// the count by comparisons, and the quotient for the rare potentials at or above n.thd.
+template <int CAPK>
+__device__ __forceinline__ float count_by_compare(float v, const Neuron &n, const Cap &cc)
+{
+    const float count = v >= n.th ? (CAPK == 0 ? cc.one : 1.f) : 0.f;
+    if (CAPK == 1) return count;
+    return v >= n.th2 ? (CAPK == 0 ? cc.two : 2.f) : count;
+}
+
+__device__ __forceinline__ float count_by_quotient(float v, const Neuron &n, const Cap &cc)
+{
+    const unsigned q = static_cast<unsigned>(__fdiv_rn(v, n.th));
+    return static_cast<float>(q < cc.cap ? q : cc.cap);
+}
+
+template <int CAPK>
+__device__ __forceinline__ float spike_count_fast(float v, const Neuron &n, const Cap &cc)
+{
+    float count = count_by_compare<CAPK>(v, n, cc);
+    if (v >= n.thd) count = count_by_quotient(v, n, cc);
+    return count;
 }
 
 // ---------------------------------------------------------------------------------------------
 // forward
 // ---------------------------------------------------------------------------------------------
-template <bool SYN, int NPL>
+// Time is walked in blocks of CKPT = 2 * FWD_UNROLL steps.  Two register buffers of FWD_UNROLL
+// steps alternate: while one is consumed the loads of the other are in flight.  Every fetch issues
+// the same number of loads (the last round re-reads its own block), so the number of outstanding
+// loads at each wait is a compile-time constant.  Steps beyond the last full block run through a
+// guarded copy of the same code.
+template <bool SYN, int NPL, int CAPK, bool REC>
 __global__ void __launch_bounds__(BLOCK) layer_lif_forward(
     float *__restrict__ spikes, float *__restrict__ v_rec, float *__restrict__ i_rec, float *__restrict__ ckpt_v,
     float *__restrict__ ckpt_i, float *__restrict__ v_last, float *__restrict__ i_last, double *spike_sum,
     const float *__restrict__ x, const LayerConsts p, const int64_t blocks_per_batch, const int64_t T,
     const int64_t M)
 {
+    static_assert(2 * FWD_UNROLL == CKPT, "two pipeline stages per checkpoint interval");
     typedef typename Vec<NPL>::type V;
-    // A block works inside one batch element: block-uniform base pointers plus a small lane offset,
-    // so that addresses cost scalar registers only.
+    typedef BufIO<NPL> IO;
+    // A block works inside one batch element, so all bases are block-uniform.
     const int64_t b = blockIdx.x / blocks_per_batch;
     const int64_t m0 = static_cast<int64_t>(blockIdx.x - b * blocks_per_batch) * (BLOCK * NPL);
     const unsigned lane_off = threadIdx.x * NPL;
@@ -118,64 +226,105 @@ __global__ void __launch_bounds__(BLOCK) layer_lif_forward(
         const int64_t n_ck = (T + CKPT - 1) / CKPT;
         const float *xp = x + (b * T) * M + m0;
         float *sp = spikes + (b * T) * M + m0;
-        float *vrp = v_rec ? v_rec + (b * T) * M + m0 : nullptr;
-        float *irp = i_rec ? i_rec + (b * T) * M + m0 : nullptr;
+        float *vrp = REC && v_rec ? v_rec + (b * T) * M + m0 : nullptr;
+        float *irp = REC && i_rec ? i_rec + (b * T) * M + m0 : nullptr;
         float *cvp = ckpt_v ? ckpt_v + (b * n_ck) * M + m0 : nullptr;
         float *cip = (SYN && ckpt_i) ? ckpt_i + (b * n_ck) * M + m0 : nullptr;
+        const unsigned voff = lane_off * 4u;                  // byte offset of this lane within a step
+        const unsigned step_bytes = static_cast<unsigned>(M) * 4u;   // the host keeps CKPT * M * 4 below 2^32
 
+        Cap cc;
+        cc.cap = p.cap;
+        cc.one = p.cap >= 1u ? 1.f : 0.f;
+        cc.two = p.cap >= 2u ? 2.f : cc.one;
         Neuron nr[NPL];
 #pragma unroll
         for (int e = 0; e < NPL; ++e) {
-            neuron_load<SYN>(nr[e], p, first + e);
+            neuron_load<SYN, CAPK>(nr[e], p, first + e);
             nr[e].vpost = p.v_init[first + e];
             nr[e].i = SYN ? p.i_init[first + e] : 0.f;
         }
 
-        V cur[FWD_UNROLL], nxt[FWD_UNROLL];
-        auto fetch = [&](V(&dst)[FWD_UNROLL], int64_t t0) {
+        V bufa[FWD_UNROLL], bufb[FWD_UNROLL];
+        auto fetch = [&](V(&dst)[FWD_UNROLL], int64_t t0) {  // FWD_UNROLL full steps from t0
+            const Rsrc r = make_rsrc(xp + t0 * M);
 #pragma unroll
-            for (int u = 0; u < FWD_UNROLL; ++u)
-                if (t0 + u < T) dst[u] = ld_stream(reinterpret_cast<const V *>(xp + (t0 + u) * M + lane_off));
+            for (int u = 0; u < FWD_UNROLL; ++u) dst[u] = IO::load(r, voff, u * step_bytes);
         };
-        fetch(cur, 0);
-        float part = 0.f;                                     // spike count of the current chunk (exact in fp32)
-        for (int64_t t0 = 0; t0 < T; t0 += FWD_UNROLL) {
-            if (t0 + FWD_UNROLL < T) fetch(nxt, t0 + FWD_UNROLL);
-            if ((t0 % CKPT) == 0) {
-                if (cvp) {
-                    V cv, ci;
+        auto fetch_tail = [&](V(&dst)[FWD_UNROLL], int64_t t0) {   // steps past the end re-read the last one
+            const Rsrc r = make_rsrc(xp + t0 * M);
+            const unsigned last = static_cast<unsigned>(T - 1 - t0);
 #pragma unroll
-                    for (int e = 0; e < NPL; ++e) {
-                        lane_put<NPL>(cv, e, nr[e].vpost);
-                        lane_put<NPL>(ci, e, nr[e].i);
-                    }
-                    st_stream(cv, reinterpret_cast<V *>(cvp + (t0 / CKPT) * M + lane_off));
-                    if (cip) st_stream(ci, reinterpret_cast<V *>(cip + (t0 / CKPT) * M + lane_off));
+            for (int u = 0; u < FWD_UNROLL; ++u) dst[u] = IO::load(r, voff, (u < last ? u : last) * step_bytes);
+        };
+        float part = 0.f;                                     // spike count since the last checkpoint (exact in fp32)
+        auto checkpoint = [&](int64_t j) {
+            if (cvp) {
+                V cv, ci;
+#pragma unroll
+                for (int e = 0; e < NPL; ++e) {
+                    lane_put<NPL>(cv, e, nr[e].vpost);
+                    lane_put<NPL>(ci, e, nr[e].i);
                 }
-                my_spikes += static_cast<double>(part);
-                part = 0.f;
+                st_stream(cv, reinterpret_cast<V *>(cvp + j * M + lane_off));
+                if (cip) st_stream(ci, reinterpret_cast<V *>(cip + j * M + lane_off));
             }
+            my_spikes += static_cast<double>(part);
+            part = 0.f;
+        };
+        auto compute = [&](const V(&buf)[FWD_UNROLL], int64_t t0, auto guard) {
+            constexpr bool GUARD = decltype(guard)::value;
+            const Rsrc rs = make_rsrc(sp + t0 * M);
+            const Rsrc rv = make_rsrc(REC ? vrp + t0 * M : nullptr);
+            const Rsrc ri = make_rsrc(REC ? irp + t0 * M : nullptr);
 #pragma unroll
             for (int u = 0; u < FWD_UNROLL; ++u) {
-                const int64_t t = t0 + u;
-                if (t < T) {
+                if (!GUARD || t0 + u < T) {
                     V s, vr, ir;
+                    float v[NPL], count[NPL];
+                    bool rare = false;                        // one branch per step for all neurons of the lane
 #pragma unroll
                     for (int e = 0; e < NPL; ++e) {
-                        float count;
-                        neuron_step<SYN>(nr[e], p, lane_get<NPL>(cur[u], e), count);
-                        lane_put<NPL>(s, e, count);
+                        v[e] = neuron_advance<SYN>(nr[e], lane_get<NPL>(buf[u], e));
+                        count[e] = count_by_compare<CAPK>(v[e], nr[e], cc);
+                        rare = rare | (v[e] >= nr[e].thd);
+                    }
+                    if (rare) {
+#pragma unroll
+                        for (int e = 0; e < NPL; ++e)
+                            if (v[e] >= nr[e].thd) count[e] = count_by_quotient(v[e], nr[e], cc);
+                    }
+#pragma unroll
+                    for (int e = 0; e < NPL; ++e) {
+                        nr[e].vpost = __fsub_rn(v[e], __fmul_rn(count[e], nr[e].c));
+                        part += count[e];
+                        lane_put<NPL>(s, e, count[e]);
                         lane_put<NPL>(vr, e, nr[e].vpost);
                         lane_put<NPL>(ir, e, nr[e].i);
-                        part += count;
                     }
-                    st_stream(s, reinterpret_cast<V *>(sp + t * M + lane_off));
-                    if (vrp) st_stream(vr, reinterpret_cast<V *>(vrp + t * M + lane_off));
-                    if (irp) st_stream(ir, reinterpret_cast<V *>(irp + t * M + lane_off));
+                    IO::store(s, rs, voff, u * step_bytes);
+                    if (REC && vrp) IO::store(vr, rv, voff, u * step_bytes);
+                    if (REC && irp) IO::store(ir, ri, voff, u * step_bytes);
                 }
             }
-#pragma unroll
-            for (int u = 0; u < FWD_UNROLL; ++u) cur[u] = nxt[u];
+        };
+
+        const int64_t n_full = T / CKPT;                      // blocks of CKPT steps that lie inside the sequence
+        if (n_full > 0) fetch(bufa, 0);
+        for (int64_t j = 0; j < n_full; ++j) {
+            const int64_t t0 = j * CKPT;
+            fetch(bufb, t0 + FWD_UNROLL);
+            checkpoint(j);
+            compute(bufa, t0, std::false_type{});
+            fetch(bufa, j + 1 < n_full ? t0 + CKPT : t0);
+            compute(bufb, t0 + FWD_UNROLL, std::false_type{});
+        }
+        if (n_full * CKPT < T) {
+            checkpoint(n_full);
+            for (int64_t t0 = n_full * CKPT; t0 < T; t0 += FWD_UNROLL) {
+                fetch_tail(bufa, t0);
+                compute(bufa, t0, std::true_type{});
+            }
         }
         my_spikes += static_cast<double>(part);
 #pragma unroll
@@ -207,7 +356,7 @@ __global__ void __launch_bounds__(BLOCK) layer_lif_forward(
 // The final potential handed out by the forward is vpost_{T-1} = v_{T-1} - c count_{T-1}; a gradient
 // gv on it reaches v_{T-1} directly and the spike count with weight -c, a gradient on the final
 // synaptic current adds to mu_{T-1}.
-template <bool SYN, int KIND>
+template <bool SYN, int KIND, int CAPK>
 __global__ void __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(EXODUS_LAYER_BWD_WAVES, EXODUS_LAYER_BWD_WAVES)))
 layer_lif_backward(
     float *__restrict__ grad_x, float *__restrict__ alpha_mem_grad, float *__restrict__ alpha_syn_grad,
@@ -216,23 +365,30 @@ layer_lif_backward(
     const float *__restrict__ ckpt_v, const float *__restrict__ ckpt_i, const LayerConsts p, const float p0,
     const float p1, const float inv_p0, const int64_t blocks_per_batch, const int64_t T, const int64_t M)
 {
+    typedef BufIO<1> IO;
     const int64_t b = blockIdx.x / blocks_per_batch;
     const int64_t m0 = static_cast<int64_t>(blockIdx.x - b * blocks_per_batch) * BLOCK;
     const unsigned lane_off = threadIdx.x;
     if (m0 + lane_off >= M) return;
     const int64_t row = b * M + m0 + lane_off;
     const int64_t n_ck = (T + CKPT - 1) / CKPT;
-    // block-uniform bases; the lane offset is added at each access
+    // block-uniform bases; lane and step offsets are added by the buffer instructions
     const float *xp = x + (b * T) * M + m0;
     const float *gp = grad_spikes + (b * T) * M + m0;
     float *op = grad_x + (b * T) * M + m0;
     const float *cvp = ckpt_v + (b * n_ck) * M + m0;
     const float *cip = SYN ? ckpt_i + (b * n_ck) * M + m0 : nullptr;
+    const unsigned voff = lane_off * 4u;
+    const unsigned step_bytes = static_cast<unsigned>(M) * 4u;
 
+    Cap cc;
+    cc.cap = p.cap;
+    cc.one = p.cap >= 1u ? 1.f : 0.f;
+    cc.two = p.cap >= 2u ? 2.f : cc.one;
     Neuron nr;
-    neuron_load<SYN>(nr, p, row);
+    neuron_load<SYN, CAPK>(nr, p, row);
     const float amc = __fmul_rn(nr.am, nr.c);
-    const float kk = p.norm_input ? nr.k : 1.0f;
+    const float xg = (SYN && p.decay_early) ? nr.as : 1.0f;   // factor between mu and grad_x
     const SurrConst sk = surrogate_consts<KIND>(nr.th, p0, p1);
     const float gvl = grad_v_last ? grad_v_last[row] : 0.f;
     const float gil = (SYN && grad_i_last) ? grad_i_last[row] : 0.f;
@@ -246,22 +402,37 @@ layer_lif_backward(
         const int64_t t0 = j * CKPT;
         const int len = (T - t0) < CKPT ? static_cast<int>(T - t0) : CKPT;
         float xr[CKPT], gr[CKPT], vr[CKPT];
+        {
+            // always CKPT loads per tensor (in the one partial block, steps past the end re-read the
+            // last step): a constant number of loads in flight lets each use wait for its own load
+            const Rsrc rx = make_rsrc(xp + t0 * M), rg = make_rsrc(gp + t0 * M);
+            if (len == CKPT) {
 #pragma unroll
-        for (int k = 0; k < CKPT; ++k)
-            if (k < len) {
-                xr[k] = ld_stream(xp + (t0 + k) * M + lane_off);
-                gr[k] = ld_stream(gp + (t0 + k) * M + lane_off);
+                for (int k = 0; k < CKPT; ++k) {
+                    xr[k] = IO::load(rx, voff, k * step_bytes);
+                    gr[k] = IO::load(rg, voff, k * step_bytes);
+                }
+            } else {
+                const unsigned last = static_cast<unsigned>(len - 1);
+#pragma unroll
+                for (int k = 0; k < CKPT; ++k) {
+                    const unsigned so = (k < last ? k : last) * step_bytes;
+                    xr[k] = IO::load(rx, voff, so);
+                    gr[k] = IO::load(rg, voff, so);
+                }
             }
+        }
         nr.vpost = ld_stream(cvp + j * M + lane_off);
         nr.i = SYN ? ld_stream(cip + j * M + lane_off) : 0.f;
 
-        // rebuild the chunk: vr[k] = pre-reset potential, xr[k] = synaptic current (the value that
+        // rebuild the block: vr[k] = pre-reset potential, xr[k] = synaptic current (the value that
         // was normalised and fed to the membrane; without synapse that is the input itself)
 #pragma unroll
         for (int k = 0; k < CKPT; ++k)
             if (k < len) {
-                float count;
-                vr[k] = neuron_step<SYN>(nr, p, xr[k], count);
+                const float v = neuron_advance<SYN>(nr, xr[k]);
+                nr.vpost = __fsub_rn(v, __fmul_rn(spike_count_fast<CAPK>(v, nr, cc), nr.c));
+                vr[k] = v;
                 xr[k] = nr.i;
             }
 
@@ -278,27 +449,30 @@ layer_lif_backward(
                 } else {
                     g = __fmul_rn(sg, gr[k]);
                 }
-                const float vpost = __fsub_rn(v, __fmul_rn(nr.c, spike_count(v, nr.th, p.cap)));
+                const float vpost = __fsub_rn(v, __fmul_rn(nr.c, spike_count_fast<CAPK>(v, nr, cc)));
                 acc_m.add(lam, vpost);                          // lambda_{t+1} * vpost_t
                 if (SYN && !p.decay_early) acc_s.add(mu, cur_i);   // mu_{t+1} * i_t
                 const float f = __fsub_rn(nr.am, __fmul_rn(amc, sg));
                 const float l = __fadd_rn(g, __fmul_rn(f, lam));
-                lam = (p.apply_low && !(v > nr.lo)) ? 0.f : l;
+                lam = v > nr.lo ? l : 0.f;                      // clamped (or NaN) steps pass nothing on
                 if (p.norm_input) acc_m.sub(lam, cur_i);
-                float du = __fmul_rn(lam, kk);
+                float du = __fmul_rn(lam, nr.k);
                 if (SYN) {
                     if (t0 + k == T - 1) du = __fadd_rn(du, gil);
                     mu = __fadd_rn(__fmul_rn(mu, nr.as), du);
                     if (p.decay_early) acc_s.add(mu, cur_i);    // mu_t * i_t
-                    gr[k] = p.decay_early ? __fmul_rn(mu, nr.as) : mu;
+                    gr[k] = __fmul_rn(mu, xg);
                 } else {
                     gr[k] = du;
                 }
             }
         }
+        {
+            const Rsrc ro = make_rsrc(op + t0 * M);
 #pragma unroll
-        for (int k = 0; k < CKPT; ++k)
-            if (k < len) st_stream(gr[k], op + (t0 + k) * M + lane_off);
+            for (int k = 0; k < CKPT; ++k)
+                if (k < len) IO::store(gr[k], ro, voff, k * step_bytes);
+        }
         acc_m.fold();
         acc_s.fold();
     }
@@ -356,12 +530,14 @@ __global__ void __launch_bounds__(BLOCK) layer_leaky_forward(float *__restrict__
     V cur[LEAKY_UNROLL], nxt[LEAKY_UNROLL];
     auto fetch = [&](V(&dst)[LEAKY_UNROLL], int64_t t0) {
 #pragma unroll
-        for (int u = 0; u < LEAKY_UNROLL; ++u)
-            if (t0 + u < T) dst[u] = ld_stream(reinterpret_cast<const V *>(xp + (t0 + u) * M + lane_off));
+        for (int u = 0; u < LEAKY_UNROLL; ++u) {
+            const int64_t t = t0 + u < T ? t0 + u : T - 1;     // constant number of loads in flight
+            dst[u] = ld_stream(reinterpret_cast<const V *>(xp + t * M + lane_off));
+        }
     };
     fetch(cur, 0);
     for (int64_t t0 = 0; t0 < T; t0 += LEAKY_UNROLL) {
-        if (t0 + LEAKY_UNROLL < T) fetch(nxt, t0 + LEAKY_UNROLL);
+        fetch(nxt, t0 + LEAKY_UNROLL);
 #pragma unroll
         for (int u = 0; u < LEAKY_UNROLL; ++u) {
             if (t0 + u < T) {
@@ -418,12 +594,11 @@ __global__ void __launch_bounds__(BLOCK) layer_leaky_backward(
         V gv[LEAKY_UNROLL], ov[LEAKY_UNROLL], xv[LEAKY_UNROLL];
 #pragma unroll
         for (int u = 0; u < LEAKY_UNROLL; ++u) {
-            const int64_t t = t_hi - 1 - u;
-            if (t >= 0) {
-                gv[u] = ld_stream(reinterpret_cast<const V *>(gp + t * M + lane_off));
-                if (WITH_X) xv[u] = ld_stream(reinterpret_cast<const V *>(xp + t * M + lane_off));
-                if (ALPHA && t >= 1) ov[u] = ld_stream(reinterpret_cast<const V *>(outp + (t - 1) * M + lane_off));
-            }
+            // steps before the first re-read step 0: constant number of loads in flight
+            const int64_t t = t_hi - 1 - u >= 0 ? t_hi - 1 - u : 0;
+            gv[u] = ld_stream(reinterpret_cast<const V *>(gp + t * M + lane_off));
+            if (WITH_X) xv[u] = ld_stream(reinterpret_cast<const V *>(xp + t * M + lane_off));
+            if (ALPHA) ov[u] = ld_stream(reinterpret_cast<const V *>(outp + (t >= 1 ? t - 1 : 0) * M + lane_off));
         }
 #pragma unroll
         for (int u = 0; u < LEAKY_UNROLL; ++u) {
@@ -496,7 +671,7 @@ inline bool bad3(int64_t b, int64_t t, int64_t m)
     return (b * t) > INT64_MAX / m;
 }
 
-template <bool SYN, int KIND>
+template <bool SYN, int KIND, int CAPK>
 int launch_bwd(float *grad_x, float *am_g, float *as_g, float *v0_g, float *i0_g, const float *grad_spikes,
                const float *gvl, const float *gil, const float *x, const float *ckpt_v, const float *ckpt_i,
                const LayerConsts &p, float p0, float p1, int64_t B, int64_t T, int64_t M, hipStream_t s)
@@ -504,11 +679,61 @@ int launch_bwd(float *grad_x, float *am_g, float *as_g, float *v0_g, float *i0_g
     const int64_t blocks_per_batch = (M + BLOCK - 1) / BLOCK;
     if (blocks_per_batch > 0x7fffffffLL / B) return hipErrorInvalidValue;
     const int64_t blocks = blocks_per_batch * B;
-    hipLaunchKernelGGL((layer_lif_backward<SYN, KIND>), dim3(static_cast<unsigned>(blocks)), dim3(BLOCK), 0, s, grad_x,
-                       am_g, as_g, v0_g, i0_g, grad_spikes, gvl, gil, x, ckpt_v, ckpt_i, p, p0, p1,
+    hipLaunchKernelGGL((layer_lif_backward<SYN, KIND, CAPK>), dim3(static_cast<unsigned>(blocks)), dim3(BLOCK), 0, s,
+                       grad_x, am_g, as_g, v0_g, i0_g, grad_spikes, gvl, gil, x, ckpt_v, ckpt_i, p, p0, p1,
                        p0 != 0.f ? 1.f / p0 : 0.f, blocks_per_batch, T, M);
     return static_cast<int>(hipGetLastError());
 }
+
+template <bool SYN, int KIND, class... A>
+int dispatch_bwd_cap(unsigned cap, A... a)
+{
+    if (cap == 1u) return launch_bwd<SYN, KIND, 1>(a...);
+    if (cap == 2u) return launch_bwd<SYN, KIND, 2>(a...);
+    return launch_bwd<SYN, KIND, 0>(a...);
+}
+
+struct FwdArgs {
+    float *spikes, *v_rec, *i_rec, *ckpt_v, *ckpt_i, *v_last, *i_last;
+    double *spike_sum;
+    const float *x;
+    LayerConsts p;
+    int64_t B, T, M;
+    hipStream_t s;
+};
+
+template <bool SYN, int NPL, int CAPK, bool REC>
+int launch_fwd(const FwdArgs &a)
+{
+    const int64_t blocks_per_batch = (a.M + BLOCK * NPL - 1) / (BLOCK * NPL);
+    if (blocks_per_batch > 0x7fffffffLL / a.B) return hipErrorInvalidValue;
+    hipLaunchKernelGGL((layer_lif_forward<SYN, NPL, CAPK, REC>), dim3(static_cast<unsigned>(blocks_per_batch * a.B)),
+                       dim3(BLOCK), 0, a.s, a.spikes, a.v_rec, a.i_rec, a.ckpt_v, a.ckpt_i, a.v_last, a.i_last,
+                       a.spike_sum, a.x, a.p, blocks_per_batch, a.T, a.M);
+    return static_cast<int>(hipGetLastError());
+}
+
+// the specialisations for caps of one and two spikes exist for the layer's usual outputs only;
+// the general kernel serves every cap and also writes the per-step state records
+template <bool SYN, int NPL>
+int dispatch_fwd_cap(const FwdArgs &a)
+{
+    if (a.p.cap == 1u) return launch_fwd<SYN, NPL, 1, false>(a);
+    if (a.p.cap == 2u) return launch_fwd<SYN, NPL, 2, false>(a);
+    return launch_fwd<SYN, NPL, 0, false>(a);
+}
+
+template <bool SYN>
+int dispatch_fwd(const FwdArgs &a, int npl)
+{
+    if (a.v_rec || a.i_rec) return launch_fwd<SYN, 1, 0, true>(a);
+    if (npl == 4) return dispatch_fwd_cap<SYN, 4>(a);
+    if (npl == 2) return dispatch_fwd_cap<SYN, 2>(a);
+    return dispatch_fwd_cap<SYN, 1>(a);
+}
+
+// step offsets inside a block of CKPT steps are 32-bit byte offsets
+inline bool too_wide(int64_t neurons) { return neurons >= (int64_t{1} << 25); }
 
 }  // namespace
 
@@ -528,6 +753,7 @@ EXODUS_API int exodus_layer_lif_forward(float *out_spikes, float *out_vmem_rec, 
 {
     if (bad3(batch, t, neurons)) return hipErrorInvalidValue;
     if (batch == 0 || t == 0 || neurons == 0) return hipSuccess;
+    if (too_wide(neurons)) return hipErrorInvalidValue;
     const bool syn = alpha_syn != nullptr;
     if (!out_spikes || !v_last || !input || !vmem_post_initial || !alpha_mem || !membr_subtract || !theta ||
         (apply_theta_low && !theta_low) || (syn && !isyn_initial) || (syn && ckpt_v && !ckpt_i))
@@ -546,21 +772,9 @@ EXODUS_API int exodus_layer_lif_forward(float *out_spikes, float *out_vmem_rec, 
     p.cap = static_cast<unsigned>(max_num_spikes);
     const int npl = pick_neurons_per_lane(
         batch, neurons, common_alignment({input, out_spikes, out_vmem_rec, out_isyn_rec, ckpt_v, ckpt_i}));
-    const int64_t blocks_per_batch = (neurons + BLOCK * npl - 1) / (BLOCK * npl);
-    if (blocks_per_batch > 0x7fffffffLL / batch) return hipErrorInvalidValue;
-    const int64_t blocks = blocks_per_batch * batch;
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    const dim3 grid(static_cast<unsigned>(blocks)), block(BLOCK);
-#define EXODUS_FWD(SYN, NPL)                                                                                     \
-    hipLaunchKernelGGL((layer_lif_forward<SYN, NPL>), grid, block, 0, s, out_spikes, out_vmem_rec, out_isyn_rec, \
-                       ckpt_v, ckpt_i, v_last, i_last, spike_sum, input, p, blocks_per_batch, t, neurons)
-    if (syn) {
-        if (npl == 4) EXODUS_FWD(true, 4); else if (npl == 2) EXODUS_FWD(true, 2); else EXODUS_FWD(true, 1);
-    } else {
-        if (npl == 4) EXODUS_FWD(false, 4); else if (npl == 2) EXODUS_FWD(false, 2); else EXODUS_FWD(false, 1);
-    }
-#undef EXODUS_FWD
-    return static_cast<int>(hipGetLastError());
+    FwdArgs a{out_spikes, out_vmem_rec, out_isyn_rec, ckpt_v, ckpt_i, v_last, i_last, spike_sum, input, p,
+              batch, t, neurons, static_cast<hipStream_t>(stream)};
+    return syn ? dispatch_fwd<true>(a, npl) : dispatch_fwd<false>(a, npl);
 }
 
 EXODUS_API int exodus_layer_lif_backward(float *grad_input, float *alpha_mem_grad, float *alpha_syn_grad,
@@ -575,6 +789,7 @@ EXODUS_API int exodus_layer_lif_backward(float *grad_input, float *alpha_mem_gra
 {
     if (bad3(batch, t, neurons)) return hipErrorInvalidValue;
     if (batch == 0 || t == 0 || neurons == 0) return hipSuccess;
+    if (too_wide(neurons)) return hipErrorInvalidValue;
     const bool syn = alpha_syn != nullptr;
     if (!grad_input || !grad_spikes || !input || !ckpt_v || !alpha_mem || !membr_subtract || !theta ||
         (apply_theta_low && !theta_low) || (syn && !ckpt_i))
@@ -595,9 +810,9 @@ EXODUS_API int exodus_layer_lif_backward(float *grad_input, float *alpha_mem_gra
     p.cap = static_cast<unsigned>(max_num_spikes);
     hipStream_t s = static_cast<hipStream_t>(stream);
 #define EXODUS_BWD(SYN, K)                                                                                        \
-    return launch_bwd<SYN, K>(grad_input, alpha_mem_grad, alpha_syn_grad, vmem_init_grad, isyn_init_grad,         \
-                              grad_spikes, grad_v_last, grad_i_last, input, ckpt_v, ckpt_i, p, surr_p0, surr_p1, \
-                              batch, t, neurons, s)
+    return dispatch_bwd_cap<SYN, K>(p.cap, grad_input, alpha_mem_grad, alpha_syn_grad, vmem_init_grad,            \
+                                    isyn_init_grad, grad_spikes, grad_v_last, grad_i_last, input, ckpt_v, ckpt_i, \
+                                    p, surr_p0, surr_p1, batch, t, neurons, s)
     switch (surrogate_kind) {
         case EXODUS_SURR_SINGLE_EXP: if (syn) EXODUS_BWD(true, EXODUS_SURR_SINGLE_EXP); EXODUS_BWD(false, EXODUS_SURR_SINGLE_EXP);
         case EXODUS_SURR_PERIODIC_EXP: if (syn) EXODUS_BWD(true, EXODUS_SURR_PERIODIC_EXP); EXODUS_BWD(false, EXODUS_SURR_PERIODIC_EXP);
