@@ -28,7 +28,10 @@ namespace {
 #define EXODUS_LAYER_FWD_UNROLL 16
 #endif
 #ifndef EXODUS_LAYER_BLOCK
-#define EXODUS_LAYER_BLOCK 256
+#define EXODUS_LAYER_BLOCK 256        // lanes per block of the kernels that hold several neurons per lane
+#endif
+#ifndef EXODUS_LAYER_BWD_BLOCK
+#define EXODUS_LAYER_BWD_BLOCK 256    // lanes per block of the spiking backward kernel (one neuron per lane)
 #endif
 #ifndef EXODUS_LAYER_BWD_WAVES
 #define EXODUS_LAYER_BWD_WAVES 3      // resident waves per SIMD the backward kernel is compiled for
@@ -36,6 +39,7 @@ namespace {
 constexpr int CKPT = 32;                             // steps between checkpoints = length of a backward chunk
 constexpr int FWD_UNROLL = EXODUS_LAYER_FWD_UNROLL;  // forward steps per software-pipeline stage (divides CKPT)
 constexpr int BLOCK = EXODUS_LAYER_BLOCK;
+constexpr int BWD_BLOCK = EXODUS_LAYER_BWD_BLOCK;
 
 struct LayerConsts {
     const float *v_init, *i_init, *alpha_mem, *alpha_syn, *c, *theta, *theta_low;
@@ -203,9 +207,9 @@ __device__ __forceinline__ float spike_count_fast(float v, const Neuron &n, cons
 // ---------------------------------------------------------------------------------------------
 // Time is walked in blocks of CKPT = 2 * FWD_UNROLL steps.  Two register buffers of FWD_UNROLL
 // steps alternate: while one is consumed the loads of the other are in flight.  Every fetch issues
-// the same number of loads (the last round re-reads its own block), so the number of outstanding
-// loads at each wait is a compile-time constant.  Steps beyond the last full block run through a
-// guarded copy of the same code.
+// the same number of loads (past the end it re-reads the last step), so the number of outstanding
+// loads at each wait is a compile-time constant.  A last, partial block runs through a guarded copy
+// of the same code.
 template <bool SYN, int NPL, int CAPK, bool REC>
 __global__ void __launch_bounds__(BLOCK) layer_lif_forward(
     float *__restrict__ spikes, float *__restrict__ v_rec, float *__restrict__ i_rec, float *__restrict__ ckpt_v,
@@ -246,16 +250,20 @@ __global__ void __launch_bounds__(BLOCK) layer_lif_forward(
         }
 
         V bufa[FWD_UNROLL], bufb[FWD_UNROLL];
-        auto fetch = [&](V(&dst)[FWD_UNROLL], int64_t t0) {  // FWD_UNROLL full steps from t0
-            const Rsrc r = make_rsrc(xp + t0 * M);
+        // FWD_UNROLL steps from t0; steps past the end re-read the last step (also when t0 itself lies
+        // past the end), so every call issues exactly FWD_UNROLL loads
+        auto fetch = [&](V(&dst)[FWD_UNROLL], int64_t t0) {
+            if (t0 + FWD_UNROLL <= T) {
+                const Rsrc r = make_rsrc(xp + t0 * M);
 #pragma unroll
-            for (int u = 0; u < FWD_UNROLL; ++u) dst[u] = IO::load(r, voff, u * step_bytes);
-        };
-        auto fetch_tail = [&](V(&dst)[FWD_UNROLL], int64_t t0) {   // steps past the end re-read the last one
-            const Rsrc r = make_rsrc(xp + t0 * M);
-            const unsigned last = static_cast<unsigned>(T - 1 - t0);
+                for (int u = 0; u < FWD_UNROLL; ++u) dst[u] = IO::load(r, voff, u * step_bytes);
+            } else {
+                const int64_t tc = t0 < T ? t0 : T - 1;
+                const Rsrc r = make_rsrc(xp + tc * M);
+                const unsigned last = static_cast<unsigned>(T - 1 - tc);
 #pragma unroll
-            for (int u = 0; u < FWD_UNROLL; ++u) dst[u] = IO::load(r, voff, (u < last ? u : last) * step_bytes);
+                for (int u = 0; u < FWD_UNROLL; ++u) dst[u] = IO::load(r, voff, (u < last ? u : last) * step_bytes);
+            }
         };
         float part = 0.f;                                     // spike count since the last checkpoint (exact in fp32)
         auto checkpoint = [&](int64_t j) {
@@ -309,21 +317,23 @@ __global__ void __launch_bounds__(BLOCK) layer_lif_forward(
             }
         };
 
-        const int64_t n_full = T / CKPT;                      // blocks of CKPT steps that lie inside the sequence
-        if (n_full > 0) fetch(bufa, 0);
+        const int64_t n_full = T / CKPT;                      // blocks that lie inside the sequence
+        fetch(bufa, 0);
         for (int64_t j = 0; j < n_full; ++j) {
             const int64_t t0 = j * CKPT;
             fetch(bufb, t0 + FWD_UNROLL);
             checkpoint(j);
             compute(bufa, t0, std::false_type{});
-            fetch(bufa, j + 1 < n_full ? t0 + CKPT : t0);
+            fetch(bufa, t0 + CKPT);                           // next block, or the start of the partial one
             compute(bufb, t0 + FWD_UNROLL, std::false_type{});
         }
-        if (n_full * CKPT < T) {
+        if (n_full * CKPT < T) {                              // partial block: bufa holds its first steps
+            const int64_t t0 = n_full * CKPT;
             checkpoint(n_full);
-            for (int64_t t0 = n_full * CKPT; t0 < T; t0 += FWD_UNROLL) {
-                fetch_tail(bufa, t0);
-                compute(bufa, t0, std::true_type{});
+            compute(bufa, t0, std::true_type{});
+            if (t0 + FWD_UNROLL < T) {
+                fetch(bufa, t0 + FWD_UNROLL);
+                compute(bufa, t0 + FWD_UNROLL, std::true_type{});
             }
         }
         my_spikes += static_cast<double>(part);
@@ -357,7 +367,7 @@ __global__ void __launch_bounds__(BLOCK) layer_lif_forward(
 // gv on it reaches v_{T-1} directly and the spike count with weight -c, a gradient on the final
 // synaptic current adds to mu_{T-1}.
 template <bool SYN, int KIND, int CAPK>
-__global__ void __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(EXODUS_LAYER_BWD_WAVES, EXODUS_LAYER_BWD_WAVES)))
+__global__ void __launch_bounds__(BWD_BLOCK) __attribute__((amdgpu_waves_per_eu(EXODUS_LAYER_BWD_WAVES, EXODUS_LAYER_BWD_WAVES)))
 layer_lif_backward(
     float *__restrict__ grad_x, float *__restrict__ alpha_mem_grad, float *__restrict__ alpha_syn_grad,
     float *__restrict__ v_init_grad, float *__restrict__ i_init_grad, const float *__restrict__ grad_spikes,
@@ -367,7 +377,7 @@ layer_lif_backward(
 {
     typedef BufIO<1> IO;
     const int64_t b = blockIdx.x / blocks_per_batch;
-    const int64_t m0 = static_cast<int64_t>(blockIdx.x - b * blocks_per_batch) * BLOCK;
+    const int64_t m0 = static_cast<int64_t>(blockIdx.x - b * blocks_per_batch) * BWD_BLOCK;
     const unsigned lane_off = threadIdx.x;
     if (m0 + lane_off >= M) return;
     const int64_t row = b * M + m0 + lane_off;
@@ -643,7 +653,7 @@ __global__ void __launch_bounds__(BLOCK) layer_leaky_backward(
 // lanes: stay at the widest width that still gives every SIMD about four waves, so that small
 // layers are not starved of parallelism.  `align` is the common alignment (bytes) of all
 // (batch, time, neurons) pointers involved.
-inline int pick_neurons_per_lane(int64_t batch, int64_t neurons, unsigned align)
+inline int pick_neurons_per_lane(int64_t batch, int64_t neurons, unsigned align, int widest = 4)
 {
     int cus = 0, dev = 0;
     if (hipGetDevice(&dev) != hipSuccess ||
@@ -651,7 +661,7 @@ inline int pick_neurons_per_lane(int64_t batch, int64_t neurons, unsigned align)
         cus = 256;
     const int64_t wanted_lanes = static_cast<int64_t>(cus) * 16 * WAVE;
     const int64_t n = batch * neurons;
-    if ((neurons % 4) == 0 && (align % 16) == 0 && n / 4 >= wanted_lanes) return 4;
+    if (widest >= 4 && (neurons % 4) == 0 && (align % 16) == 0 && n / 4 >= wanted_lanes) return 4;
     if ((neurons % 2) == 0 && (align % 8) == 0 && n / 2 >= wanted_lanes) return 2;
     return 1;
 }
@@ -676,10 +686,10 @@ int launch_bwd(float *grad_x, float *am_g, float *as_g, float *v0_g, float *i0_g
                const float *gvl, const float *gil, const float *x, const float *ckpt_v, const float *ckpt_i,
                const LayerConsts &p, float p0, float p1, int64_t B, int64_t T, int64_t M, hipStream_t s)
 {
-    const int64_t blocks_per_batch = (M + BLOCK - 1) / BLOCK;
+    const int64_t blocks_per_batch = (M + BWD_BLOCK - 1) / BWD_BLOCK;
     if (blocks_per_batch > 0x7fffffffLL / B) return hipErrorInvalidValue;
     const int64_t blocks = blocks_per_batch * B;
-    hipLaunchKernelGGL((layer_lif_backward<SYN, KIND, CAPK>), dim3(static_cast<unsigned>(blocks)), dim3(BLOCK), 0, s,
+    hipLaunchKernelGGL((layer_lif_backward<SYN, KIND, CAPK>), dim3(static_cast<unsigned>(blocks)), dim3(BWD_BLOCK), 0, s,
                        grad_x, am_g, as_g, v0_g, i0_g, grad_spikes, gvl, gil, x, ckpt_v, ckpt_i, p, p0, p1,
                        p0 != 0.f ? 1.f / p0 : 0.f, blocks_per_batch, T, M);
     return static_cast<int>(hipGetLastError());
@@ -727,7 +737,6 @@ template <bool SYN>
 int dispatch_fwd(const FwdArgs &a, int npl)
 {
     if (a.v_rec || a.i_rec) return launch_fwd<SYN, 1, 0, true>(a);
-    if (npl == 4) return dispatch_fwd_cap<SYN, 4>(a);
     if (npl == 2) return dispatch_fwd_cap<SYN, 2>(a);
     return dispatch_fwd_cap<SYN, 1>(a);
 }
@@ -770,8 +779,10 @@ EXODUS_API int exodus_layer_lif_forward(float *out_spikes, float *out_vmem_rec, 
     p.decay_early = decay_early ? 1 : 0;
     p.norm_input = norm_input ? 1 : 0;
     p.cap = static_cast<unsigned>(max_num_spikes);
+    // two neurons per lane at most: with four the spiking kernel needs so many registers for its two
+    // load buffers that only two waves fit a SIMD, and it measures slower than two neurons, three waves
     const int npl = pick_neurons_per_lane(
-        batch, neurons, common_alignment({input, out_spikes, out_vmem_rec, out_isyn_rec, ckpt_v, ckpt_i}));
+        batch, neurons, common_alignment({input, out_spikes, out_vmem_rec, out_isyn_rec, ckpt_v, ckpt_i}), 2);
     FwdArgs a{out_spikes, out_vmem_rec, out_isyn_rec, ckpt_v, ckpt_i, v_last, i_last, spike_sum, input, p,
               batch, t, neurons, static_cast<hipStream_t>(stream)};
     return syn ? dispatch_fwd<true>(a, npl) : dispatch_fwd<false>(a, npl);
