@@ -515,7 +515,13 @@ struct LeakyConsts {
 
 constexpr int LEAKY_UNROLL = 8;
 
+// Both leaky kernels walk time in pairs of stages of LEAKY_UNROLL steps with two register buffers:
+// while one stage is consumed, the loads of the other are in flight, and because every fetch
+// issues the same number of loads, each wait covers only the loads it needs.  The steps that do
+// not fill a pair (fewer than 2 * LEAKY_UNROLL) are done one at a time.
+
 // xin = norm_input ? (1 - alpha) * x : x;  xin = decay_early ? xin * alpha : xin;  v = v * alpha + xin
+// (the two input factors are applied as kn = 1 - alpha or 1 and kd = alpha or 1: a factor of 1 is exact)
 template <int NPL>
 __global__ void __launch_bounds__(BLOCK) layer_leaky_forward(float *__restrict__ out, float *__restrict__ v_last,
                                                              const float *__restrict__ x, const LeakyConsts p,
@@ -523,6 +529,8 @@ __global__ void __launch_bounds__(BLOCK) layer_leaky_forward(float *__restrict__
                                                              const int64_t M)
 {
     typedef typename Vec<NPL>::type V;
+    typedef BufIO<NPL> IO;
+    constexpr int U = LEAKY_UNROLL;
     const int64_t b = blockIdx.x / blocks_per_batch;
     const int64_t m0 = static_cast<int64_t>(blockIdx.x - b * blocks_per_batch) * (BLOCK * NPL);
     const unsigned lane_off = threadIdx.x * NPL;
@@ -530,41 +538,51 @@ __global__ void __launch_bounds__(BLOCK) layer_leaky_forward(float *__restrict__
     const int64_t first = b * M + m0 + lane_off;
     const float *xp = x + (b * T) * M + m0;
     float *op = out + (b * T) * M + m0;
-    float a[NPL], k[NPL], v[NPL];
+    const unsigned voff = lane_off * 4u;
+    const unsigned step_bytes = static_cast<unsigned>(M) * 4u;
+    float a[NPL], kn[NPL], kd[NPL], v[NPL];
 #pragma unroll
     for (int e = 0; e < NPL; ++e) {
         a[e] = p.alpha[first + e];
-        k[e] = __fsub_rn(1.0f, a[e]);
+        kn[e] = p.norm_input ? __fsub_rn(1.0f, a[e]) : 1.0f;
+        kd[e] = p.decay_early ? a[e] : 1.0f;
         v[e] = p.v_init[first + e];
     }
-    V cur[LEAKY_UNROLL], nxt[LEAKY_UNROLL];
-    auto fetch = [&](V(&dst)[LEAKY_UNROLL], int64_t t0) {
+    auto advance = [&](const V &xv) {
+        V o;
 #pragma unroll
-        for (int u = 0; u < LEAKY_UNROLL; ++u) {
-            const int64_t t = t0 + u < T ? t0 + u : T - 1;     // constant number of loads in flight
-            dst[u] = ld_stream(reinterpret_cast<const V *>(xp + t * M + lane_off));
+        for (int e = 0; e < NPL; ++e) {
+            const float xin = __fmul_rn(__fmul_rn(kn[e], lane_get<NPL>(xv, e)), kd[e]);
+            v[e] = __fadd_rn(__fmul_rn(v[e], a[e]), xin);
+            lane_put<NPL>(o, e, v[e]);
         }
+        return o;
     };
-    fetch(cur, 0);
-    for (int64_t t0 = 0; t0 < T; t0 += LEAKY_UNROLL) {
-        fetch(nxt, t0 + LEAKY_UNROLL);
+    // `spread` = step_bytes, or 0 for a fetch whose data will not be used (same count of loads, one step)
+    auto fetch = [&](V(&dst)[U], int64_t t0, unsigned spread) {
+        const Rsrc r = make_rsrc(xp + t0 * M);
 #pragma unroll
-        for (int u = 0; u < LEAKY_UNROLL; ++u) {
-            if (t0 + u < T) {
-                V o;
+        for (int u = 0; u < U; ++u) dst[u] = IO::load(r, voff, u * spread);
+    };
+    auto compute = [&](const V(&buf)[U], int64_t t0) {
+        const Rsrc r = make_rsrc(op + t0 * M);
 #pragma unroll
-                for (int e = 0; e < NPL; ++e) {
-                    float xin = lane_get<NPL>(cur[u], e);
-                    if (p.norm_input) xin = __fmul_rn(k[e], xin);
-                    if (p.decay_early) xin = __fmul_rn(xin, a[e]);
-                    v[e] = __fadd_rn(__fmul_rn(v[e], a[e]), xin);
-                    lane_put<NPL>(o, e, v[e]);
-                }
-                st_stream(o, reinterpret_cast<V *>(op + (t0 + u) * M + lane_off));
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < LEAKY_UNROLL; ++u) cur[u] = nxt[u];
+        for (int u = 0; u < U; ++u) IO::store(advance(buf[u]), r, voff, u * step_bytes);
+    };
+    const int64_t pairs = T / (2 * U);
+    V bufa[U], bufb[U];
+    if (pairs > 0) fetch(bufa, 0, step_bytes);
+    for (int64_t q = 0; q < pairs; ++q) {
+        const int64_t t0 = q * 2 * U;
+        fetch(bufb, t0 + U, step_bytes);
+        compute(bufa, t0);
+        const bool more = q + 1 < pairs;
+        fetch(bufa, more ? t0 + 2 * U : t0, more ? step_bytes : 0u);
+        compute(bufb, t0 + U);
+    }
+    for (int64_t t = pairs * 2 * U; t < T; ++t) {
+        const V xv = IO::load(make_rsrc(xp + t * M), voff, 0u);
+        IO::store(advance(xv), make_rsrc(op + t * M), voff, 0u);
     }
 #pragma unroll
     for (int e = 0; e < NPL; ++e) v_last[first + e] = v[e];
@@ -581,6 +599,8 @@ __global__ void __launch_bounds__(BLOCK) layer_leaky_backward(
     const float *__restrict__ x, const LeakyConsts p, const int64_t blocks_per_batch, const int64_t T, const int64_t M)
 {
     typedef typename Vec<NPL>::type V;
+    typedef BufIO<NPL> IO;
+    constexpr int U = LEAKY_UNROLL;
     const int64_t b = blockIdx.x / blocks_per_batch;
     const int64_t m0 = static_cast<int64_t>(blockIdx.x - b * blocks_per_batch) * (BLOCK * NPL);
     const unsigned lane_off = threadIdx.x * NPL;
@@ -590,53 +610,90 @@ __global__ void __launch_bounds__(BLOCK) layer_leaky_backward(
     const float *outp = ALPHA ? out + (b * T) * M + m0 : nullptr;
     const float *xp = WITH_X ? x + (b * T) * M + m0 : nullptr;
     float *op = grad_x + (b * T) * M + m0;
-    float a[NPL], k[NPL], g[NPL];
+    const unsigned voff = lane_off * 4u;
+    const unsigned step_bytes = static_cast<unsigned>(M) * 4u;
+    float a[NPL], k[NPL], h[NPL], g[NPL];
     TileSum acc[NPL];
 #pragma unroll
     for (int e = 0; e < NPL; ++e) {
         a[e] = p.alpha[first + e];
         k[e] = __fsub_rn(1.0f, a[e]);
-        g[e] = grad_v_last ? grad_v_last[first + e] : 0.f;     // joins grad_out at the last step
+        h[e] = grad_v_last ? grad_v_last[first + e] : 0.f;     // what reaches step t from later steps: alpha g_{t+1}
+        g[e] = 0.f;
         acc[e].clear();
     }
-    // step t needs out_{t-1}: walk t = T-1 .. 0 in groups, newest first
-    for (int64_t t_hi = T; t_hi > 0; t_hi -= LEAKY_UNROLL) {
-        V gv[LEAKY_UNROLL], ov[LEAKY_UNROLL], xv[LEAKY_UNROLL];
+    // one step; `ov` = out_{t-1} (ignored at t = 0, where the initial state takes its place)
+    auto advance = [&](int64_t t, const V &gv, const V &ov, const V &xv) {
+        V o;
 #pragma unroll
-        for (int u = 0; u < LEAKY_UNROLL; ++u) {
-            // steps before the first re-read step 0: constant number of loads in flight
-            const int64_t t = t_hi - 1 - u >= 0 ? t_hi - 1 - u : 0;
-            gv[u] = ld_stream(reinterpret_cast<const V *>(gp + t * M + lane_off));
-            if (WITH_X) xv[u] = ld_stream(reinterpret_cast<const V *>(xp + t * M + lane_off));
-            if (ALPHA) ov[u] = ld_stream(reinterpret_cast<const V *>(outp + (t >= 1 ? t - 1 : 0) * M + lane_off));
-        }
-#pragma unroll
-        for (int u = 0; u < LEAKY_UNROLL; ++u) {
-            const int64_t t = t_hi - 1 - u;
-            if (t >= 0) {
-                V o;
-#pragma unroll
-                for (int e = 0; e < NPL; ++e) {
-                    // first processed step (t = T-1): g holds grad_v_last and there is no later step to decay
-                    const float carried = (t == T - 1) ? g[e] : __fmul_rn(g[e], a[e]);
-                    g[e] = __fadd_rn(carried, lane_get<NPL>(gv[u], e));
-                    float gx = g[e];
-                    if (p.decay_early) gx = __fmul_rn(gx, a[e]);
-                    if (ALPHA) {
-                        const float prev = t >= 1 ? lane_get<NPL>(ov[u], e) : p.v_init[first + e];
-                        acc[e].add(g[e], prev);
-                        if (WITH_X) {
-                            const float xe = lane_get<NPL>(xv[u], e);
-                            if (p.decay_early) acc[e].add(g[e], p.norm_input ? __fmul_rn(k[e], xe) : xe);
-                            if (p.norm_input) acc[e].sub(gx, xe);
-                        }
-                    }
-                    if (p.norm_input) gx = __fmul_rn(gx, k[e]);
-                    lane_put<NPL>(o, e, gx);
+        for (int e = 0; e < NPL; ++e) {
+            g[e] = __fadd_rn(h[e], lane_get<NPL>(gv, e));
+            h[e] = __fmul_rn(g[e], a[e]);
+            float gx = p.decay_early ? h[e] : g[e];
+            if (ALPHA) {
+                const float prev = t >= 1 ? lane_get<NPL>(ov, e) : p.v_init[first + e];
+                acc[e].add(g[e], prev);
+                if (WITH_X) {
+                    const float xe = lane_get<NPL>(xv, e);
+                    if (p.decay_early) acc[e].add(g[e], p.norm_input ? __fmul_rn(k[e], xe) : xe);
+                    if (p.norm_input) acc[e].sub(gx, xe);
                 }
-                st_stream(o, reinterpret_cast<V *>(op + t * M + lane_off));
             }
+            if (p.norm_input) gx = __fmul_rn(gx, k[e]);
+            lane_put<NPL>(o, e, gx);
         }
+        return o;
+    };
+    struct Stage {
+        V g[U], o[ALPHA ? U : 1], x[WITH_X ? U : 1];
+    };
+    // steps t0 .. t0 + U - 1; `spread` = step_bytes, or 0 for a fetch whose data will not be used
+    auto fetch = [&](Stage &s, int64_t t0, unsigned spread) {
+        const Rsrc rg = make_rsrc(gp + t0 * M);
+#pragma unroll
+        for (int u = 0; u < U; ++u) s.g[u] = IO::load(rg, voff, u * spread);
+        if (WITH_X) {
+            const Rsrc rx = make_rsrc(xp + t0 * M);
+#pragma unroll
+            for (int u = 0; u < U; ++u) s.x[u] = IO::load(rx, voff, u * spread);
+        }
+        if (ALPHA) {
+            // out_{t-1}: one step back, except that step 0 has no predecessor (it re-reads out_0, unused)
+            const Rsrc ro = make_rsrc(outp + (t0 >= 1 ? t0 - 1 : 0) * M);
+            const unsigned shift = t0 >= 1 ? 0u : 1u;
+#pragma unroll
+            for (int u = 0; u < U; ++u) s.o[u] = IO::load(ro, voff, (u >= shift ? u - shift : 0u) * spread);
+        }
+    };
+    auto compute = [&](const Stage &s, int64_t t0) {          // newest step first
+        const Rsrc r = make_rsrc(op + t0 * M);
+#pragma unroll
+        for (int uu = 0; uu < U; ++uu) {
+            const int u = U - 1 - uu;
+            IO::store(advance(t0 + u, s.g[u], s.o[ALPHA ? u : 0], s.x[WITH_X ? u : 0]), r, voff, u * step_bytes);
+        }
+    };
+    const int64_t pairs = T / (2 * U);
+    // the steps that do not fill a pair are the newest ones: one at a time
+    for (int64_t t = T - 1; t >= pairs * 2 * U; --t) {
+        const V gv = IO::load(make_rsrc(gp + t * M), voff, 0u);
+        V ov = gv, xv = gv;
+        if (ALPHA && t >= 1) ov = IO::load(make_rsrc(outp + (t - 1) * M), voff, 0u);
+        if (WITH_X) xv = IO::load(make_rsrc(xp + t * M), voff, 0u);
+        IO::store(advance(t, gv, ov, xv), make_rsrc(op + t * M), voff, 0u);
+    }
+    if (ALPHA) {
+#pragma unroll
+        for (int e = 0; e < NPL; ++e) acc[e].fold();
+    }
+    Stage sa, sb;
+    if (pairs > 0) fetch(sa, (pairs - 1) * 2 * U + U, step_bytes);
+    for (int64_t q = pairs - 1; q >= 0; --q) {
+        const int64_t t0 = q * 2 * U;
+        fetch(sb, t0, step_bytes);
+        compute(sa, t0 + U);
+        fetch(sa, q > 0 ? t0 - U : t0, q > 0 ? step_bytes : 0u);
+        compute(sb, t0);
         if (ALPHA) {
 #pragma unroll
             for (int e = 0; e < NPL; ++e) acc[e].fold();
@@ -644,25 +701,26 @@ __global__ void __launch_bounds__(BLOCK) layer_leaky_backward(
     }
 #pragma unroll
     for (int e = 0; e < NPL; ++e) {
-        if (v_init_grad) v_init_grad[first + e] = __fmul_rn(a[e], g[e]);
+        if (v_init_grad) v_init_grad[first + e] = h[e];
         if (ALPHA) alpha_grad[first + e] = static_cast<float>(acc[e].total);
     }
 }
 
-// Neurons per lane of the forward kernels.  Wider lanes mean wider memory accesses but fewer
-// lanes: stay at the widest width that still gives every SIMD about four waves, so that small
-// layers are not starved of parallelism.  `align` is the common alignment (bytes) of all
-// (batch, time, neurons) pointers involved.
-inline int pick_neurons_per_lane(int64_t batch, int64_t neurons, unsigned align, int widest = 4)
+// Neurons per lane of the kernels that support several.  Wider lanes mean wider memory accesses
+// but fewer lanes: stay at the widest width that still gives every compute unit `waves_per_cu`
+// waves, so that small layers are not starved of parallelism (the spiking forward kernel has a long
+// dependent chain per step and wants 16; the leaky kernels measure best from 8 on).  `align` is the
+// common alignment (bytes) of all (batch, time, neurons) pointers involved.
+inline int pick_neurons_per_lane(int64_t batch, int64_t neurons, unsigned align, int widest, int waves_per_cu)
 {
     int cus = 0, dev = 0;
     if (hipGetDevice(&dev) != hipSuccess ||
         hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
         cus = 256;
-    const int64_t wanted_lanes = static_cast<int64_t>(cus) * 16 * WAVE;
+    const int64_t wanted_lanes = static_cast<int64_t>(cus) * waves_per_cu * WAVE;
     const int64_t n = batch * neurons;
     if (widest >= 4 && (neurons % 4) == 0 && (align % 16) == 0 && n / 4 >= wanted_lanes) return 4;
-    if ((neurons % 2) == 0 && (align % 8) == 0 && n / 2 >= wanted_lanes) return 2;
+    if (widest >= 2 && (neurons % 2) == 0 && (align % 8) == 0 && n / 2 >= wanted_lanes) return 2;
     return 1;
 }
 
@@ -782,7 +840,7 @@ EXODUS_API int exodus_layer_lif_forward(float *out_spikes, float *out_vmem_rec, 
     // two neurons per lane at most: with four the spiking kernel needs so many registers for its two
     // load buffers that only two waves fit a SIMD, and it measures slower than two neurons, three waves
     const int npl = pick_neurons_per_lane(
-        batch, neurons, common_alignment({input, out_spikes, out_vmem_rec, out_isyn_rec, ckpt_v, ckpt_i}), 2);
+        batch, neurons, common_alignment({input, out_spikes, out_vmem_rec, out_isyn_rec, ckpt_v, ckpt_i}), 2, 16);
     FwdArgs a{out_spikes, out_vmem_rec, out_isyn_rec, ckpt_v, ckpt_i, v_last, i_last, spike_sum, input, p,
               batch, t, neurons, static_cast<hipStream_t>(stream)};
     return syn ? dispatch_fwd<true>(a, npl) : dispatch_fwd<false>(a, npl);
@@ -839,13 +897,14 @@ EXODUS_API int exodus_layer_leaky_forward(float *out, float *v_last, const float
 {
     if (bad3(batch, t, neurons)) return hipErrorInvalidValue;
     if (batch == 0 || t == 0 || neurons == 0) return hipSuccess;
+    if (too_wide(neurons)) return hipErrorInvalidValue;
     if (!out || !v_last || !input || !vmem_initial || !alpha) return hipErrorInvalidValue;
     LeakyConsts p;
     p.v_init = vmem_initial;
     p.alpha = alpha;
     p.decay_early = decay_early ? 1 : 0;
     p.norm_input = norm_input ? 1 : 0;
-    const int npl = pick_neurons_per_lane(batch, neurons, common_alignment({input, out}));
+    const int npl = pick_neurons_per_lane(batch, neurons, common_alignment({input, out}), 4, 8);
     const int64_t blocks_per_batch = (neurons + BLOCK * npl - 1) / (BLOCK * npl);
     if (blocks_per_batch > 0x7fffffffLL / batch) return hipErrorInvalidValue;
     const dim3 grid(static_cast<unsigned>(blocks_per_batch * batch)), block(BLOCK);
@@ -867,6 +926,7 @@ EXODUS_API int exodus_layer_leaky_backward(float *grad_input, float *alpha_grad,
 {
     if (bad3(batch, t, neurons)) return hipErrorInvalidValue;
     if (batch == 0 || t == 0 || neurons == 0) return hipSuccess;
+    if (too_wide(neurons)) return hipErrorInvalidValue;
     if (!grad_input || !grad_out || !alpha) return hipErrorInvalidValue;
     const bool want_alpha = alpha_grad != nullptr;
     const bool with_x = want_alpha && (decay_early || norm_input);
@@ -877,7 +937,9 @@ EXODUS_API int exodus_layer_leaky_backward(float *grad_input, float *alpha_grad,
     p.alpha = alpha;
     p.decay_early = decay_early ? 1 : 0;
     p.norm_input = norm_input ? 1 : 0;
-    const int npl = pick_neurons_per_lane(batch, neurons, common_alignment({grad_input, grad_out, out, input}));
+    // with the alpha gradient two or three tensors are double-buffered: two neurons per lane at most
+    const int npl = pick_neurons_per_lane(batch, neurons, common_alignment({grad_input, grad_out, out, input}),
+                                          want_alpha ? 2 : 4, 8);
     const int64_t blocks_per_batch = (neurons + BLOCK * npl - 1) / (BLOCK * npl);
     if (blocks_per_batch > 0x7fffffffLL / batch) return hipErrorInvalidValue;
     const dim3 grid(static_cast<unsigned>(blocks_per_batch * batch)), block(BLOCK);
@@ -886,7 +948,7 @@ EXODUS_API int exodus_layer_leaky_backward(float *grad_input, float *alpha_grad,
     hipLaunchKernelGGL((layer_leaky_backward<NPL, AL, WX>), grid, block, 0, s, grad_input, alpha_grad,        \
                        vmem_init_grad, grad_out, grad_v_last, out, input, p, blocks_per_batch, t, neurons)
     if (npl == 4) {
-        if (with_x) EXODUS_LK(4, true, true); else if (want_alpha) EXODUS_LK(4, true, false); else EXODUS_LK(4, false, false);
+        EXODUS_LK(4, false, false);
     } else if (npl == 2) {
         if (with_x) EXODUS_LK(2, true, true); else if (want_alpha) EXODUS_LK(2, true, false); else EXODUS_LK(2, false, false);
     } else {
