@@ -74,15 +74,21 @@ __device__ __forceinline__ float spike_count(float v, float theta, unsigned cap)
     //   v >= 2*theta (exact)  <=>  RN(v/theta) >= 2   (no fp32 number lies strictly between the
     //                              predecessor of 2*theta and 2*theta, and the rounding boundary
     //                              2*theta*(1 - 2^-25) falls inside that gap)
-    // so below 2*theta the count is 0 or 1 without dividing, and a cap of 1 or 2 never divides.
-    if (v < theta) return 0.f;
-    if (theta > 0.f) {
-        if (cap <= 1u) return static_cast<float>(cap);
-        if (v < __fadd_rn(theta, theta)) return 1.f;
-        if (cap == 2u) return 2.f;
+    // so counts up to 2 come from two comparisons and selects, without branches; the one (rare)
+    // branch is taken from 2*theta on when the cap allows more than two spikes, and for thresholds
+    // that are not positive.
+    const float one = cap >= 1u ? 1.f : 0.f;
+    const float two = cap >= 2u ? 2.f : one;
+    const bool fire = v >= theta;
+    const bool plain = theta > 0.f;
+    const bool second = plain & (v >= __fadd_rn(theta, theta));
+    float count = fire ? one : 0.f;
+    count = second ? two : count;
+    if (fire & (!plain | (second & (cap > 2u)))) {
+        const unsigned k = static_cast<unsigned>(__fdiv_rn(v, theta));
+        count = static_cast<float>(k < cap ? k : cap);
     }
-    const unsigned k = static_cast<unsigned>(__fdiv_rn(v, theta));
-    return static_cast<float>(k < cap ? k : cap);
+    return count;
 }
 
 // Per-row constants of the in-kernel surrogate gradients.  Surrogate values enter gradients only
