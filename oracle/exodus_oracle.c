@@ -34,6 +34,18 @@
 
 #define EXPORT __attribute__((visibility("default")))
 
+/* float -> unsigned the way the device does it (saturating: negative and NaN give 0, values
+ * beyond 32 bits give UINT_MAX).  A plain C cast is undefined for those inputs; they occur when a
+ * threshold is not positive. */
+static unsigned to_unsigned_sat(float q)
+{
+    if (!(q > 0.0f))
+        return 0u;
+    if (q >= 4294967296.0f)
+        return 0xffffffffu;
+    return (unsigned)q;
+}
+
 /* number of worker threads used by the row loops (1 = scalar) */
 static int g_threads = 1;
 
@@ -124,7 +136,7 @@ EXPORT void oracle_lif_forward(float *spikes, float *v_mem, const float *in, con
             if (apply_theta_low && v < lo)
                 v = lo;
             if (v >= th) {
-                unsigned k = (unsigned)(v / th);
+                unsigned k = to_unsigned_sat(v / th);
                 count = k < cap ? k : cap;
             } else {
                 count = 0;
@@ -234,7 +246,7 @@ EXPORT void oracle_spike_forward(float *spikes, float *u, float alpha, float mem
         for (int64_t i = 0; i < n_steps; ++i) {
             s[i] = 0.0f;
             if (v[i] >= theta) {
-                unsigned k = (unsigned)(v[i] / theta);
+                unsigned k = to_unsigned_sat(v[i] / theta);
                 if (k > cap)
                     k = cap;
                 s[i] = (float)k;

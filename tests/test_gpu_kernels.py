@@ -72,6 +72,22 @@ def test_lif_forward_bitwise(hip, ref, n, t, cap, use_lo):
     assert torch.equal(s.cpu(), ws)
 
 
+@pytest.mark.parametrize("cap", [-1, 0, 1, 2, 3])
+def test_lif_forward_other_caps_and_nonpositive_thresholds(hip, ref, cap):
+    """Caps beyond the usual ones and thresholds that are zero or negative (the count then comes from
+    the quotient, converted to unsigned with saturation as the device does): still bit for bit."""
+    n, t = 130, 77
+    c = lif_case(900 + cap, n, t, lo=True, scale=1.5, shift=0.4)
+    th = c["theta"].clone()
+    th[::3] = -0.2 * th[::3]
+    th[1::7] = 0.0
+    s = torch.empty(n, t, device="cuda"); v = torch.empty(n, t, device="cuda")
+    hip.lifForward(s, v, D(c["x"]), D(c["v0"]), D(c["alpha"]), D(c["c"]), D(th), D(c["lo"]), True, cap)
+    ws, wv = ref.lif_forward(c["x"], c["v0"], c["alpha"], c["c"], th, c["lo"], True, cap)
+    assert torch.equal(s.cpu(), ws) and torch.equal(v.cpu(), wv)
+    assert ws[2::3].max() >= min(3, cap if cap >= 0 else 3) or cap == 0
+
+
 def test_lif_forward_many_spikes_per_step(hip, ref):
     # the regime of reference tests/test_iaf.py:71-79 and tests/test_lif.py:78: inputs of 1e2..1e4 thresholds
     n, t = 40, 50

@@ -126,3 +126,46 @@ def test_native_expleak_records_and_squeeze(L):
     native, rows = pair(el, el.ExpLeakSqueeze, tau_mem=12.0, batch_size=5, record_states=True)
     a = native(x); b = rows(x)
     assert torch.equal(a, b) and torch.equal(native.recordings["v_mem"], rows.recordings["v_mem"])
+
+
+@pytest.mark.parametrize("cap", [0, 1, 2, 3, 5, -1])
+@pytest.mark.parametrize("b,t,m", [(2, 31, 6), (3, 32, 10), (2, 33, 7), (1, 64, 260), (2, 97, 64), (1, 5, 1), (20, 40, 2048)])
+@pytest.mark.parametrize("theta_sign", ["positive", "mixed"])
+def test_native_membrane_against_cpu_oracle_all_caps(L, cap, b, t, m, theta_sign):
+    """Every spike-count specialisation (cap 1, cap 2, general), every lane width, sequences that
+    end inside / at / just after a checkpoint block, and thresholds that are not positive (which take
+    the quotient path): spikes and states bit for bit, gradients within tolerance, against the C
+    restatement of the reference kernels."""
+    _, _, hip = L
+    from oracle import exodus_ref as ref
+    from oracle import sinabs_cpu as sc
+    n = b * m
+    g = gen(cap * 1000 + t * 10 + m)
+    x = torch.randn(b, t, m, generator=g) * 1.5 + 0.4          # up to ~6 spikes per step
+    alpha = 0.3 + 0.7 * torch.rand(n, generator=g); v0 = torch.randn(n, generator=g) * 0.3
+    th = 0.5 + torch.rand(n, generator=g); c = 0.3 + 0.5 * torch.rand(n, generator=g)
+    lo = -0.5 - torch.rand(n, generator=g)
+    if theta_sign == "mixed":
+        th[::3] = -th[::3] * 0.2                               # still above the lower bound
+        th[1::7] = 0.0
+    ws, wv = ref.lif_forward(sc.bt_to_rows(x), v0, alpha, c, th, lo, True, cap)
+    D = lambda z: z.cuda()
+    res = hip.layerLifForward(D(x), D(v0), None, D(alpha), None, D(c), D(th), D(lo), True, cap, True, False)
+    assert torch.equal(res["spikes"].cpu(), sc.rows_to_bt(ws, b))
+    vpost = wv - c[:, None] * ws
+    assert torch.equal(res["v_last"].cpu(), vpost[:, -1])
+    total = float(ws.double().sum())                       # a zero threshold without cap gives 2^32 - 1 "spikes"
+    assert abs(float(res["spike_sum"]) - total) <= 1e-6 * total
+    if cap > 0:
+        assert ws.max() <= cap
+    if theta_sign == "mixed":
+        return                                                 # surrogates divide by the threshold
+    go = torch.randn(b, t, m, generator=g)
+    gi, ga, gv0 = ref.integrate_and_fire_backward(sc.bt_to_rows(go), None, wv, ws, v0, alpha, c, th, lo,
+                                                  ref.SingleExponential(), True, gate_initial=True)
+    got = hip.layerLifBackward(D(go), None, None, D(x), res["ckpt_v"], None, D(v0), None, D(alpha), None, D(c),
+                               D(th), D(lo), True, cap, True, False, hip.SURR_SINGLE_EXP, 0.5, 1.0)
+    from _util import assert_close_rowscaled
+    assert_close_rowscaled(sc.bt_to_rows(got[0].cpu()), gi, "grad input")
+    assert_close(got[3].cpu(), gv0, "grad v_init", atol=1e-5 * max(1.0, gv0.abs().max().item()))
+    assert_close(got[1].cpu(), ga, "grad alpha", rtol=2e-4, atol=2e-5 * max(1.0, ga.abs().max().item()))
