@@ -163,7 +163,9 @@ int exodus_synlif_backward(float *grad_input, float *alpha_mem_grad, float *alph
  * (batch, time, *neurons) input into (rows, time), runs the Functions and views the results back
  * (reference sinabs/exodus/layers/lif.py:152-183, 260-307).  These entry points work on the
  * (batch, t, neurons) tensors directly (neurons = product of the trailing dimensions, contiguous)
- * and write only what the layer hands out.  Per-neuron vectors have batch*neurons entries, in
+ * and write only what the layer hands out (neurons < 2^25 per batch element: step offsets are
+ * 32-bit byte offsets; wider layers get hipErrorInvalidValue and belong on the (rows, time)
+ * entry points).  Per-neuron vectors have batch*neurons entries, in
  * the order of the layer's state tensors.
  * ------------------------------------------------------------------------------------------- */
 

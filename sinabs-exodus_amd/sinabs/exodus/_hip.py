@@ -403,6 +403,10 @@ def synLifBackward(gradSpikes, gradVmem, gradIsyn, vmem, isyn, vmemPostInitial, 
 # layer-layout kernels: (batch, time, neurons) tensors, no transposition
 # ------------------------------------------------------------------------------------------
 
+# neurons per batch element the layer-layout entry points accept (they return invalid-value beyond)
+LAYER_MAX_NEURONS = 1 << 25
+
+
 def checkpointInterval() -> int:
     return int(lib.exodus_layer_checkpoint_interval())
 

@@ -13,6 +13,7 @@ import torch
 
 from .._compat import (LIFBase, MaxSpike, MembraneSubtract, MultiSpike, SingleExponential, SingleSpike,
                        SqueezeMixin)
+from .. import _hip
 from ..leaky import LeakyIntegrator
 from ..layer_function import LeakyLayerFunction, SpikingLayerFunction
 from ..spike import IntegrateAndFire
@@ -213,6 +214,8 @@ class LIF(LIFBase):
     def _use_native_layout(self, input_data: torch.Tensor) -> bool:
         if not (self.native_layout and input_data.is_cuda and input_data.dtype == torch.float32
                 and input_data.ndim >= 2):
+            return False
+        if input_data[0, 0].numel() >= _hip.LAYER_MAX_NEURONS:   # the kernels keep step offsets in 32 bits
             return False
         if self.spike_fn is None:                      # leaky integrator: the output is the state record
             return self.tau_syn_calculated is None

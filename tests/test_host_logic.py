@@ -43,6 +43,19 @@ def test_library_exports_every_declared_symbol():
     assert lib.exodus_hip_abi_version() == 1
 
 
+def test_layer_entry_points_reject_too_wide_layers_before_touching_the_device():
+    """Argument checks come first, so this needs no GPU: 2^25 neurons per batch element is beyond the
+    32-bit step offsets of the layer-layout kernels."""
+    from sinabs.exodus import _hip
+    wide = _hip.LAYER_MAX_NEURONS
+    null = None
+    rc = _hip.lib.exodus_layer_lif_forward(*([null] * 16), 0, -1, 1, 1, 1, 4, wide, null)
+    assert rc == 1
+    rc = _hip.lib.exodus_layer_leaky_forward(*([null] * 5), 1, 1, 1, 4, wide, null)
+    assert rc == 1
+    assert _hip.lib.exodus_layer_lif_forward(*([null] * 16), 0, -1, 1, 1, 0, 4, 8, null) == 0   # empty batch
+
+
 def test_loader_signatures_cover_the_header():
     from sinabs.exodus import _hip
     assert sorted(_hip._SIGNATURES) == declared_functions()
