@@ -49,6 +49,10 @@ MEASURED_TRAFFIC = {
     ("c5", "exodus_layer_lif_forward"): 17.34e9,
     ("c5", "exodus_synlif_backward"): 33.79e9,
     ("c5", "exodus_synlif_forward"): 33.64e9,
+    ("c2", "exodus_layer_lif_backward"): 15.37e9,
+    ("c2", "exodus_layer_lif_forward"): 10.30e9,
+    ("c3", "exodus_layer_leaky_backward"): 3.15e9,
+    ("c3", "exodus_layer_leaky_forward"): 2.10e9,
 }
 
 
