@@ -29,7 +29,7 @@ extern "C" {
 #endif
 
 /* ABI version of this header; bumped on any signature change. */
-#define EXODUS_HIP_ABI_VERSION 1
+#define EXODUS_HIP_ABI_VERSION 2
 
 int exodus_hip_abi_version(void);
 const char *exodus_hip_error_string(int status);
@@ -206,10 +206,12 @@ int exodus_layer_lif_backward(float *grad_input, float *alpha_mem_grad, float *a
 /* Forward of the non-spiking leaky-integrator layer (ExpLeak) on (batch,t,neurons): per neuron
  *   xin = norm_input ? (1 - alpha) * input : input;  xin = decay_early ? xin * alpha : xin;
  *   out_t = alpha * out_{t-1} + xin_t,  out_{-1} = vmem_initial
- * (reference sinabs/exodus/layers/lif.py:206-223).  v_last (batch*neurons) receives out[:, -1]. */
-int exodus_layer_leaky_forward(float *out, float *v_last, const float *input, const float *vmem_initial,
-                               const float *alpha, int decay_early, int norm_input, int64_t batch,
-                               int64_t t, int64_t neurons, void *stream);
+ * (reference sinabs/exodus/layers/lif.py:206-223).  v_last (batch*neurons) receives out[:, -1];
+ * out_sum (optional, one double that the caller has zeroed) receives the sum of all outputs, which
+ * the layer divides by their number (lif.py:305) without reading the output again. */
+int exodus_layer_leaky_forward(float *out, float *v_last, double *out_sum, const float *input,
+                               const float *vmem_initial, const float *alpha, int decay_early, int norm_input,
+                               int64_t batch, int64_t t, int64_t neurons, void *stream);
 
 /* Backward of the above: grad_input (batch,t,neurons); optional per-neuron alpha_grad (needs `out`
  * and `vmem_initial`, and `input` when one of the input scalings is on) and vmem_init_grad;

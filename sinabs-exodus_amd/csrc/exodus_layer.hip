@@ -524,7 +524,8 @@ constexpr int LEAKY_UNROLL = 8;
 // (the two input factors are applied as kn = 1 - alpha or 1 and kd = alpha or 1: a factor of 1 is exact)
 template <int NPL>
 __global__ void __launch_bounds__(BLOCK) layer_leaky_forward(float *__restrict__ out, float *__restrict__ v_last,
-                                                             const float *__restrict__ x, const LeakyConsts p,
+                                                             double *out_sum, const float *__restrict__ x,
+                                                             const LeakyConsts p,
                                                              const int64_t blocks_per_batch, const int64_t T,
                                                              const int64_t M)
 {
@@ -534,13 +535,15 @@ __global__ void __launch_bounds__(BLOCK) layer_leaky_forward(float *__restrict__
     const int64_t b = blockIdx.x / blocks_per_batch;
     const int64_t m0 = static_cast<int64_t>(blockIdx.x - b * blocks_per_batch) * (BLOCK * NPL);
     const unsigned lane_off = threadIdx.x * NPL;
-    if (m0 + lane_off >= M) return;
+    double my_sum = 0.0;                                       // sum of this lane's outputs (for the layer's mean)
+    if (m0 + lane_off < M) {
     const int64_t first = b * M + m0 + lane_off;
     const float *xp = x + (b * T) * M + m0;
     float *op = out + (b * T) * M + m0;
     const unsigned voff = lane_off * 4u;
     const unsigned step_bytes = static_cast<unsigned>(M) * 4u;
     float a[NPL], kn[NPL], kd[NPL], v[NPL];
+    float part = 0.f;                                          // outputs of one stage, then folded into my_sum
 #pragma unroll
     for (int e = 0; e < NPL; ++e) {
         a[e] = p.alpha[first + e];
@@ -554,6 +557,7 @@ __global__ void __launch_bounds__(BLOCK) layer_leaky_forward(float *__restrict__
         for (int e = 0; e < NPL; ++e) {
             const float xin = __fmul_rn(__fmul_rn(kn[e], lane_get<NPL>(xv, e)), kd[e]);
             v[e] = __fadd_rn(__fmul_rn(v[e], a[e]), xin);
+            part += v[e];
             lane_put<NPL>(o, e, v[e]);
         }
         return o;
@@ -568,6 +572,8 @@ __global__ void __launch_bounds__(BLOCK) layer_leaky_forward(float *__restrict__
         const Rsrc r = make_rsrc(op + t0 * M);
 #pragma unroll
         for (int u = 0; u < U; ++u) IO::store(advance(buf[u]), r, voff, u * step_bytes);
+        my_sum += static_cast<double>(part);
+        part = 0.f;
     };
     const int64_t pairs = T / (2 * U);
     V bufa[U], bufb[U];
@@ -584,8 +590,16 @@ __global__ void __launch_bounds__(BLOCK) layer_leaky_forward(float *__restrict__
         const V xv = IO::load(make_rsrc(xp + t * M), voff, 0u);
         IO::store(advance(xv), make_rsrc(op + t * M), voff, 0u);
     }
+    my_sum += static_cast<double>(part);
 #pragma unroll
     for (int e = 0; e < NPL; ++e) v_last[first + e] = v[e];
+    }
+    if (out_sum) {
+        // wave reduction, then one atomic per wave
+#pragma unroll
+        for (int off = WAVE / 2; off > 0; off >>= 1) my_sum += __shfl_xor(my_sum, off, WAVE);
+        if ((threadIdx.x & (WAVE - 1)) == 0 && my_sum != 0.0) atomicAdd(out_sum, my_sum);
+    }
 }
 
 // g_t = alpha g_{t+1} + grad_out_t (+ grad_v_last at the last step)
@@ -891,9 +905,9 @@ EXODUS_API int exodus_layer_lif_backward(float *grad_input, float *alpha_mem_gra
 #undef EXODUS_BWD
 }
 
-EXODUS_API int exodus_layer_leaky_forward(float *out, float *v_last, const float *input, const float *vmem_initial,
-                                          const float *alpha, int decay_early, int norm_input, int64_t batch,
-                                          int64_t t, int64_t neurons, void *stream)
+EXODUS_API int exodus_layer_leaky_forward(float *out, float *v_last, double *out_sum, const float *input,
+                                          const float *vmem_initial, const float *alpha, int decay_early,
+                                          int norm_input, int64_t batch, int64_t t, int64_t neurons, void *stream)
 {
     if (bad3(batch, t, neurons)) return hipErrorInvalidValue;
     if (batch == 0 || t == 0 || neurons == 0) return hipSuccess;
@@ -910,11 +924,11 @@ EXODUS_API int exodus_layer_leaky_forward(float *out, float *v_last, const float
     const dim3 grid(static_cast<unsigned>(blocks_per_batch * batch)), block(BLOCK);
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (npl == 4)
-        hipLaunchKernelGGL((layer_leaky_forward<4>), grid, block, 0, s, out, v_last, input, p, blocks_per_batch, t, neurons);
+        hipLaunchKernelGGL((layer_leaky_forward<4>), grid, block, 0, s, out, v_last, out_sum, input, p, blocks_per_batch, t, neurons);
     else if (npl == 2)
-        hipLaunchKernelGGL((layer_leaky_forward<2>), grid, block, 0, s, out, v_last, input, p, blocks_per_batch, t, neurons);
+        hipLaunchKernelGGL((layer_leaky_forward<2>), grid, block, 0, s, out, v_last, out_sum, input, p, blocks_per_batch, t, neurons);
     else
-        hipLaunchKernelGGL((layer_leaky_forward<1>), grid, block, 0, s, out, v_last, input, p, blocks_per_batch, t, neurons);
+        hipLaunchKernelGGL((layer_leaky_forward<1>), grid, block, 0, s, out, v_last, out_sum, input, p, blocks_per_batch, t, neurons);
     return static_cast<int>(hipGetLastError());
 }
 

@@ -21,7 +21,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("EXODUS_HIP_LIBRARY") or os.path.join(_HERE, "libexodus_hip.so")
 
 SURR_TENSOR, SURR_SINGLE_EXP, SURR_PERIODIC_EXP, SURR_HEAVISIDE = 0, 1, 2, 3
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 _p = ctypes.c_void_p
 _i64 = ctypes.c_int64
@@ -46,7 +46,7 @@ _SIGNATURES = {
     "exodus_layer_checkpoint_interval": ([], _int),
     "exodus_layer_lif_forward": ([_p] * 16 + [_int, _int, _int, _int, _i64, _i64, _i64, _p], _int),
     "exodus_layer_lif_backward": ([_p] * 18 + [_int, _int, _int, _int, _int, _f, _f, _i64, _i64, _i64, _p], _int),
-    "exodus_layer_leaky_forward": ([_p] * 5 + [_int, _int, _i64, _i64, _i64, _p], _int),
+    "exodus_layer_leaky_forward": ([_p] * 6 + [_int, _int, _i64, _i64, _i64, _p], _int),
     "exodus_layer_leaky_backward": ([_p] * 9 + [_int, _int, _i64, _i64, _i64, _p], _int),
 }
 
@@ -509,8 +509,9 @@ def layerLifBackward(gradSpikes, gradVLast, gradILast, input, ckptV, ckptI, vmem
 
 
 def layerLeakyForward(input, vmemInitial, alpha, decayEarly: bool, normInput: bool,
-                      stateShape: Optional[tuple] = None):
-    """Leaky-integrator layer on (batch, time, neurons): returns (out, v_last)."""
+                      stateShape: Optional[tuple] = None, wantSum: bool = False):
+    """Leaky-integrator layer on (batch, time, neurons): returns (out, v_last), or with ``wantSum``
+    (out, v_last, out_sum) where out_sum is a float64 scalar holding the sum of all outputs."""
     _btm(input, "input")
     b, t, m = input.shape
     n = b * m
@@ -521,13 +522,14 @@ def layerLeakyForward(input, vmemInitial, alpha, decayEarly: bool, normInput: bo
         raise RuntimeError(f"stateShape {state_shape} does not hold {n} neurons")
     out = torch.empty_like(input)
     v_last = torch.empty(state_shape, dtype=torch.float32, device=input.device)
+    out_sum = torch.zeros((), dtype=torch.float64, device=input.device) if wantSum else None
     if t == 0:
         v_last.copy_(vmemInitial.reshape(state_shape))
     with torch.cuda.device(input.device):
-        _check(lib.exodus_layer_leaky_forward(_ptr(out), _ptr(v_last), _ptr(input), _ptr(vmemInitial), _ptr(alpha),
-                                              int(bool(decayEarly)), int(bool(normInput)), b, t, m, _stream(input)),
-               "exodus_layer_leaky_forward")
-    return out, v_last
+        _check(lib.exodus_layer_leaky_forward(_ptr(out), _ptr(v_last), _ptr(out_sum), _ptr(input), _ptr(vmemInitial),
+                                              _ptr(alpha), int(bool(decayEarly)), int(bool(normInput)), b, t, m,
+                                              _stream(input)), "exodus_layer_leaky_forward")
+    return (out, v_last, out_sum) if wantSum else (out, v_last)
 
 
 def layerLeakyBackward(gradOut, gradVLast, out, input, vmemInitial, alpha, decayEarly: bool, normInput: bool,

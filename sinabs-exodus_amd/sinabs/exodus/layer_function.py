@@ -36,8 +36,9 @@ class SpikingLayerFunction(torch.autograd.Function):
         state_shape: Optional[tuple] = None,
     ):
         """Returns ``(spikes (batch,time,neurons), v_mem_last, i_syn_last | None, spike_total)``;
-        ``v_mem_last`` is the potential after the last reset, ``spike_total`` a float64 scalar
-        (not differentiable).  The final states come as flat vectors, or in ``state_shape`` if given."""
+        ``v_mem_last`` is the potential after the last reset, ``spike_total`` a float64 scalar (the sum
+        of ``spikes``; a gradient arriving at it is added to every element of the gradient of
+        ``spikes``).  The final states come as flat vectors, or in ``state_shape`` if given."""
         kind, p0, p1 = classify_surrogate(surrogate_grad_fn)
         if kind == _hip.SURR_TENSOR:
             raise ValueError("surrogate_grad_fn is not one the layer kernel can evaluate")
@@ -66,13 +67,12 @@ class SpikingLayerFunction(torch.autograd.Function):
             if apply_min:
                 saved.append(min_v_mem)
             ctx.save_for_backward(*saved)
-        ctx.mark_non_differentiable(res["spike_sum"])
         if syn:
             return res["spikes"], res["v_last"], res["i_last"], res["spike_sum"]
         return res["spikes"], res["v_last"], None, res["spike_sum"]
 
     @staticmethod
-    def backward(ctx, grad_spikes, grad_v_last, grad_i_last, _grad_total):
+    def backward(ctx, grad_spikes, grad_v_last, grad_i_last, grad_total):
         syn, apply_min, max_spikes, decay_early, norm_input, kind, p0, p1 = ctx.cfg
         saved = list(ctx.saved_tensors)
         inp, ckpt_v, v_mem_init, alpha_mem, membrane_subtract, threshold = saved[:6]
@@ -82,10 +82,12 @@ class SpikingLayerFunction(torch.autograd.Function):
             ckpt_i, i_syn_init, alpha_syn = rest[:3]
             rest = rest[3:]
         min_v_mem = rest[0] if apply_min else None
-        if grad_spikes is None and grad_v_last is None and grad_i_last is None:
+        if grad_spikes is None and grad_v_last is None and grad_i_last is None and grad_total is None:
             return (None,) * 13
         if grad_spikes is None:
             grad_spikes = torch.zeros_like(inp)
+        if grad_total is not None:                  # d(sum of spikes) / d(spike) = 1 for every element
+            grad_spikes = grad_spikes + grad_total.to(grad_spikes.dtype)
         cont = lambda x: None if x is None else x.contiguous()
         grad_input, g_am, g_as, g_v0, g_i0 = _hip.layerLifBackward(
             cont(grad_spikes), cont(grad_v_last), cont(grad_i_last) if syn else None, inp, ckpt_v, ckpt_i,
@@ -101,36 +103,37 @@ class LeakyLayerFunction(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, inp, alpha, v_mem_init, decay_early: bool, norm_input: bool, state_shape=None):
-        """Returns ``(out (batch,time,neurons), v_mem_last)``."""
+        """Returns ``(out (batch,time,neurons), v_mem_last, out_total)``; ``out_total`` is the float64
+        sum of ``out`` (a gradient arriving at it is added to every element of the gradient of ``out``)."""
         if inp.ndim != 3:
             raise ValueError("'inp' must be 3D, (batch, time, neurons)")
         if not inp.is_contiguous():
             raise ValueError("'inp' has to be contiguous.")
-        out, v_last = _hip.layerLeakyForward(inp, v_mem_init, alpha, decay_early, norm_input, stateShape=state_shape)
-        ctx.cfg = (bool(decay_early), bool(norm_input), alpha.requires_grad)
+        out, v_last, total = _hip.layerLeakyForward(inp, v_mem_init, alpha, decay_early, norm_input,
+                                                    stateShape=state_shape, wantSum=True)
+        ctx.cfg = (bool(decay_early), bool(norm_input), alpha.requires_grad, tuple(inp.shape))
         ctx.set_materialize_grads(False)
         if alpha.requires_grad:
             need_x = decay_early or norm_input
             ctx.save_for_backward(alpha, v_mem_init, out, inp if need_x else None)
         else:
             ctx.save_for_backward(alpha)
-        return out, v_last
+        return out, v_last, total
 
     @staticmethod
-    def backward(ctx, grad_out, grad_v_last):
-        decay_early, norm_input, need_alpha = ctx.cfg
+    def backward(ctx, grad_out, grad_v_last, grad_total):
+        decay_early, norm_input, need_alpha, shape = ctx.cfg
         if need_alpha:
             alpha, v_mem_init, out, inp = ctx.saved_tensors
         else:
             (alpha,) = ctx.saved_tensors
             v_mem_init = out = inp = None
-        if grad_out is None and grad_v_last is None:
+        if grad_out is None and grad_v_last is None and grad_total is None:
             return (None,) * 6
         if grad_out is None:
-            shape = out.shape if out is not None else None
-            if shape is None:
-                raise RuntimeError("gradient of the final state alone needs the output's shape")
             grad_out = torch.zeros(shape, dtype=torch.float32, device=alpha.device)
+        if grad_total is not None:
+            grad_out = grad_out + grad_total.to(grad_out.dtype)
         cont = lambda x: None if x is None else x.contiguous()
         grad_input, grad_alpha, grad_init = _hip.layerLeakyBackward(
             cont(grad_out), cont(grad_v_last), out, inp, v_mem_init, alpha, decay_early, norm_input, need_alpha)

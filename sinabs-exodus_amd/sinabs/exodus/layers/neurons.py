@@ -227,7 +227,7 @@ class LIF(LIFBase):
         if not self.is_state_initialised() or not self.state_has_shape(state_shape):
             self.init_state_with_shape(state_shape)
         alpha_mem = expand_to_1d_contiguous(self.alpha_mem_calculated, state_shape, self.v_mem.device)
-        out, v_last = LeakyLayerFunction.apply(
+        out, v_last, total = LeakyLayerFunction.apply(
             input_data.reshape(batch_size, time_steps, -1).contiguous(),
             alpha_mem,
             self.v_mem.flatten().contiguous(),
@@ -238,7 +238,7 @@ class LIF(LIFBase):
         out = out.reshape(input_data.shape)
         self.recordings = {"v_mem": out} if self.record_states else dict()
         self.v_mem = v_last
-        self.firing_rate = out.sum() / max(out.numel(), 1)
+        self.firing_rate = (total / max(out.numel(), 1)).float()
         return out
 
     def _forward_native(self, input_data: torch.Tensor) -> torch.Tensor:

@@ -37,7 +37,7 @@ def test_lif_basic(L):
     out = layer(x)
     assert layer.does_spike and out.shape == x.shape and not torch.isnan(out).any() and out.sum() > 0
     assert "EXODUS" in repr(layer)
-    assert layer.v_mem.shape == (10, 2, 7, 7) and 0 < float(layer.firing_rate)
+    assert layer.v_mem.shape == (10, 2, 7, 7) and 0 < layer.firing_rate.item()
 
 
 def test_lif_squeeze(L):

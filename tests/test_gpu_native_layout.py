@@ -169,3 +169,28 @@ def test_native_membrane_against_cpu_oracle_all_caps(L, cap, b, t, m, theta_sign
     assert_close_rowscaled(sc.bt_to_rows(got[0].cpu()), gi, "grad input")
     assert_close(got[3].cpu(), gv0, "grad v_init", atol=1e-5 * max(1.0, gv0.abs().max().item()))
     assert_close(got[1].cpu(), ga, "grad alpha", rtol=2e-4, atol=2e-5 * max(1.0, ga.abs().max().item()))
+
+
+@pytest.mark.parametrize("kind", ["lif", "synaptic", "expleak"])
+def test_firing_rate_carries_gradient_like_the_reference(L, kind):
+    """The reference computes ``firing_rate = output.sum() / output.numel()`` with autograd
+    (layers/lif.py:305), so a loss on it reaches the input; the kernels hand the sum out as a
+    differentiable scalar instead of reading the output again."""
+    el, act, _ = L
+    kw = dict(tau_mem=12.0, train_alphas=True)
+    if kind == "expleak":
+        native, rows = pair(el, el.ExpLeak, **kw)
+    else:
+        native, rows = pair(el, el.LIF, tau_syn=5.0 if kind == "synaptic" else None, min_v_mem=-0.5, **kw)
+    data = (torch.rand(3, 45, 70, generator=gen(8)) * 6 - 1).cuda()
+    xa = data.clone().requires_grad_(True); xb = data.clone().requires_grad_(True)
+    a = native(xa); b = rows(xb)
+    w = torch.rand(a.shape, generator=gen(9)).cuda()
+    ((a * w).sum() * 0.01 + 3.0 * native.firing_rate).backward()
+    ((b * w).sum() * 0.01 + 3.0 * rows.firing_rate).backward()
+    assert torch.allclose(native.firing_rate, rows.firing_rate, rtol=1e-5, atol=1e-7)
+    assert xa.grad.abs().sum() > 0
+    assert_close(xa.grad, xb.grad, "grad input through firing_rate")
+    for (k, p), (_, q) in zip(native.named_parameters(), rows.named_parameters()):
+        if q.grad is not None:
+            assert_close(p.grad, q.grad, f"grad {k}", rtol=1e-4, atol=2e-5)
