@@ -230,6 +230,39 @@ def cpu_baseline(key, torch, budget_s=12.0):
                        f"(per-step torch loop + autograd, {threads} threads)")
 
 
+def measure_ceilings(args, torch, hip, dev):
+    """GB/s of data-movement-only kernels on tensors of the chosen workload's shape."""
+    w = WORKLOADS[args.workload]
+    B, T, M = w["batch"], w["steps"], w["neurons"]
+    n = B * T * M
+    a = torch.randn(B, T, M, device=dev); b = torch.randn(B, T, M, device=dev); out = torch.empty_like(a)
+    alpha = torch.rand(B * M, device=dev) * 0.5 + 0.4
+    zeros = torch.zeros(B * M, device=dev)
+
+    def timed(fn):
+        for _ in range(max(1, args.warmup)):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(args.steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / args.steps
+
+    res = {"workload": w["name"], "tensor_GB": n * 4 / 1e9, "peak_GBs": HBM_PEAK_GBS}
+    ms = timed(lambda: hip.probeStream(out, a))
+    res["flat_copy_1r1w"] = {"ms": ms, "GBs": n * 8 / ms / 1e6}
+    ms = timed(lambda: hip.probeStream(out, a, b))
+    res["flat_add_2r1w"] = {"ms": ms, "GBs": n * 12 / ms / 1e6}
+    ms = timed(lambda: hip.layerLeakyForward(a, zeros, alpha, False, False))
+    res["time_strided_1r1w (leaky layer forward)"] = {"ms": ms, "GBs": n * 8 / ms / 1e6}
+    ms = timed(lambda: hip.layerLeakyBackward(a, None, b, None, zeros, alpha, False, False, True))
+    res["time_strided_2r1w (leaky layer backward with alpha gradient)"] = {"ms": ms, "GBs": n * 12 / ms / 1e6}
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -244,6 +277,10 @@ def main():
                     help="also launch one plain elementwise kernel (torch.neg) over exactly 1 GiB before the timed region, so that a "
                          "counter run (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE) has a kernel of known traffic "
                          "to scale its readings by")
+    ap.add_argument("--ceilings", action="store_true",
+                    help="instead of the benchmark, measure what this machine gives kernels that only move data at the "
+                         "default workload's tensor size: a flat copy, a flat 2-read-1-write kernel, and the leaky-"
+                         "integrator layer kernels, which walk memory exactly as the spiking kernels do")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (rows shard across GPUs without exchange; "
@@ -262,6 +299,10 @@ def main():
         args.path = "rows"
         wl = build_workload(args.workload, torch, hip, act, dev)
     fwd, bwd, N, T = wl["fwd"], wl["bwd"], wl["N"], wl["T"]
+
+    if args.ceilings:
+        print(json.dumps(measure_ceilings(args, torch, hip, dev)))
+        return
 
     if args.copy_probe:
         src = torch.ones(1 << 28, device=dev)          # 2^28 floats = 1 GiB read + 1 GiB written

@@ -244,6 +244,13 @@ int exodus_spike_backward(float *input_grad, const float *surr, const float *out
                           const float *not_clipped, float alpha, float membr_subtract, int64_t n,
                           int64_t t, void *stream);
 
+/* ---- measurement aid, no counterpart in the reference ------------------------------------------
+ * dst[i] = a[i] (b == NULL) or a[i] + b[i], n floats (multiple of 4, 16-byte aligned pointers),
+ * with the same non-temporal 16-byte accesses the recurrence kernels use but consecutive addresses
+ * per block: the bandwidth this machine gives a kernel that only moves data, and a kernel of
+ * exactly known traffic to scale hardware counters by. */
+int exodus_probe_stream(float *dst, const float *a, const float *b, int64_t n, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -816,6 +816,34 @@ int dispatch_fwd(const FwdArgs &a, int npl)
 // step offsets inside a block of CKPT steps are 32-bit byte offsets
 inline bool too_wide(int64_t neurons) { return neurons >= (int64_t{1} << 25); }
 
+// ---------------------------------------------------------------------------------------------
+// streaming probes: what the memory system gives a kernel that does nothing but move floats,
+// flat (consecutive addresses per block).  Used to calibrate counters and to put the recurrence
+// kernels' bandwidth next to a ceiling measured on the same machine.
+// ---------------------------------------------------------------------------------------------
+constexpr int PROBE_PER_THREAD = 4;                            // 16-byte chunks per thread
+
+template <bool TWO_INPUTS>
+__global__ void __launch_bounds__(256) probe_stream(f32x4 *__restrict__ dst, const f32x4 *__restrict__ a,
+                                                    const f32x4 *__restrict__ b, const int64_t n_chunks)
+{
+    const int64_t base = (static_cast<int64_t>(blockIdx.x) * PROBE_PER_THREAD) * 256 + threadIdx.x;
+    f32x4 va[PROBE_PER_THREAD], vb[PROBE_PER_THREAD];
+#pragma unroll
+    for (int k = 0; k < PROBE_PER_THREAD; ++k) {
+        const int64_t i = base + k * 256;
+        if (i < n_chunks) {
+            va[k] = ld_stream(a + i);
+            if (TWO_INPUTS) vb[k] = ld_stream(b + i);
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < PROBE_PER_THREAD; ++k) {
+        const int64_t i = base + k * 256;
+        if (i < n_chunks) st_stream(TWO_INPUTS ? va[k] + vb[k] : va[k], dst + i);
+    }
+}
+
 }  // namespace
 
 extern "C" {
@@ -969,6 +997,27 @@ EXODUS_API int exodus_layer_leaky_backward(float *grad_input, float *alpha_grad,
         if (with_x) EXODUS_LK(1, true, true); else if (want_alpha) EXODUS_LK(1, true, false); else EXODUS_LK(1, false, false);
     }
 #undef EXODUS_LK
+    return static_cast<int>(hipGetLastError());
+}
+
+EXODUS_API int exodus_probe_stream(float *dst, const float *a, const float *b, int64_t n, void *stream)
+{
+    if (n < 0 || (n % 4) != 0 || !dst || !a) return hipErrorInvalidValue;
+    for (const void *q : {static_cast<const void *>(dst), static_cast<const void *>(a), static_cast<const void *>(b)})
+        if (reinterpret_cast<uintptr_t>(q) & 15u) return hipErrorInvalidValue;
+    if (n == 0) return hipSuccess;
+    const int64_t n_chunks = n / 4;
+    const int64_t blocks = (n_chunks + 256 * PROBE_PER_THREAD - 1) / (256 * PROBE_PER_THREAD);
+    if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (b)
+        hipLaunchKernelGGL((probe_stream<true>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s,
+                           reinterpret_cast<f32x4 *>(dst), reinterpret_cast<const f32x4 *>(a),
+                           reinterpret_cast<const f32x4 *>(b), n_chunks);
+    else
+        hipLaunchKernelGGL((probe_stream<false>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s,
+                           reinterpret_cast<f32x4 *>(dst), reinterpret_cast<const f32x4 *>(a),
+                           static_cast<const f32x4 *>(nullptr), n_chunks);
     return static_cast<int>(hipGetLastError());
 }
 

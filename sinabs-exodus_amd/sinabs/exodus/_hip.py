@@ -43,6 +43,7 @@ _SIGNATURES = {
     "exodus_synlif_backward": ([_p] * 17 + [_int, _int, _int, _int, _int, _f, _f, _i64, _i64, _p], _int),
     "exodus_spike_forward": ([_p, _p, _f, _f, _f, _f, _int, _int, _i64, _i64, _p], _int),
     "exodus_spike_backward": ([_p] * 4 + [_f, _f, _i64, _i64, _p], _int),
+    "exodus_probe_stream": ([_p, _p, _p, _i64, _p], _int),
     "exodus_layer_checkpoint_interval": ([], _int),
     "exodus_layer_lif_forward": ([_p] * 16 + [_int, _int, _int, _int, _i64, _i64, _i64, _p], _int),
     "exodus_layer_lif_backward": ([_p] * 18 + [_int, _int, _int, _int, _int, _f, _f, _i64, _i64, _i64, _p], _int),
@@ -402,6 +403,18 @@ def synLifBackward(gradSpikes, gradVmem, gradIsyn, vmem, isyn, vmemPostInitial, 
 # ------------------------------------------------------------------------------------------
 # layer-layout kernels: (batch, time, neurons) tensors, no transposition
 # ------------------------------------------------------------------------------------------
+
+def probeStream(dst, a, b=None) -> None:
+    """dst = a (b is None) or a + b with flat streaming accesses: a bandwidth yardstick."""
+    _dev(a, "a")
+    _dev(dst, "dst", a)
+    if b is not None:
+        _dev(b, "b", a)
+    if dst.numel() != a.numel() or (b is not None and b.numel() != a.numel()):
+        raise RuntimeError("dst, a and b must have the same number of elements")
+    with torch.cuda.device(a.device):
+        _check(lib.exodus_probe_stream(_ptr(dst), _ptr(a), _ptr(b), a.numel(), _stream(a)), "exodus_probe_stream")
+
 
 # neurons per batch element the layer-layout entry points accept (they return invalid-value beyond)
 LAYER_MAX_NEURONS = 1 << 25
