@@ -263,6 +263,58 @@ def measure_ceilings(args, torch, hip, dev):
     return res
 
 
+def measure_conv_snn(args, torch, dev):
+    """Wall clock of one forward + backward of the convolutional spiking network, PyTorch-ROCm for the
+    convolution / pooling / linear layers, this package's layers in between."""
+    import torch.nn as nn
+    import sinabs.exodus.layers as el
+    B, T = 64, 300
+
+    def network(neuron):
+        layers = [nn.Conv2d(2, 32, 3), neuron(), nn.AvgPool2d(2), nn.Conv2d(32, 64, 3), neuron(), nn.Flatten(),
+                  nn.Linear(64 * 14 * 14, 10), neuron()]
+        return nn.Sequential(*[l for l in layers if l is not None]).to(dev)
+
+    torch.manual_seed(0)
+    x = (torch.rand(B, T, 2, 34, 34, device=dev) < 0.02).float()
+    labels = torch.randint(0, 10, (B,), device=dev)
+
+    def timed(model, spiking=True):
+        def step():
+            for m in model:
+                if hasattr(m, "reset_states"):
+                    m.reset_states()
+            model.zero_grad()
+            out = model(x.flatten(0, 1))
+            if spiking:
+                loss = nn.functional.cross_entropy(out.reshape(B, T, 10).sum(1), labels)
+            else:
+                loss = out.sum()
+            loss.backward()
+        for _ in range(max(1, args.warmup)):
+            step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / args.steps * 1e3
+
+    fast = network(lambda: el.IAFSqueeze(batch_size=B))
+    with torch.no_grad():
+        for i in (0, 3, 6):
+            fast[i].weight.mul_(3.0)                # enough drive for all three layers to spike
+    res = {"workload": "C4 conv SNN fwd+bwd (B=64,T=300, 2x34x34 Bernoulli(0.02) input)",
+           "neuron_layer_rows": [64 * 32 * 32 * 32, 64 * 64 * 14 * 14, 64 * 10], "time_steps": T}
+    res["ms_layer_kernels"] = timed(fast)
+    for m in fast:
+        if hasattr(m, "native_layout"):
+            m.native_layout = False
+    res["ms_rows_functions_with_transposes"] = timed(fast)
+    res["ms_conv_pool_linear_alone"] = timed(network(lambda: None), spiking=False)
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -281,6 +333,11 @@ def main():
                     help="instead of the benchmark, measure what this machine gives kernels that only move data at the "
                          "default workload's tensor size: a flat copy, a flat 2-read-1-write kernel, and the leaky-"
                          "integrator layer kernels, which walk memory exactly as the spiking kernels do")
+    ap.add_argument("--conv-snn", action="store_true",
+                    help="instead of the benchmark, time the convolutional configuration end to end through the public "
+                         "layer API (Conv2d -> IAFSqueeze -> AvgPool -> Conv2d -> IAFSqueeze -> Flatten -> Linear -> "
+                         "IAFSqueeze, batch 64 x 300 steps, cross-entropy on spike counts): layer-layout kernels, the "
+                         "transposing (rows, time) Functions, and the convolution / pooling / linear layers alone")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (rows shard across GPUs without exchange; "
@@ -302,6 +359,9 @@ def main():
 
     if args.ceilings:
         print(json.dumps(measure_ceilings(args, torch, hip, dev)))
+        return
+    if args.conv_snn:
+        print(json.dumps(measure_conv_snn(args, torch, dev)))
         return
 
     if args.copy_probe:
