@@ -97,13 +97,15 @@ __device__ __forceinline__ float spike_count(float v, float theta, unsigned cap)
 // about |argument| * 6e-8).
 struct SurrConst { float a, b; };
 
+constexpr float NEG_LOG2_E = -1.44269504088896340736f;         // exp(-x) = exp2(x * NEG_LOG2_E)
+
 template <int KIND>
 __device__ __forceinline__ SurrConst surrogate_consts(float theta, float p0, float p1)
 {
     SurrConst k;
     if (KIND == EXODUS_SURR_SINGLE_EXP) {
         const float w = __fmul_rn(theta, p0);                 // p1/(theta p0) * exp(-|v - theta| / (theta p0))
-        k.a = __fdiv_rn(1.f, w);
+        k.a = __fdiv_rn(NEG_LOG2_E, w);
         k.b = __fdiv_rn(p1, w);
     } else if (KIND == EXODUS_SURR_PERIODIC_EXP) {
         k.a = __fmul_rn(theta, 0.5f);                          // p1 * exp(-|u - theta/2| / p0) / theta
@@ -115,15 +117,17 @@ __device__ __forceinline__ SurrConst surrogate_consts(float theta, float p0, flo
     return k;
 }
 
+// exp() is the hardware's base-2 exponential with the change of base folded into the constants
+// (results below the smallest normal number come out as 0, which no gradient notices).
 template <int KIND>
 __device__ __forceinline__ float surrogate(float v, float theta, float inv_p0, SurrConst k)
 {
     if (KIND == EXODUS_SURR_SINGLE_EXP) {
-        return k.b * __expf(-fabsf(v - theta) * k.a);
+        return k.b * __builtin_amdgcn_exp2f(fabsf(v - theta) * k.a);
     } else if (KIND == EXODUS_SURR_PERIODIC_EXP) {
         float u = v - k.a;
         if (v >= theta) u = fmodf(u, theta);                 // u > 0 here, so fmod == floor-mod
-        return k.b * __expf(-fabsf(u - k.a) * inv_p0);
+        return k.b * __builtin_amdgcn_exp2f(fabsf(u - k.a) * (NEG_LOG2_E * inv_p0));
     } else {
         return v >= k.a ? k.b : 0.f;
     }

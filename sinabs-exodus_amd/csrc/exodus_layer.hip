@@ -397,39 +397,40 @@ layer_lif_backward(
     cc.two = p.cap >= 2u ? 2.f : cc.one;
     Neuron nr;
     neuron_load<SYN, CAPK>(nr, p, row);
-    const float amc = __fmul_rn(nr.am, nr.c);
     const float xg = (SYN && p.decay_early) ? nr.as : 1.0f;   // factor between mu and grad_x
+    const bool pair_new = p.decay_early != 0;                  // the synapse sum pairs i_t with mu_t (else mu_{t+1})
     const SurrConst sk = surrogate_consts<KIND>(nr.th, p0, p1);
-    const float gvl = grad_v_last ? grad_v_last[row] : 0.f;
-    const float gil = (SYN && grad_i_last) ? grad_i_last[row] : 0.f;
 
+    // Running adjoints.  Besides lambda_{t+1} and mu_{t+1} themselves the walk carries what reaches the
+    // step below them, h = a_mem lambda_{t+1} and hm = a_syn mu_{t+1}: a gradient arriving at the final
+    // states is then nothing but their initial value (the final potential is vpost_{T-1}, whose
+    // gradient enters v_{T-1} with the same factor 1 - c s_{T-1} as a_mem lambda_T would), and no step
+    // needs a special case.
     float lam = 0.f, mu = 0.f;
-    TileSum acc_m, acc_s;
+    float h = grad_v_last ? grad_v_last[row] : 0.f;
+    float hm = (SYN && grad_i_last) ? grad_i_last[row] : 0.f;
+    TileSum acc_m, acc_n, acc_s;                               // sums of lambda_{t+1} vpost_t, lambda_t i_t, mu i
     acc_m.clear();
+    acc_n.clear();
     acc_s.clear();
 
-    for (int64_t j = n_ck - 1; j >= 0; --j) {
+    // One block of CKPT steps: load, rebuild forward from the checkpoint, walk in reverse, store.
+    // GUARD = the block may end before CKPT steps (only the newest block of a sequence can).
+    auto block = [&](const int64_t j, auto guard) {
+        constexpr bool GUARD = decltype(guard)::value;
         const int64_t t0 = j * CKPT;
-        const int len = (T - t0) < CKPT ? static_cast<int>(T - t0) : CKPT;
+        const int len = GUARD ? static_cast<int>(T - t0) : CKPT;
         float xr[CKPT], gr[CKPT], vr[CKPT];
         {
-            // always CKPT loads per tensor (in the one partial block, steps past the end re-read the
-            // last step): a constant number of loads in flight lets each use wait for its own load
+            // always CKPT loads per tensor (steps past the end re-read the last step): a constant number
+            // of loads in flight lets each use wait for its own load only
             const Rsrc rx = make_rsrc(xp + t0 * M), rg = make_rsrc(gp + t0 * M);
-            if (len == CKPT) {
+            const unsigned last = static_cast<unsigned>(len - 1);
 #pragma unroll
-                for (int k = 0; k < CKPT; ++k) {
-                    xr[k] = IO::load(rx, voff, k * step_bytes);
-                    gr[k] = IO::load(rg, voff, k * step_bytes);
-                }
-            } else {
-                const unsigned last = static_cast<unsigned>(len - 1);
-#pragma unroll
-                for (int k = 0; k < CKPT; ++k) {
-                    const unsigned so = (k < last ? k : last) * step_bytes;
-                    xr[k] = IO::load(rx, voff, so);
-                    gr[k] = IO::load(rg, voff, so);
-                }
+            for (int k = 0; k < CKPT; ++k) {
+                const unsigned so = (GUARD ? (k < last ? k : last) : k) * step_bytes;
+                xr[k] = IO::load(rx, voff, so);
+                gr[k] = IO::load(rg, voff, so);
             }
         }
         nr.vpost = ld_stream(cvp + j * M + lane_off);
@@ -439,7 +440,7 @@ layer_lif_backward(
         // was normalised and fed to the membrane; without synapse that is the input itself)
 #pragma unroll
         for (int k = 0; k < CKPT; ++k)
-            if (k < len) {
+            if (!GUARD || k < len) {
                 const float v = neuron_advance<SYN>(nr, xr[k]);
                 nr.vpost = __fsub_rn(v, __fmul_rn(spike_count_fast<CAPK>(v, nr, cc), nr.c));
                 vr[k] = v;
@@ -450,27 +451,22 @@ layer_lif_backward(
 #pragma unroll
         for (int kq = 0; kq < CKPT; ++kq) {
             const int k = CKPT - 1 - kq;
-            if (k < len) {
+            if (!GUARD || k < len) {
                 const float v = vr[k], cur_i = xr[k];
                 const float sg = surrogate<KIND>(v, nr.th, inv_p0, sk);
-                float g;
-                if (t0 + k == T - 1 && grad_v_last) {
-                    g = __fadd_rn(__fmul_rn(sg, __fsub_rn(gr[k], __fmul_rn(nr.c, gvl))), gvl);
-                } else {
-                    g = __fmul_rn(sg, gr[k]);
-                }
                 const float vpost = __fsub_rn(v, __fmul_rn(nr.c, spike_count_fast<CAPK>(v, nr, cc)));
                 acc_m.add(lam, vpost);                          // lambda_{t+1} * vpost_t
-                if (SYN && !p.decay_early) acc_s.add(mu, cur_i);   // mu_{t+1} * i_t
-                const float f = __fsub_rn(nr.am, __fmul_rn(amc, sg));
-                const float l = __fadd_rn(g, __fmul_rn(f, lam));
+                const float through = __fsub_rn(1.0f, __fmul_rn(nr.c, sg));   // d vpost_t / d v_t
+                const float l = __fadd_rn(__fmul_rn(sg, gr[k]), __fmul_rn(through, h));
                 lam = v > nr.lo ? l : 0.f;                      // clamped (or NaN) steps pass nothing on
-                if (p.norm_input) acc_m.sub(lam, cur_i);
-                float du = __fmul_rn(lam, nr.k);
+                h = __fmul_rn(nr.am, lam);
+                acc_n.add(lam, cur_i);                          // lambda_t * i_t
+                const float du = __fmul_rn(lam, nr.k);
                 if (SYN) {
-                    if (t0 + k == T - 1) du = __fadd_rn(du, gil);
-                    mu = __fadd_rn(__fmul_rn(mu, nr.as), du);
-                    if (p.decay_early) acc_s.add(mu, cur_i);    // mu_t * i_t
+                    const float mu_next = mu;
+                    mu = __fadd_rn(hm, du);
+                    hm = __fmul_rn(nr.as, mu);
+                    acc_s.add(pair_new ? mu : mu_next, cur_i);
                     gr[k] = __fmul_rn(mu, xg);
                 } else {
                     gr[k] = du;
@@ -481,18 +477,26 @@ layer_lif_backward(
             const Rsrc ro = make_rsrc(op + t0 * M);
 #pragma unroll
             for (int k = 0; k < CKPT; ++k)
-                if (k < len) IO::store(gr[k], ro, voff, k * step_bytes);
+                if (!GUARD || k < len) IO::store(gr[k], ro, voff, k * step_bytes);
         }
         acc_m.fold();
+        acc_n.fold();
         acc_s.fold();
-    }
+    };
 
-    if (v_init_grad) v_init_grad[row] = __fmul_rn(nr.am, lam);
-    if (SYN && i_init_grad) i_init_grad[row] = __fmul_rn(nr.as, mu);
+    int64_t j = n_ck - 1;
+    if (T - j * CKPT < CKPT) {
+        block(j, std::true_type{});
+        --j;
+    }
+    for (; j >= 0; --j) block(j, std::false_type{});
+
+    if (v_init_grad) v_init_grad[row] = h;
+    if (SYN && i_init_grad) i_init_grad[row] = hm;
     if (alpha_mem_grad) {
         acc_m.add(lam, p.v_init[row]);
         acc_m.fold();
-        alpha_mem_grad[row] = static_cast<float>(acc_m.total);
+        alpha_mem_grad[row] = static_cast<float>(p.norm_input ? acc_m.total - acc_n.total : acc_m.total);
     }
     if (SYN && alpha_syn_grad) {
         if (p.decay_early) {
@@ -733,6 +737,9 @@ inline int pick_neurons_per_lane(int64_t batch, int64_t neurons, unsigned align,
         cus = 256;
     const int64_t wanted_lanes = static_cast<int64_t>(cus) * waves_per_cu * WAVE;
     const int64_t n = batch * neurons;
+#ifdef EXODUS_FORCE_NPL
+    if (EXODUS_FORCE_NPL <= widest) widest = EXODUS_FORCE_NPL;
+#endif
     if (widest >= 4 && (neurons % 4) == 0 && (align % 16) == 0 && n / 4 >= wanted_lanes) return 4;
     if (widest >= 2 && (neurons % 2) == 0 && (align % 8) == 0 && n / 2 >= wanted_lanes) return 2;
     return 1;
