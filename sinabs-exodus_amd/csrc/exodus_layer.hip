@@ -30,6 +30,9 @@ namespace {
 #ifndef EXODUS_LAYER_BLOCK
 #define EXODUS_LAYER_BLOCK 256        // lanes per block of the kernels that hold several neurons per lane
 #endif
+#ifndef EXODUS_LIF_FWD_WIDEST
+#define EXODUS_LIF_FWD_WIDEST 2       // most neurons per lane of the spiking forward kernel
+#endif
 #ifndef EXODUS_LAYER_BWD_BLOCK
 #define EXODUS_LAYER_BWD_BLOCK 256    // lanes per block of the spiking backward kernel (one neuron per lane)
 #endif
@@ -205,8 +208,8 @@ __device__ __forceinline__ float spike_count_fast(float v, const Neuron &n, cons
 // ---------------------------------------------------------------------------------------------
 // forward
 // ---------------------------------------------------------------------------------------------
-// Time is walked in blocks of CKPT = 2 * FWD_UNROLL steps.  Two register buffers of FWD_UNROLL
-// steps alternate: while one is consumed the loads of the other are in flight.  Every fetch issues
+// Time is walked in blocks of CKPT steps = an even number of stages of FWD_UNROLL steps.  Two
+// register buffers of one stage each alternate: while one is consumed the loads of the other are in flight.  Every fetch issues
 // the same number of loads (past the end it re-reads the last step), so the number of outstanding
 // loads at each wait is a compile-time constant.  A last, partial block runs through a guarded copy
 // of the same code.
@@ -217,7 +220,8 @@ __global__ void __launch_bounds__(BLOCK) layer_lif_forward(
     const float *__restrict__ x, const LayerConsts p, const int64_t blocks_per_batch, const int64_t T,
     const int64_t M)
 {
-    static_assert(2 * FWD_UNROLL == CKPT, "two pipeline stages per checkpoint interval");
+    constexpr int STAGES = CKPT / FWD_UNROLL;                 // pipeline stages per checkpoint interval
+    static_assert(STAGES * FWD_UNROLL == CKPT && STAGES % 2 == 0, "an even number of stages per checkpoint interval");
     typedef typename Vec<NPL>::type V;
     typedef BufIO<NPL> IO;
     // A block works inside one batch element, so all bases are block-uniform.
@@ -321,19 +325,20 @@ __global__ void __launch_bounds__(BLOCK) layer_lif_forward(
         fetch(bufa, 0);
         for (int64_t j = 0; j < n_full; ++j) {
             const int64_t t0 = j * CKPT;
-            fetch(bufb, t0 + FWD_UNROLL);
             checkpoint(j);
-            compute(bufa, t0, std::false_type{});
-            fetch(bufa, t0 + CKPT);                           // next block, or the start of the partial one
-            compute(bufb, t0 + FWD_UNROLL, std::false_type{});
+#pragma unroll
+            for (int s = 0; s < STAGES; s += 2) {
+                fetch(bufb, t0 + (s + 1) * FWD_UNROLL);
+                compute(bufa, t0 + s * FWD_UNROLL, std::false_type{});
+                fetch(bufa, t0 + (s + 2) * FWD_UNROLL);       // next pair, next block, or the start of the partial block
+                compute(bufb, t0 + (s + 1) * FWD_UNROLL, std::false_type{});
+            }
         }
-        if (n_full * CKPT < T) {                              // partial block: bufa holds its first steps
-            const int64_t t0 = n_full * CKPT;
+        if (n_full * CKPT < T) {                              // partial block: bufa holds its first stage
             checkpoint(n_full);
-            compute(bufa, t0, std::true_type{});
-            if (t0 + FWD_UNROLL < T) {
-                fetch(bufa, t0 + FWD_UNROLL);
-                compute(bufa, t0 + FWD_UNROLL, std::true_type{});
+            for (int64_t t0 = n_full * CKPT; t0 < T; t0 += FWD_UNROLL) {
+                if (t0 > n_full * CKPT) fetch(bufa, t0);
+                compute(bufa, t0, std::true_type{});
             }
         }
         my_spikes += static_cast<double>(part);
@@ -816,6 +821,9 @@ template <bool SYN>
 int dispatch_fwd(const FwdArgs &a, int npl)
 {
     if (a.v_rec || a.i_rec) return launch_fwd<SYN, 1, 0, true>(a);
+#if EXODUS_LIF_FWD_WIDEST >= 4
+    if (npl == 4) return dispatch_fwd_cap<SYN, 4>(a);
+#endif
     if (npl == 2) return dispatch_fwd_cap<SYN, 2>(a);
     return dispatch_fwd_cap<SYN, 1>(a);
 }
@@ -889,7 +897,7 @@ EXODUS_API int exodus_layer_lif_forward(float *out_spikes, float *out_vmem_rec, 
     // two neurons per lane at most: with four the spiking kernel needs so many registers for its two
     // load buffers that only two waves fit a SIMD, and it measures slower than two neurons, three waves
     const int npl = pick_neurons_per_lane(
-        batch, neurons, common_alignment({input, out_spikes, out_vmem_rec, out_isyn_rec, ckpt_v, ckpt_i}), 2, 16);
+        batch, neurons, common_alignment({input, out_spikes, out_vmem_rec, out_isyn_rec, ckpt_v, ckpt_i}), EXODUS_LIF_FWD_WIDEST, 16);
     FwdArgs a{out_spikes, out_vmem_rec, out_isyn_rec, ckpt_v, ckpt_i, v_last, i_last, spike_sum, input, p,
               batch, t, neurons, static_cast<hipStream_t>(stream)};
     return syn ? dispatch_fwd<true>(a, npl) : dispatch_fwd<false>(a, npl);
