@@ -45,7 +45,7 @@ WORKLOADS = {
 # reading of a plain copy of known size); bytes per launch of the dominant kernel, or None.
 MEASURED_TRAFFIC = {
     # FETCH_SIZE x2 + WRITE_SIZE x1 (KiB), factors from the 1 GiB probe kernel
-    ("c5", "exodus_layer_lif_backward"): 25.73e9,
+    ("c5", "exodus_layer_lif_backward"): 25.74e9,
     ("c5", "exodus_layer_lif_forward"): 17.34e9,
     ("c5", "exodus_synlif_backward"): 33.79e9,
     ("c5", "exodus_synlif_forward"): 33.64e9,
