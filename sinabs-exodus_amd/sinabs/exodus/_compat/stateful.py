@@ -9,7 +9,7 @@ layers/iaf.py:83-93; layers/exp_leak.py:64-72; conversion.py:30,54) so that ``st
 Behaviour beyond those call sites is restated from memory of sinabs 1.2-2.0.
 """
 from copy import deepcopy
-from typing import Callable, Optional, Tuple, Union
+from typing import Callable, Optional, Union
 
 import torch
 import torch.nn as nn
