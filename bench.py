@@ -216,18 +216,66 @@ def cpu_baseline(key, torch, budget_s=12.0):
             out, _, _ = sc.lif_forward(x, a_m, None, {"v_mem": torch.zeros(1, m)}, None, None, None, None, None,
                                        False, spiking=False)
         out.sum().backward()
-        return time.perf_counter() - t0
+        dt = time.perf_counter() - t0
+        alphas = a_m if key != "c1" else None
+        return dt, x, out.detach(), x.grad, alphas
 
     m = min(w["batch"] * w["neurons"], 4096)
     run(min(m, 256))                       # warm-up of the op dispatch paths
-    dt = run(m)
+    res = run(m)
     total = w["batch"] * w["neurons"]
-    while dt < budget_s / 4 and m < total and m * T * 4 * 40 < 48e9:   # keep the autograd tape under ~48 GB
+    while res[0] < budget_s / 4 and m < total and m * T * 4 * 40 < 48e9:   # keep the autograd tape under ~48 GB
         m = min(total, m * 4)
-        dt = run(m)
+        res = run(m)
+    dt = res[0]
     return dict(value=m * T / dt, unit="neuron-timesteps/s", cores=threads, kind="port",
                 sample=f"{m} of {total} rows x {T} steps, one fwd+bwd in {dt:.2f} s "
-                       f"(per-step torch loop + autograd, {threads} threads)")
+                       f"(per-step torch loop + autograd, {threads} threads)",
+                parity_on_sample=parity_on_sample(key, torch, m, *res[1:]))
+
+
+def parity_on_sample(key, torch, m, x, out_cpu, grad_cpu, alphas):
+    """The kernels on the very rows the CPU loop just processed (grad_output = ones): fraction of rows
+    whose spike trains differ (the CPU loop rounds the synapse update in another order, so a potential
+    within rounding distance of the threshold can fall on the other side, after which the row
+    legitimately diverges) and the largest gradient error over the rows that agree."""
+    from sinabs.exodus import _hip as hip
+    dev = torch.device("cuda:0")
+    xd = x.detach().to(dev).contiguous()
+    full = lambda v: torch.full((m,), float(v), device=dev)
+    zeros = torch.zeros(m, device=dev)
+    go = torch.ones_like(xd)
+    if key == "c3":
+        a = alphas.detach().to(dev)
+        out, _ = hip.layerLeakyForward(xd, zeros, a, False, False)
+        gx = hip.layerLeakyBackward(go, None, out, None, zeros, a, False, False, True)[0]
+    else:
+        a_m = full(1.0) if key == "c1" else full(math.exp(-1 / 20.0))
+        a_s = full(math.exp(-1 / 5.0)) if key == "c5" else None
+        lo = full(-1.0) if key == "c5" else None
+        cap = {"c5": 2, "c2": 1, "c1": -1}[key]
+        norm = key != "c1"
+        f = hip.layerLifForward(xd, zeros, zeros if a_s is not None else None, a_m, a_s, full(1.0), full(1.0), lo,
+                                lo is not None, cap, True, norm)
+        out = f["spikes"]
+        gx = hip.layerLifBackward(go, None, None, xd, f["ckpt_v"], f["ckpt_i"], zeros, zeros if a_s is not None else None,
+                                  a_m, a_s, full(1.0), full(1.0), lo, lo is not None, cap, True, norm,
+                                  hip.SURR_SINGLE_EXP, 0.5, 1.0)[0]
+    out = out.cpu()[0].T                                       # (rows, time)
+    gx = gx.cpu()[0].T
+    want = out_cpu[0].T
+    gwant = grad_cpu[0].T
+    if key == "c3":
+        same = torch.ones(m, dtype=torch.bool)
+        out_err = ((out - want).abs() / (1e-5 + 1e-4 * want.abs())).max().item()
+    else:
+        same = (out == want).all(1)
+        out_err = 0.0
+    err = ((gx - gwant).abs() / (1e-5 + 1e-4 * gwant.abs()))[same]
+    return {"rows": m, "rows_with_differing_spikes": int((~same).sum()), "fraction": float((~same).float().mean()),
+            "output_error_in_tolerances": out_err,
+            "grad_input_max_abs_error": float((gx - gwant).abs()[same].max()) if same.any() else None,
+            "grad_input_error_in_tolerances (rtol 1e-4, atol 1e-5)": float(err.max()) if same.any() else None}
 
 
 def measure_ceilings(args, torch, hip, dev):
