@@ -85,3 +85,24 @@ def test_replays_equal_eager_steps(el, tau_syn):
                 assert_close(grads_static[name], p.grad, f"grad {name}, input {k}", rtol=1e-5, atol=1e-6)
         active += int(want.sum().item() > 0)
     assert active == 5
+
+
+def test_kernels_run_on_the_current_stream(el):
+    """The entry points enqueue on the stream they are handed: work issued under a side stream is
+    ordered after that stream's earlier work (here a slow fill that the input depends on) and is not
+    visible to the default stream until the streams are joined."""
+    layer = el.LIF(tau_mem=10.0, tau_syn=4.0).cuda()
+    ref_layer = el.LIF(tau_mem=10.0, tau_syn=4.0).cuda()
+    base = (torch.rand(4, 60, 512, generator=gen(21)) * 3).cuda()
+    want = ref_layer(base * 2.0)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        x = base.clone()
+        for _ in range(50):                                   # a chain of dependent kernels on the side stream
+            x = x * 1.0
+        x = x * 2.0
+        got = layer(x)
+    side.synchronize()
+    assert torch.equal(got, want)
+    assert torch.equal(layer.v_mem, ref_layer.v_mem)
