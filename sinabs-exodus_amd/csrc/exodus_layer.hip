@@ -112,9 +112,16 @@ template <> struct BufIO<4> {
     {
         return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, AUX_LOAD));
     }
+    // A 16-byte store takes more than one pass to read its data registers.  The compiler keeps the
+    // next instruction from overwriting them only when the store has no SGPR offset; with one, a
+    // vector instruction that rewrites the data right behind the store corrupted the last lanes of
+    // each group of 16 on gfx950 (seen as sporadic wrong outputs when two blocks shared a compute
+    // unit).  So the step offset travels in the vector offset here and the scalar offset stays 0, and a
+    // short wait that reads the data keeps every writer away until the store has taken it.
     static __device__ __forceinline__ void store(f32x4 v, Rsrc r, unsigned voff, unsigned soff)
     {
-        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), r, voff, soff, AUX_STORE);
+        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), r, voff + soff, 0, AUX_STORE);
+        asm volatile("s_nop 1" : : "v"(v));                    // the data registers stay untouched two more cycles
     }
 };
 

@@ -145,3 +145,45 @@ def test_c5_rows_kernels_full_size_sampled(mods):
     assert_close(c(gi), wgi, "grad_input of sampled rows")
     assert_close(c(ginit), wginit, "grad_init of sampled rows")
     assert_close(c(ga), wga, "grad_alpha of sampled rows", rtol=1e-4, atol=1e-5 * t ** 0.5)
+
+
+def test_layer_kernels_index_tensors_beyond_2_31_elements(mods):
+    """(9, 2000, 131072) has 2.36e9 elements per tensor, more than a 32-bit index holds.  Neurons are
+    independent, so the last batch element computed inside the big call must equal the same batch
+    element computed alone, bit for bit, forward and backward, spiking and leaky."""
+    hip, _ = mods
+    need_gib(80)
+    B, T, M = 9, 2000, 131072
+    dev = "cuda"
+    g = torch.Generator(device=dev).manual_seed(12)
+    x = torch.randn(B, T, M, generator=g, device=dev) * 0.5 + 0.05
+    go = torch.randn(B, T, M, generator=g, device=dev)
+    full = lambda n, v: torch.full((n,), v, device=dev)
+    am, asn = math.exp(-1 / 20.0), math.exp(-1 / 5.0)
+
+    def spiking(xx, gg):
+        n = xx.shape[0] * M
+        f = hip.layerLifForward(xx, full(n, 0.0), full(n, 0.0), full(n, am), full(n, asn), full(n, 1.0), full(n, 1.0),
+                                full(n, -1.0), True, 2, True, True)
+        b = hip.layerLifBackward(gg, None, None, xx, f["ckpt_v"], f["ckpt_i"], full(n, 0.0), full(n, 0.0), full(n, am),
+                                 full(n, asn), full(n, 1.0), full(n, 1.0), full(n, -1.0), True, 2, True, True,
+                                 hip.SURR_SINGLE_EXP, 0.5, 1.0)
+        return f["spikes"], f["v_last"], b[0], b[1]
+
+    s_big, v_big, gx_big, ga_big = spiking(x, go)
+    s_one, v_one, gx_one, ga_one = spiking(x[B - 1:].contiguous(), go[B - 1:].contiguous())
+    assert torch.equal(s_big[B - 1], s_one[0]) and s_one.sum() > 0
+    assert torch.equal(v_big[(B - 1) * M:], v_one)
+    assert torch.equal(gx_big[B - 1], gx_one[0]) and torch.equal(ga_big[(B - 1) * M:], ga_one)
+    del s_big, gx_big, s_one, gx_one
+
+    def leaky(xx, gg):
+        n = xx.shape[0] * M
+        out, v_last = hip.layerLeakyForward(xx, full(n, 0.0), full(n, am), True, True)
+        gi, ga, _ = hip.layerLeakyBackward(gg, None, out, xx, full(n, 0.0), full(n, am), True, True, True)
+        return out, gi, ga
+
+    o_big, gi_big, ga_big = leaky(x, go)
+    o_one, gi_one, ga_one = leaky(x[B - 1:].contiguous(), go[B - 1:].contiguous())
+    assert torch.equal(o_big[B - 1], o_one[0]) and torch.equal(gi_big[B - 1], gi_one[0])
+    assert torch.equal(ga_big[(B - 1) * M:], ga_one)

@@ -194,3 +194,48 @@ def test_firing_rate_carries_gradient_like_the_reference(L, kind):
     for (k, p), (_, q) in zip(native.named_parameters(), rows.named_parameters()):
         if q.grad is not None:
             assert_close(p.grad, q.grad, f"grad {k}", rtol=1e-4, atol=2e-5)
+
+
+def test_wide_lane_kernels_equal_one_neuron_per_lane(L):
+    """Layers large enough for 2 or 4 neurons per lane (8- and 16-byte accesses) against the same
+    batch elements computed alone, which is small enough to run with one neuron per lane: bit for bit,
+    in every output, on repeated runs (two blocks per compute unit overlap here, which is where a
+    store whose data registers are rewritten too early shows up)."""
+    _, _, hip = L
+    dev = "cuda"
+    g = torch.Generator(device=dev).manual_seed(3)
+    full = lambda n, v: torch.full((n,), v, device=dev)
+
+    B, T, M = 4, 40, 131072                                   # leaky: 4 neurons per lane (2 with alpha gradient)
+    x = torch.randn(B, T, M, generator=g, device=dev); go = torch.randn(B, T, M, generator=g, device=dev)
+
+    def leaky(xx, gg):
+        n = xx.shape[0] * M
+        out, v_last = hip.layerLeakyForward(xx, full(n, 0.1), full(n, 0.9), True, True)
+        gi, ga, gv = hip.layerLeakyBackward(gg, None, out, xx, full(n, 0.1), full(n, 0.9), True, True, True)
+        gi2 = hip.layerLeakyBackward(gg, None, None, None, None, full(n, 0.9), True, True, False)[0]
+        return out, gi, gi2, v_last, ga, gv
+
+    for _ in range(3):
+        big = leaky(x, go)
+        for b in range(B):
+            one = leaky(x[b:b + 1].contiguous(), go[b:b + 1].contiguous())
+            for p, q in zip(big, one):
+                assert torch.equal(p[b] if p.ndim == 3 else p[b * M:(b + 1) * M], q[0] if q.ndim == 3 else q)
+
+    B, T, M = 8, 40, 65536                                    # spiking forward: 2 neurons per lane
+    x = torch.randn(B, T, M, generator=g, device=dev) * 0.8 + 0.2
+
+    def spiking(xx):
+        n = xx.shape[0] * M
+        f = hip.layerLifForward(xx, full(n, 0.0), full(n, 0.0), full(n, 0.95), full(n, 0.8), full(n, 1.0), full(n, 1.0),
+                                full(n, -1.0), True, -1, True, True)
+        return f["spikes"], f["v_last"], f["i_last"], f["ckpt_v"]
+
+    for _ in range(3):
+        big = spiking(x)
+        assert big[0].sum() > 0
+        for b in range(B):
+            one = spiking(x[b:b + 1].contiguous())
+            for p, q in zip(big, one):
+                assert torch.equal(p[b] if p.ndim == 3 else p[b * M:(b + 1) * M], q[0] if q.ndim == 3 else q)
