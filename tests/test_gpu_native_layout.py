@@ -216,12 +216,13 @@ def test_wide_lane_kernels_equal_one_neuron_per_lane(L):
         gi2 = hip.layerLeakyBackward(gg, None, None, None, None, full(n, 0.9), True, True, False)[0]
         return out, gi, gi2, v_last, ga, gv
 
-    for _ in range(3):
-        big = leaky(x, go)
-        for b in range(B):
-            one = leaky(x[b:b + 1].contiguous(), go[b:b + 1].contiguous())
-            for p, q in zip(big, one):
-                assert torch.equal(p[b] if p.ndim == 3 else p[b * M:(b + 1) * M], q[0] if q.ndim == 3 else q)
+    for nb in (B, 2):                                          # 4 batch elements: 4 neurons per lane; 2: 2 per lane
+        for _ in range(3):
+            big = leaky(x[:nb].contiguous(), go[:nb].contiguous())
+            for b in range(nb):
+                one = leaky(x[b:b + 1].contiguous(), go[b:b + 1].contiguous())
+                for p, q in zip(big, one):
+                    assert torch.equal(p[b] if p.ndim == 3 else p[b * M:(b + 1) * M], q[0] if q.ndim == 3 else q)
 
     B, T, M = 8, 40, 65536                                    # spiking forward: 2 neurons per lane
     x = torch.randn(B, T, M, generator=g, device=dev) * 0.8 + 0.2
