@@ -187,3 +187,49 @@ def test_layer_kernels_index_tensors_beyond_2_31_elements(mods):
     o_one, gi_one, ga_one = leaky(x[B - 1:].contiguous(), go[B - 1:].contiguous())
     assert torch.equal(o_big[B - 1], o_one[0]) and torch.equal(gi_big[B - 1], gi_one[0])
     assert torch.equal(ga_big[(B - 1) * M:], ga_one)
+
+
+def test_identical_batch_elements_give_identical_results_at_full_size(mods):
+    """Every element of the outputs is checked here, not a sample: all 16 batch elements of a C5-sized
+    input are copies of one another, neurons are independent, so every output must repeat 16 times bit
+    for bit -- on the layer kernels and on the (rows, time) kernels, forward and backward.  A write that
+    goes astray anywhere in 2e9 elements breaks the repetition."""
+    hip, _ = mods
+    need_gib(90)
+    B, T, M = 16, 2000, 65536
+    dev = "cuda"
+    g = torch.Generator(device=dev).manual_seed(21)
+    x = (torch.randn(1, T, M, generator=g, device=dev) * 0.5 + 0.05).expand(B, T, M).contiguous()
+    go = torch.randn(1, T, M, generator=g, device=dev).expand(B, T, M).contiguous()
+    n = B * M
+    full = lambda v: torch.full((n,), v, device=dev)
+    am, asn = math.exp(-1 / 20.0), math.exp(-1 / 5.0)
+
+    def repeats(z):
+        z = z.reshape(B, -1)
+        return bool((z == z[:1]).all())
+
+    f = hip.layerLifForward(x, full(0.0), full(0.0), full(am), full(asn), full(1.0), full(1.0), full(-1.0), True, 2,
+                            True, True)
+    assert f["spikes"].sum() > 0
+    assert repeats(f["spikes"]) and repeats(f["v_last"]) and repeats(f["i_last"]) and repeats(f["ckpt_v"])
+    b = hip.layerLifBackward(go, None, None, x, f["ckpt_v"], f["ckpt_i"], full(0.0), full(0.0), full(am), full(asn),
+                             full(1.0), full(1.0), full(-1.0), True, 2, True, True, hip.SURR_SINGLE_EXP, 0.5, 1.0)
+    assert all(repeats(t) for t in b if t is not None)
+    del f, b
+
+    out, v_last = hip.layerLeakyForward(x, full(0.0), full(am), True, True)
+    gi, ga, gv = hip.layerLeakyBackward(go, None, out, x, full(0.0), full(am), True, True, True)
+    gi2 = hip.layerLeakyBackward(go, None, None, None, None, full(am), False, False, False)[0]
+    assert repeats(out) and repeats(v_last) and repeats(gi) and repeats(ga) and repeats(gv) and repeats(gi2)
+    del out, gi, gi2
+
+    # (rows, time): row r = b * M + m, so rows repeat with period M
+    xr = x.movedim(1, 2).reshape(n, T).contiguous(); gor = go.movedim(1, 2).reshape(n, T).contiguous()
+    del x, go
+    s = torch.empty_like(xr); v = torch.empty_like(xr)
+    hip.lifForward(s, v, xr, full(0.0), full(am), full(1.0), full(1.0), full(-1.0), True, 2)
+    assert repeats(s) and repeats(v)
+    gir, gar, ginit = hip.lifBackwardFused(gor, None, v, full(0.0), full(am), full(1.0), full(1.0), full(-1.0), True, 2,
+                                           hip.SURR_SINGLE_EXP, 0.5, 1.0, needAlphaGrad=True)
+    assert repeats(gir) and repeats(gar) and repeats(ginit)
