@@ -240,3 +240,53 @@ def test_wide_lane_kernels_equal_one_neuron_per_lane(L):
             one = spiking(x[b:b + 1].contiguous())
             for p, q in zip(big, one):
                 assert torch.equal(p[b] if p.ndim == 3 else p[b * M:(b + 1) * M], q[0] if q.ndim == 3 else q)
+
+
+def test_random_configurations_forward_against_cpu_oracle(L):
+    """A seeded sweep over shapes (every remainder of the 32-step blocks and 16-step stages, odd and
+    even neuron counts), options, caps and initial states: spikes, final states and checkpoints bit
+    for bit against the oracle composed the way the reference layer composes its Functions."""
+    _, _, hip = L
+    from oracle import exodus_ref as ref
+    from oracle import sinabs_cpu as sc
+    import random
+    rnd = random.Random(1234)
+    D = lambda z: None if z is None else z.cuda()
+    for case in range(60):
+        b = rnd.choice([1, 2, 3, 5])
+        t = rnd.choice([1, 2, 15, 16, 17, 31, 32, 33, 47, 48, 49, 63, 64, 65, 95, 96, 100, 129])
+        m = rnd.choice([1, 2, 3, 6, 64, 65, 130, 256, 258, 1000])
+        syn = rnd.random() < 0.5
+        decay_early = rnd.random() < 0.5
+        norm_input = rnd.random() < 0.5
+        use_lo = rnd.random() < 0.6
+        cap = rnd.choice([-1, 1, 2, 3])
+        n = b * m
+        g = gen(1000 + case)
+        scale = (6.0 if norm_input else 0.7) * (0.5 if syn else 1.0)
+        x = torch.randn(b, t, m, generator=g) * scale + 0.3 * scale
+        am = 0.5 + 0.5 * torch.rand(n, generator=g); asn = 0.3 + 0.6 * torch.rand(n, generator=g)
+        v0 = torch.randn(n, generator=g) * 0.3; i0 = torch.randn(n, generator=g) * 0.3
+        th = 0.5 + torch.rand(n, generator=g); c = 0.3 + 0.6 * torch.rand(n, generator=g)
+        lo = -0.2 - torch.rand(n, generator=g)
+        xr = sc.bt_to_rows(x)
+        if syn:
+            xin = (xr * asn[:, None]).contiguous() if decay_early else xr
+            i_rows = ref.leaky_forward(xin, i0, asn)
+        else:
+            i_rows = xr
+        u = ((1.0 - am)[:, None] * i_rows).contiguous() if norm_input else i_rows
+        ws, wv = ref.lif_forward(u, v0, am, c, th, lo if use_lo else None, use_lo, cap)
+        res = hip.layerLifForward(D(x), D(v0), D(i0) if syn else None, D(am), D(asn) if syn else None, D(c), D(th),
+                                  D(lo) if use_lo else None, use_lo, cap, decay_early, norm_input)
+        what = f"case {case}: b={b} t={t} m={m} syn={syn} de={decay_early} norm={norm_input} lo={use_lo} cap={cap}"
+        assert torch.equal(res["spikes"].cpu(), sc.rows_to_bt(ws, b)), what
+        vpost = wv - c[:, None] * ws
+        assert torch.equal(res["v_last"].cpu(), vpost[:, -1]), what
+        if syn:
+            assert torch.equal(res["i_last"].cpu(), i_rows[:, -1]), what
+        ck = hip.checkpointInterval()
+        n_ck = (t + ck - 1) // ck
+        want_ck = torch.stack([v0] + [vpost[:, k * ck - 1] for k in range(1, n_ck)], 1)
+        assert torch.equal(res["ckpt_v"].cpu(), sc.rows_to_bt(want_ck, b)), what
+        assert float(res["spike_sum"]) == float(ws.double().sum()), what
