@@ -465,6 +465,10 @@ def layerLifForward(input, vmemPostInitial, isynInitial, alphaMem, alphaSyn, mem
                ckpt_i=new(b, n_ck, m) if (wantCheckpoints and syn) else None,
                v_rec=new(b, t, m) if wantRecords else None, i_rec=new(b, t, m) if (wantRecords and syn) else None,
                spike_sum=torch.zeros((), dtype=torch.float64, device=input.device) if wantSpikeSum else None)
+    if t == 0:                                   # nothing to integrate: the final states are the initial ones
+        res["v_last"].copy_(vmemPostInitial.reshape(state_shape))
+        if syn:
+            res["i_last"].copy_(isynInitial.reshape(state_shape))
     with torch.cuda.device(input.device):
         _check(lib.exodus_layer_lif_forward(
             _ptr(spikes), _ptr(res["v_rec"]), _ptr(res["i_rec"]), _ptr(res["ckpt_v"]), _ptr(res["ckpt_i"]),

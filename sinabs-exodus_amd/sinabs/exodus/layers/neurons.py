@@ -215,7 +215,7 @@ class LIF(LIFBase):
         if not (self.native_layout and input_data.is_cuda and input_data.dtype == torch.float32
                 and input_data.ndim >= 2):
             return False
-        if input_data[0, 0].numel() >= _hip.LAYER_MAX_NEURONS:   # the kernels keep step offsets in 32 bits
+        if int(np.prod(input_data.shape[2:])) >= _hip.LAYER_MAX_NEURONS:   # the kernels keep step offsets in 32 bits
             return False
         if self.spike_fn is None:                      # leaky integrator: the output is the state record
             return self.tau_syn_calculated is None
@@ -228,7 +228,7 @@ class LIF(LIFBase):
             self.init_state_with_shape(state_shape)
         alpha_mem = expand_to_1d_contiguous(self.alpha_mem_calculated, state_shape, self.v_mem.device)
         out, v_last, total = LeakyLayerFunction.apply(
-            input_data.reshape(batch_size, time_steps, -1).contiguous(),
+            input_data.reshape(batch_size, time_steps, int(np.prod(trailing_dim))).contiguous(),
             alpha_mem,
             self.v_mem.flatten().contiguous(),
             self.decay_early,
@@ -259,7 +259,7 @@ class LIF(LIFBase):
         else:
             membrane_subtract = expand_to_1d_contiguous(membrane_subtract, state_shape, dev)
         spikes, v_last, i_last, spike_total = SpikingLayerFunction.apply(
-            input_data.reshape(batch_size, time_steps, -1).contiguous(),
+            input_data.reshape(batch_size, time_steps, int(np.prod(trailing_dim))).contiguous(),
             alpha_mem,
             alpha_syn,
             self.v_mem.flatten().contiguous(),

@@ -290,3 +290,23 @@ def test_random_configurations_forward_against_cpu_oracle(L):
         want_ck = torch.stack([v0] + [vpost[:, k * ck - 1] for k in range(1, n_ck)], 1)
         assert torch.equal(res["ckpt_v"].cpu(), sc.rows_to_bt(want_ck, b)), what
         assert float(res["spike_sum"]) == float(ws.double().sum()), what
+
+
+def test_empty_sequences_and_batches(L):
+    """Zero time steps leave the states where they were; zero batch elements or neurons give empty
+    outputs; nothing is launched and nothing faults."""
+    el, _, hip = L
+    D = lambda z: z.cuda()
+    v0 = torch.tensor([0.3, -0.2, 0.7]); i0 = torch.tensor([0.1, 0.2, 0.3]); one = torch.ones(3)
+    x = torch.empty(1, 0, 3)
+    res = hip.layerLifForward(D(x), D(v0), D(i0), D(one * 0.9), D(one * 0.8), D(one), D(one), None, False, -1, True, True)
+    assert res["spikes"].shape == (1, 0, 3) and torch.equal(res["v_last"].cpu(), v0) and torch.equal(res["i_last"].cpu(), i0)
+    out, v_last = hip.layerLeakyForward(D(x), D(v0), D(one * 0.9), True, True)
+    assert out.shape == (1, 0, 3) and torch.equal(v_last.cpu(), v0)
+    for shape in [(0, 5, 3), (2, 5, 0)]:
+        n = shape[0] * shape[2]
+        e = torch.empty(n)
+        res = hip.layerLifForward(D(torch.empty(shape)), D(e), None, D(e), None, D(e), D(e), None, False, -1, True, True)
+        assert res["spikes"].shape == shape and res["v_last"].numel() == 0
+    layer = el.IAF().cuda()
+    assert layer(torch.empty(2, 0, 4).cuda()).shape == (2, 0, 4)
