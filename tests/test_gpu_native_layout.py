@@ -310,3 +310,31 @@ def test_empty_sequences_and_batches(L):
         assert res["spikes"].shape == shape and res["v_last"].numel() == 0
     layer = el.IAF().cuda()
     assert layer(torch.empty(2, 0, 4).cuda()).shape == (2, 0, 4)
+
+
+@pytest.mark.parametrize("mode", ["no_grad", "inference_mode", "non_contiguous", "half_input"])
+def test_inference_and_unusual_inputs(L, mode):
+    """Inference needs no checkpoints and gives the same spikes; a transposed view is made contiguous;
+    a half-precision input does not take the float32 kernels' fast path and is refused by the
+    (rows, time) Functions the way the reference refuses it (its kernels are float32 only)."""
+    el, _, _ = L
+    native, rows = pair(el, el.LIF, tau_mem=10.0, tau_syn=5.0, min_v_mem=-1.0)
+    x = (torch.rand(3, 40, 50, generator=gen(2)) * 4).cuda()
+    want = rows(x)
+    if mode == "no_grad":
+        with torch.no_grad():
+            got = native(x)
+        assert not got.requires_grad
+    elif mode == "inference_mode":
+        with torch.inference_mode():
+            got = native(x)
+    elif mode == "non_contiguous":
+        xt = x.transpose(0, 2).contiguous().transpose(0, 2)   # same values, strides of another layout
+        assert not xt.is_contiguous()
+        got = native(xt)
+    else:
+        assert not native._use_native_layout(x.half())
+        with pytest.raises((RuntimeError, ValueError, TypeError)):
+            native(x.half())
+        return
+    assert torch.equal(got, want) and torch.equal(native.v_mem, rows.v_mem)
