@@ -14,6 +14,7 @@ import torch
 from .._compat import (LIFBase, MaxSpike, MembraneSubtract, MultiSpike, SingleExponential, SingleSpike,
                        SqueezeMixin)
 from .. import _hip
+from .._validate import check_parameters
 from ..leaky import LeakyIntegrator
 from ..layer_function import LeakyLayerFunction, SpikingLayerFunction
 from ..spike import IntegrateAndFire
@@ -219,7 +220,15 @@ class LIF(LIFBase):
             return False
         if self.spike_fn is None:                      # leaky integrator: the output is the state record
             return self.tau_syn_calculated is None
+        if not self._needs_grad(input_data):           # inference: any surrogate, with or without records
+            return True
         return not self.record_states and fusable(self.surrogate_grad_fn)
+
+    def _needs_grad(self, input_data: torch.Tensor) -> bool:
+        if not torch.is_grad_enabled():
+            return False
+        return (input_data.requires_grad or any(p.requires_grad for p in self.parameters())
+                or any(b.requires_grad for b in self.buffers()))
 
     def _forward_native_leaky(self, input_data: torch.Tensor) -> torch.Tensor:
         batch_size, time_steps, *trailing_dim = input_data.shape
@@ -258,8 +267,30 @@ class LIF(LIFBase):
             membrane_subtract = spike_threshold
         else:
             membrane_subtract = expand_to_1d_contiguous(membrane_subtract, state_shape, dev)
+        flat_input = input_data.reshape(batch_size, time_steps, int(np.prod(trailing_dim))).contiguous()
+        if not self._needs_grad(input_data):
+            # nothing to differentiate: no checkpoints, and the per-step states can be written along the way
+            with torch.no_grad():
+                check_parameters([alpha_mem, alpha_syn] if has_syn else [alpha_mem], spike_threshold, min_v_mem)
+                res = _hip.layerLifForward(
+                    flat_input, self.v_mem.flatten().contiguous(),
+                    self.i_syn.flatten().contiguous() if has_syn else None, alpha_mem, alpha_syn, membrane_subtract,
+                    spike_threshold, min_v_mem, min_v_mem is not None,
+                    -1 if self.max_num_spikes_per_bin is None else int(self.max_num_spikes_per_bin),
+                    self.decay_early, self.norm_input, wantCheckpoints=False, wantRecords=self.record_states,
+                    stateShape=state_shape)
+            self.recordings = dict()
+            if self.record_states:
+                self.recordings["v_mem"] = res["v_rec"].reshape(input_data.shape)
+                if has_syn:
+                    self.recordings["i_syn"] = res["i_rec"].reshape(input_data.shape)
+            self.v_mem = res["v_last"]
+            if has_syn:
+                self.i_syn = res["i_last"]
+            self.firing_rate = (res["spike_sum"] / max(flat_input.numel(), 1)).float()
+            return res["spikes"].reshape(input_data.shape)
         spikes, v_last, i_last, spike_total = SpikingLayerFunction.apply(
-            input_data.reshape(batch_size, time_steps, int(np.prod(trailing_dim))).contiguous(),
+            flat_input,
             alpha_mem,
             alpha_syn,
             self.v_mem.flatten().contiguous(),

@@ -69,10 +69,12 @@ def test_native_iaf_squeeze_and_unknown_surrogate_fallback(L):
     native, rows = pair(el, el.IAFSqueeze, batch_size=6, min_v_mem=-1.0)
     assert torch.equal(native(x), rows(x)) and native(x).is_contiguous()
     custom = el.IAF(surrogate_grad_fn=lambda v, th: 1.0 / (1.0 + (v - th) ** 2)).cuda()
-    assert not custom._use_native_layout(x.reshape(6, 50, 2, 5, 5))
+    xg = x.reshape(6, 50, 2, 5, 5).clone().requires_grad_(True)      # with gradients these need the Functions
+    assert not custom._use_native_layout(xg)
     rec = el.IAF(record_states=True).cuda()
-    assert not rec._use_native_layout(x.reshape(6, 50, 2, 5, 5))
-    out = custom(x.reshape(6, 50, 2, 5, 5)); assert out.shape == (6, 50, 2, 5, 5)
+    assert not rec._use_native_layout(xg)
+    out = custom(xg); assert out.shape == (6, 50, 2, 5, 5)
+    out.sum().backward(); assert xg.grad is not None and bool(torch.isfinite(xg.grad).all())
 
 
 def test_native_forward_against_cpu_oracle(L):
@@ -338,3 +340,29 @@ def test_inference_and_unusual_inputs(L, mode):
             native(x.half())
         return
     assert torch.equal(got, want) and torch.equal(native.v_mem, rows.v_mem)
+
+
+@pytest.mark.parametrize("tau_syn", [None, 5.0])
+def test_inference_records_states_and_accepts_any_surrogate(L, tau_syn):
+    """Without gradients the layer kernels serve every configuration: they write the per-step states
+    themselves (``record_states``) and never evaluate the surrogate."""
+    el, act, _ = L
+    custom = lambda v, th: 1.0 / (1.0 + (v - th) ** 2)
+    kw = dict(tau_mem=12.0, tau_syn=tau_syn, min_v_mem=-0.5, record_states=True, surrogate_grad_fn=custom)
+    native, rows = pair(el, el.LIF, **kw)
+    x = (torch.rand(3, 70, 5, 8, generator=gen(4)) * 5 - 1).cuda()
+    with torch.no_grad():
+        assert native._use_native_layout(x)
+        for _ in range(2):                                     # second call continues from the first call's states
+            a = native(x); b = rows(x)
+            assert torch.equal(a, b)
+            assert torch.equal(native.recordings["v_mem"], rows.recordings["v_mem"])
+            assert torch.equal(native.v_mem, rows.v_mem) and torch.equal(native.recordings["v_mem"][:, -1], native.v_mem)
+            if tau_syn is not None:
+                assert torch.equal(native.recordings["i_syn"], rows.recordings["i_syn"])
+            assert torch.allclose(native.firing_rate, rows.firing_rate, rtol=1e-6, atol=0)
+    assert not native._use_native_layout(x.requires_grad_(True))      # with gradients: the Functions
+    with pytest.raises(ValueError):
+        bad = el.LIF(tau_mem=10.0, min_v_mem=2.0).cuda()
+        with torch.no_grad():
+            bad(x)
