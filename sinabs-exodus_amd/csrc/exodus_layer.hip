@@ -75,8 +75,15 @@ template <> __device__ __forceinline__ void lane_put<4>(f32x4 &v, int e, float x
 // arithmetic or 64-bit address registers.  num_records is set to the maximum: every access is
 // guarded by the code, not by the hardware range check.
 typedef __amdgpu_buffer_rsrc_t Rsrc;
-constexpr int AUX_LOAD = EXODUS_NT_LOAD ? 2 : 0;     // bit 1 = non-temporal
-constexpr int AUX_STORE = EXODUS_NT_STORE ? 2 : 0;
+// Cache hint of the streamed accesses (bit 1 = non-temporal).  Streaming data that nobody reads twice
+// is marked non-temporal, which measures a few percent faster; but when a step's neurons do not start
+// and end on 128-byte lines (neuron count not a multiple of 32, or a view at an odd offset) neighbouring
+// waves and blocks share lines, and a non-temporal line is dropped before the neighbour gets to it:
+// reads from memory grow by a third and partial writes appear.  Such layers use NT = false.
+template <bool NT> struct Aux {
+    static constexpr int load = (NT && EXODUS_NT_LOAD) ? 2 : 0;
+    static constexpr int store = (NT && EXODUS_NT_STORE) ? 2 : 0;
+};
 
 __device__ __forceinline__ Rsrc make_rsrc(const float *base)
 {
@@ -86,31 +93,31 @@ __device__ __forceinline__ Rsrc make_rsrc(const float *base)
 typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 
-template <int NPL> struct BufIO;
-template <> struct BufIO<1> {
+template <int NPL, bool NT> struct BufIO;
+template <bool NT> struct BufIO<1, NT> {
     static __device__ __forceinline__ float load(Rsrc r, unsigned voff, unsigned soff)
     {
-        return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, AUX_LOAD));
+        return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, Aux<NT>::load));
     }
     static __device__ __forceinline__ void store(float v, Rsrc r, unsigned voff, unsigned soff)
     {
-        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), r, voff, soff, AUX_STORE);
+        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), r, voff, soff, Aux<NT>::store);
     }
 };
-template <> struct BufIO<2> {
+template <bool NT> struct BufIO<2, NT> {
     static __device__ __forceinline__ f32x2 load(Rsrc r, unsigned voff, unsigned soff)
     {
-        return __builtin_bit_cast(f32x2, __builtin_amdgcn_raw_buffer_load_b64(r, voff, soff, AUX_LOAD));
+        return __builtin_bit_cast(f32x2, __builtin_amdgcn_raw_buffer_load_b64(r, voff, soff, Aux<NT>::load));
     }
     static __device__ __forceinline__ void store(f32x2 v, Rsrc r, unsigned voff, unsigned soff)
     {
-        __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(u32x2, v), r, voff, soff, AUX_STORE);
+        __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(u32x2, v), r, voff, soff, Aux<NT>::store);
     }
 };
-template <> struct BufIO<4> {
+template <bool NT> struct BufIO<4, NT> {
     static __device__ __forceinline__ f32x4 load(Rsrc r, unsigned voff, unsigned soff)
     {
-        return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, AUX_LOAD));
+        return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, Aux<NT>::load));
     }
     // A 16-byte store takes more than one pass to read its data registers.  The compiler keeps the
     // next instruction from overwriting them only when the store has no SGPR offset; with one, a
@@ -120,7 +127,7 @@ template <> struct BufIO<4> {
     // short wait that reads the data keeps every writer away until the store has taken it.
     static __device__ __forceinline__ void store(f32x4 v, Rsrc r, unsigned voff, unsigned soff)
     {
-        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), r, voff + soff, 0, AUX_STORE);
+        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), r, voff + soff, 0, Aux<NT>::store);
         asm volatile("s_nop 1" : : "v"(v));                    // the data registers stay untouched two more cycles
     }
 };
@@ -220,7 +227,7 @@ __device__ __forceinline__ float spike_count_fast(float v, const Neuron &n, cons
 // the same number of loads (past the end it re-reads the last step), so the number of outstanding
 // loads at each wait is a compile-time constant.  A last, partial block runs through a guarded copy
 // of the same code.
-template <bool SYN, int NPL, int CAPK, bool REC>
+template <bool SYN, int NPL, int CAPK, bool REC, bool NT>
 __global__ void __launch_bounds__(BLOCK) layer_lif_forward(
     float *__restrict__ spikes, float *__restrict__ v_rec, float *__restrict__ i_rec, float *__restrict__ ckpt_v,
     float *__restrict__ ckpt_i, float *__restrict__ v_last, float *__restrict__ i_last, double *spike_sum,
@@ -230,7 +237,7 @@ __global__ void __launch_bounds__(BLOCK) layer_lif_forward(
     constexpr int STAGES = CKPT / FWD_UNROLL;                 // pipeline stages per checkpoint interval
     static_assert(STAGES * FWD_UNROLL == CKPT && STAGES % 2 == 0, "an even number of stages per checkpoint interval");
     typedef typename Vec<NPL>::type V;
-    typedef BufIO<NPL> IO;
+    typedef BufIO<NPL, NT> IO;
     // A block works inside one batch element, so all bases are block-uniform.
     const int64_t b = blockIdx.x / blocks_per_batch;
     const int64_t m0 = static_cast<int64_t>(blockIdx.x - b * blocks_per_batch) * (BLOCK * NPL);
@@ -378,7 +385,7 @@ __global__ void __launch_bounds__(BLOCK) layer_lif_forward(
 // The final potential handed out by the forward is vpost_{T-1} = v_{T-1} - c count_{T-1}; a gradient
 // gv on it reaches v_{T-1} directly and the spike count with weight -c, a gradient on the final
 // synaptic current adds to mu_{T-1}.
-template <bool SYN, int KIND, int CAPK>
+template <bool SYN, int KIND, int CAPK, bool NT>
 __global__ void __launch_bounds__(BWD_BLOCK) __attribute__((amdgpu_waves_per_eu(EXODUS_LAYER_BWD_WAVES, EXODUS_LAYER_BWD_WAVES)))
 layer_lif_backward(
     float *__restrict__ grad_x, float *__restrict__ alpha_mem_grad, float *__restrict__ alpha_syn_grad,
@@ -387,7 +394,7 @@ layer_lif_backward(
     const float *__restrict__ ckpt_v, const float *__restrict__ ckpt_i, const LayerConsts p, const float p0,
     const float p1, const float inv_p0, const int64_t blocks_per_batch, const int64_t T, const int64_t M)
 {
-    typedef BufIO<1> IO;
+    typedef BufIO<1, NT> IO;
     const int64_t b = blockIdx.x / blocks_per_batch;
     const int64_t m0 = static_cast<int64_t>(blockIdx.x - b * blocks_per_batch) * BWD_BLOCK;
     const unsigned lane_off = threadIdx.x;
@@ -538,7 +545,7 @@ constexpr int LEAKY_UNROLL = 8;
 
 // xin = norm_input ? (1 - alpha) * x : x;  xin = decay_early ? xin * alpha : xin;  v = v * alpha + xin
 // (the two input factors are applied as kn = 1 - alpha or 1 and kd = alpha or 1: a factor of 1 is exact)
-template <int NPL>
+template <int NPL, bool NT>
 __global__ void __launch_bounds__(BLOCK) layer_leaky_forward(float *__restrict__ out, float *__restrict__ v_last,
                                                              double *out_sum, const float *__restrict__ x,
                                                              const LeakyConsts p,
@@ -546,7 +553,7 @@ __global__ void __launch_bounds__(BLOCK) layer_leaky_forward(float *__restrict__
                                                              const int64_t M)
 {
     typedef typename Vec<NPL>::type V;
-    typedef BufIO<NPL> IO;
+    typedef BufIO<NPL, NT> IO;
     constexpr int U = LEAKY_UNROLL;
     const int64_t b = blockIdx.x / blocks_per_batch;
     const int64_t m0 = static_cast<int64_t>(blockIdx.x - b * blocks_per_batch) * (BLOCK * NPL);
@@ -622,14 +629,14 @@ __global__ void __launch_bounds__(BLOCK) layer_leaky_forward(float *__restrict__
 // grad_x_t = ((decay_early ? g_t alpha : g_t) * (norm_input ? 1 - alpha : 1))
 // grad_alpha = sum_t g_t out_{t-1}  +  (decay_early ? sum_t g_t (k x_t) : 0)  -  (norm_input ? sum_t (g_t [alpha]) x_t : 0)
 // `x` is only read when WITH_X (alpha gradient wanted and one of the input scalings is on).
-template <int NPL, bool ALPHA, bool WITH_X>
+template <int NPL, bool ALPHA, bool WITH_X, bool NT>
 __global__ void __launch_bounds__(BLOCK) layer_leaky_backward(
     float *__restrict__ grad_x, float *__restrict__ alpha_grad, float *__restrict__ v_init_grad,
     const float *__restrict__ grad_out, const float *__restrict__ grad_v_last, const float *__restrict__ out,
     const float *__restrict__ x, const LeakyConsts p, const int64_t blocks_per_batch, const int64_t T, const int64_t M)
 {
     typedef typename Vec<NPL>::type V;
-    typedef BufIO<NPL> IO;
+    typedef BufIO<NPL, NT> IO;
     constexpr int U = LEAKY_UNROLL;
     const int64_t b = blockIdx.x / blocks_per_batch;
     const int64_t m0 = static_cast<int64_t>(blockIdx.x - b * blocks_per_batch) * (BLOCK * NPL);
@@ -764,6 +771,15 @@ inline unsigned common_alignment(std::initializer_list<const void *> ptrs)
     return static_cast<unsigned>(bits & 15u) == 0 ? 16u : ((bits & 7u) == 0 ? 8u : 4u);
 }
 
+// true when every step's neurons start and end on 128-byte memory lines for all the given tensors:
+// then no line is shared between waves and the streamed accesses can be marked non-temporal
+inline bool whole_lines(int64_t neurons, std::initializer_list<const void *> ptrs)
+{
+    uintptr_t bits = 0;
+    for (const void *q : ptrs) bits |= reinterpret_cast<uintptr_t>(q);
+    return (neurons % 32) == 0 && (bits & 127u) == 0;
+}
+
 inline bool bad3(int64_t b, int64_t t, int64_t m)
 {
     if (b < 0 || t < 0 || m < 0) return true;
@@ -780,9 +796,14 @@ int launch_bwd(float *grad_x, float *am_g, float *as_g, float *v0_g, float *i0_g
     const int64_t blocks_per_batch = (M + BWD_BLOCK - 1) / BWD_BLOCK;
     if (blocks_per_batch > 0x7fffffffLL / B) return hipErrorInvalidValue;
     const int64_t blocks = blocks_per_batch * B;
-    hipLaunchKernelGGL((layer_lif_backward<SYN, KIND, CAPK>), dim3(static_cast<unsigned>(blocks)), dim3(BWD_BLOCK), 0, s,
-                       grad_x, am_g, as_g, v0_g, i0_g, grad_spikes, gvl, gil, x, ckpt_v, ckpt_i, p, p0, p1,
-                       p0 != 0.f ? 1.f / p0 : 0.f, blocks_per_batch, T, M);
+    if (whole_lines(M, {grad_x, grad_spikes, x}))
+        hipLaunchKernelGGL((layer_lif_backward<SYN, KIND, CAPK, true>), dim3(static_cast<unsigned>(blocks)), dim3(BWD_BLOCK), 0, s,
+                           grad_x, am_g, as_g, v0_g, i0_g, grad_spikes, gvl, gil, x, ckpt_v, ckpt_i, p, p0, p1,
+                           p0 != 0.f ? 1.f / p0 : 0.f, blocks_per_batch, T, M);
+    else
+        hipLaunchKernelGGL((layer_lif_backward<SYN, KIND, CAPK, false>), dim3(static_cast<unsigned>(blocks)), dim3(BWD_BLOCK), 0, s,
+                           grad_x, am_g, as_g, v0_g, i0_g, grad_spikes, gvl, gil, x, ckpt_v, ckpt_i, p, p0, p1,
+                           p0 != 0.f ? 1.f / p0 : 0.f, blocks_per_batch, T, M);
     return static_cast<int>(hipGetLastError());
 }
 
@@ -808,9 +829,14 @@ int launch_fwd(const FwdArgs &a)
 {
     const int64_t blocks_per_batch = (a.M + BLOCK * NPL - 1) / (BLOCK * NPL);
     if (blocks_per_batch > 0x7fffffffLL / a.B) return hipErrorInvalidValue;
-    hipLaunchKernelGGL((layer_lif_forward<SYN, NPL, CAPK, REC>), dim3(static_cast<unsigned>(blocks_per_batch * a.B)),
-                       dim3(BLOCK), 0, a.s, a.spikes, a.v_rec, a.i_rec, a.ckpt_v, a.ckpt_i, a.v_last, a.i_last,
-                       a.spike_sum, a.x, a.p, blocks_per_batch, a.T, a.M);
+    if (whole_lines(a.M, {a.x, a.spikes, a.v_rec, a.i_rec}))
+        hipLaunchKernelGGL((layer_lif_forward<SYN, NPL, CAPK, REC, true>), dim3(static_cast<unsigned>(blocks_per_batch * a.B)),
+                           dim3(BLOCK), 0, a.s, a.spikes, a.v_rec, a.i_rec, a.ckpt_v, a.ckpt_i, a.v_last, a.i_last,
+                           a.spike_sum, a.x, a.p, blocks_per_batch, a.T, a.M);
+    else
+        hipLaunchKernelGGL((layer_lif_forward<SYN, NPL, CAPK, REC, false>), dim3(static_cast<unsigned>(blocks_per_batch * a.B)),
+                           dim3(BLOCK), 0, a.s, a.spikes, a.v_rec, a.i_rec, a.ckpt_v, a.ckpt_i, a.v_last, a.i_last,
+                           a.spike_sum, a.x, a.p, blocks_per_batch, a.T, a.M);
     return static_cast<int>(hipGetLastError());
 }
 
@@ -973,12 +999,18 @@ EXODUS_API int exodus_layer_leaky_forward(float *out, float *v_last, double *out
     if (blocks_per_batch > 0x7fffffffLL / batch) return hipErrorInvalidValue;
     const dim3 grid(static_cast<unsigned>(blocks_per_batch * batch)), block(BLOCK);
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (npl == 4)
-        hipLaunchKernelGGL((layer_leaky_forward<4>), grid, block, 0, s, out, v_last, out_sum, input, p, blocks_per_batch, t, neurons);
-    else if (npl == 2)
-        hipLaunchKernelGGL((layer_leaky_forward<2>), grid, block, 0, s, out, v_last, out_sum, input, p, blocks_per_batch, t, neurons);
-    else
-        hipLaunchKernelGGL((layer_leaky_forward<1>), grid, block, 0, s, out, v_last, out_sum, input, p, blocks_per_batch, t, neurons);
+    const bool nt = whole_lines(neurons, {input, out});
+#define EXODUS_LF(NPL, NT)                                                                                     \
+    hipLaunchKernelGGL((layer_leaky_forward<NPL, NT>), grid, block, 0, s, out, v_last, out_sum, input, p,     \
+                       blocks_per_batch, t, neurons)
+    if (npl == 4) {
+        if (nt) EXODUS_LF(4, true); else EXODUS_LF(4, false);
+    } else if (npl == 2) {
+        if (nt) EXODUS_LF(2, true); else EXODUS_LF(2, false);
+    } else {
+        if (nt) EXODUS_LF(1, true); else EXODUS_LF(1, false);
+    }
+#undef EXODUS_LF
     return static_cast<int>(hipGetLastError());
 }
 
@@ -1008,9 +1040,14 @@ EXODUS_API int exodus_layer_leaky_backward(float *grad_input, float *alpha_grad,
     if (blocks_per_batch > 0x7fffffffLL / batch) return hipErrorInvalidValue;
     const dim3 grid(static_cast<unsigned>(blocks_per_batch * batch)), block(BLOCK);
     hipStream_t s = static_cast<hipStream_t>(stream);
-#define EXODUS_LK(NPL, AL, WX)                                                                                 \
-    hipLaunchKernelGGL((layer_leaky_backward<NPL, AL, WX>), grid, block, 0, s, grad_input, alpha_grad,        \
+    const bool nt = whole_lines(neurons, {grad_input, grad_out, out, input});
+#define EXODUS_LK1(NPL, AL, WX, NT)                                                                            \
+    hipLaunchKernelGGL((layer_leaky_backward<NPL, AL, WX, NT>), grid, block, 0, s, grad_input, alpha_grad,    \
                        vmem_init_grad, grad_out, grad_v_last, out, input, p, blocks_per_batch, t, neurons)
+#define EXODUS_LK(NPL, AL, WX)                                                                                 \
+    do {                                                                                                       \
+        if (nt) EXODUS_LK1(NPL, AL, WX, true); else EXODUS_LK1(NPL, AL, WX, false);                            \
+    } while (0)
     if (npl == 4) {
         EXODUS_LK(4, false, false);
     } else if (npl == 2) {
@@ -1019,6 +1056,7 @@ EXODUS_API int exodus_layer_leaky_backward(float *grad_input, float *alpha_grad,
         if (with_x) EXODUS_LK(1, true, true); else if (want_alpha) EXODUS_LK(1, true, false); else EXODUS_LK(1, false, false);
     }
 #undef EXODUS_LK
+#undef EXODUS_LK1
     return static_cast<int>(hipGetLastError());
 }
 
