@@ -29,7 +29,7 @@ extern "C" {
 #endif
 
 /* ABI version of this header; bumped on any signature change. */
-#define EXODUS_HIP_ABI_VERSION 2
+#define EXODUS_HIP_ABI_VERSION 3
 
 int exodus_hip_abi_version(void);
 const char *exodus_hip_error_string(int status);
@@ -176,8 +176,10 @@ int exodus_layer_checkpoint_interval(void);
  * order as exodus_synlif_forward / exodus_lif_forward after the layer's input scalings.
  *   out_spikes (batch,t,neurons); v_last, i_last (batch*neurons): potential after the last reset
  *   and last synaptic current (i_last may be NULL without synapse).
- * Optional (NULL = skip): out_vmem_rec / out_isyn_rec (batch,t,neurons) post-reset potential and
- * synaptic current of every step; ckpt_v / ckpt_i (batch, ceil(t/interval), neurons) state at the
+ * Optional (NULL = skip): out_vmem_rec / out_isyn_rec (batch,t,neurons) potential and synaptic
+ * current of every step, the potential after the reset (what the layer records, reference
+ * sinabs/exodus/layers/lif.py:256) or, with record_pre_reset != 0, before it (what
+ * IntegrateAndFire hands to the surrogate function, reference sinabs/exodus/spike.py:251); ckpt_v / ckpt_i (batch, ceil(t/interval), neurons) state at the
  * start of every checkpoint interval, needed by exodus_layer_lif_backward; spike_sum, one double
  * to which the total spike count is added atomically. */
 int exodus_layer_lif_forward(float *out_spikes, float *out_vmem_rec, float *out_isyn_rec, float *ckpt_v,
@@ -186,13 +188,16 @@ int exodus_layer_lif_forward(float *out_spikes, float *out_vmem_rec, float *out_
                              const float *isyn_initial, const float *alpha_mem, const float *alpha_syn,
                              const float *membr_subtract, const float *theta, const float *theta_low,
                              int apply_theta_low, int max_num_spikes, int decay_early, int norm_input,
-                             int64_t batch, int64_t t, int64_t neurons, void *stream);
+                             int record_pre_reset, int64_t batch, int64_t t, int64_t neurons, void *stream);
 
 /* Backward of the above.  Re-reads `input`, rebuilds membrane potential and synaptic current of
  * each checkpoint interval from ckpt_v / ckpt_i and walks it in reverse.  grad_v_last /
  * grad_i_last (batch*neurons, optional) are gradients arriving at the final states.  Outputs:
  * grad_input (batch,t,neurons) and the optional per-neuron alpha_mem_grad, alpha_syn_grad,
- * vmem_init_grad, isyn_init_grad.  surrogate_kind must be an in-kernel kind (1..3). */
+ * vmem_init_grad, isyn_init_grad.  With surrogate_kind == EXODUS_SURR_TENSOR the derivative of
+ * the spike function at every step comes from `surr` (batch,t,neurons) — what a caller computes
+ * from the pre-reset potential record with any function of its own (the reference evaluates an
+ * arbitrary Python callable there, sinabs/exodus/spike.py:251); otherwise `surr` is ignored. */
 int exodus_layer_lif_backward(float *grad_input, float *alpha_mem_grad, float *alpha_syn_grad,
                               float *vmem_init_grad, float *isyn_init_grad, const float *grad_spikes,
                               const float *grad_v_last, const float *grad_i_last, const float *input,
@@ -200,8 +205,8 @@ int exodus_layer_lif_backward(float *grad_input, float *alpha_mem_grad, float *a
                               const float *isyn_initial, const float *alpha_mem, const float *alpha_syn,
                               const float *membr_subtract, const float *theta, const float *theta_low,
                               int apply_theta_low, int max_num_spikes, int decay_early, int norm_input,
-                              int surrogate_kind, float surr_p0, float surr_p1, int64_t batch, int64_t t,
-                              int64_t neurons, void *stream);
+                              int surrogate_kind, float surr_p0, float surr_p1, const float *surr,
+                              int64_t batch, int64_t t, int64_t neurons, void *stream);
 
 /* Forward of the non-spiking leaky-integrator layer (ExpLeak) on (batch,t,neurons): per neuron
  *   xin = norm_input ? (1 - alpha) * input : input;  xin = decay_early ? xin * alpha : xin;

@@ -48,6 +48,7 @@ struct LayerConsts {
     const float *v_init, *i_init, *alpha_mem, *alpha_syn, *c, *theta, *theta_low;
     int apply_low, decay_early, norm_input;
     unsigned cap;
+    int rec_pre;        // the potential record holds the value before the reset instead of after it
 };
 
 template <int NPL> struct Vec;
@@ -325,7 +326,7 @@ __global__ void __launch_bounds__(BLOCK) layer_lif_forward(
                         nr[e].vpost = __fsub_rn(v[e], __fmul_rn(count[e], nr[e].c));
                         part += count[e];
                         lane_put<NPL>(s, e, count[e]);
-                        lane_put<NPL>(vr, e, nr[e].vpost);
+                        lane_put<NPL>(vr, e, (REC && p.rec_pre) ? v[e] : nr[e].vpost);
                         lane_put<NPL>(ir, e, nr[e].i);
                     }
                     IO::store(s, rs, voff, u * step_bytes);
@@ -385,13 +386,19 @@ __global__ void __launch_bounds__(BLOCK) layer_lif_forward(
 // The final potential handed out by the forward is vpost_{T-1} = v_{T-1} - c count_{T-1}; a gradient
 // gv on it reaches v_{T-1} directly and the spike count with weight -c, a gradient on the final
 // synaptic current adds to mu_{T-1}.
+// KIND == EXODUS_SURR_TENSOR reads the surrogate derivative of every step from `surr` (a third
+// streamed tensor, whose register buffer costs the kernel one wave per SIMD); the other kinds
+// evaluate it from the rebuilt potential and ignore `surr`.
 template <bool SYN, int KIND, int CAPK, bool NT>
-__global__ void __launch_bounds__(BWD_BLOCK) __attribute__((amdgpu_waves_per_eu(EXODUS_LAYER_BWD_WAVES, EXODUS_LAYER_BWD_WAVES)))
+__global__ void __launch_bounds__(BWD_BLOCK)
+    __attribute__((amdgpu_waves_per_eu(KIND == EXODUS_SURR_TENSOR ? 2 : EXODUS_LAYER_BWD_WAVES,
+                                       KIND == EXODUS_SURR_TENSOR ? 2 : EXODUS_LAYER_BWD_WAVES)))
 layer_lif_backward(
     float *__restrict__ grad_x, float *__restrict__ alpha_mem_grad, float *__restrict__ alpha_syn_grad,
     float *__restrict__ v_init_grad, float *__restrict__ i_init_grad, const float *__restrict__ grad_spikes,
     const float *__restrict__ grad_v_last, const float *__restrict__ grad_i_last, const float *__restrict__ x,
-    const float *__restrict__ ckpt_v, const float *__restrict__ ckpt_i, const LayerConsts p, const float p0,
+    const float *__restrict__ surr, const float *__restrict__ ckpt_v, const float *__restrict__ ckpt_i,
+    const LayerConsts p, const float p0,
     const float p1, const float inv_p0, const int64_t blocks_per_batch, const int64_t T, const int64_t M)
 {
     typedef BufIO<1, NT> IO;
@@ -405,6 +412,8 @@ layer_lif_backward(
     const float *xp = x + (b * T) * M + m0;
     const float *gp = grad_spikes + (b * T) * M + m0;
     float *op = grad_x + (b * T) * M + m0;
+    constexpr bool FROM_TENSOR = KIND == EXODUS_SURR_TENSOR;
+    const float *srp = FROM_TENSOR ? surr + (b * T) * M + m0 : nullptr;
     const float *cvp = ckpt_v + (b * n_ck) * M + m0;
     const float *cip = SYN ? ckpt_i + (b * n_ck) * M + m0 : nullptr;
     const unsigned voff = lane_off * 4u;
@@ -439,17 +448,19 @@ layer_lif_backward(
         constexpr bool GUARD = decltype(guard)::value;
         const int64_t t0 = j * CKPT;
         const int len = GUARD ? static_cast<int>(T - t0) : CKPT;
-        float xr[CKPT], gr[CKPT], vr[CKPT];
+        float xr[CKPT], gr[CKPT], vr[CKPT], sr[FROM_TENSOR ? CKPT : 1];
         {
             // always CKPT loads per tensor (steps past the end re-read the last step): a constant number
             // of loads in flight lets each use wait for its own load only
             const Rsrc rx = make_rsrc(xp + t0 * M), rg = make_rsrc(gp + t0 * M);
+            const Rsrc rs = make_rsrc(FROM_TENSOR ? srp + t0 * M : nullptr);
             const unsigned last = static_cast<unsigned>(len - 1);
 #pragma unroll
             for (int k = 0; k < CKPT; ++k) {
                 const unsigned so = (GUARD ? (k < last ? k : last) : k) * step_bytes;
                 xr[k] = IO::load(rx, voff, so);
                 gr[k] = IO::load(rg, voff, so);
+                if (FROM_TENSOR) sr[k] = IO::load(rs, voff, so);
             }
         }
         nr.vpost = ld_stream(cvp + j * M + lane_off);
@@ -472,7 +483,7 @@ layer_lif_backward(
             const int k = CKPT - 1 - kq;
             if (!GUARD || k < len) {
                 const float v = vr[k], cur_i = xr[k];
-                const float sg = surrogate<KIND>(v, nr.th, inv_p0, sk);
+                const float sg = FROM_TENSOR ? sr[FROM_TENSOR ? k : 0] : surrogate<KIND>(v, nr.th, inv_p0, sk);
                 const float vpost = __fsub_rn(v, __fmul_rn(nr.c, spike_count_fast<CAPK>(v, nr, cc)));
                 acc_m.add(lam, vpost);                          // lambda_{t+1} * vpost_t
                 const float through = __fsub_rn(1.0f, __fmul_rn(nr.c, sg));   // d vpost_t / d v_t
@@ -790,19 +801,20 @@ inline bool bad3(int64_t b, int64_t t, int64_t m)
 
 template <bool SYN, int KIND, int CAPK>
 int launch_bwd(float *grad_x, float *am_g, float *as_g, float *v0_g, float *i0_g, const float *grad_spikes,
-               const float *gvl, const float *gil, const float *x, const float *ckpt_v, const float *ckpt_i,
-               const LayerConsts &p, float p0, float p1, int64_t B, int64_t T, int64_t M, hipStream_t s)
+               const float *gvl, const float *gil, const float *x, const float *surr, const float *ckpt_v,
+               const float *ckpt_i, const LayerConsts &p, float p0, float p1, int64_t B, int64_t T, int64_t M,
+               hipStream_t s)
 {
     const int64_t blocks_per_batch = (M + BWD_BLOCK - 1) / BWD_BLOCK;
     if (blocks_per_batch > 0x7fffffffLL / B) return hipErrorInvalidValue;
     const int64_t blocks = blocks_per_batch * B;
-    if (whole_lines(M, {grad_x, grad_spikes, x}))
+    if (whole_lines(M, {grad_x, grad_spikes, x, surr}))
         hipLaunchKernelGGL((layer_lif_backward<SYN, KIND, CAPK, true>), dim3(static_cast<unsigned>(blocks)), dim3(BWD_BLOCK), 0, s,
-                           grad_x, am_g, as_g, v0_g, i0_g, grad_spikes, gvl, gil, x, ckpt_v, ckpt_i, p, p0, p1,
+                           grad_x, am_g, as_g, v0_g, i0_g, grad_spikes, gvl, gil, x, surr, ckpt_v, ckpt_i, p, p0, p1,
                            p0 != 0.f ? 1.f / p0 : 0.f, blocks_per_batch, T, M);
     else
         hipLaunchKernelGGL((layer_lif_backward<SYN, KIND, CAPK, false>), dim3(static_cast<unsigned>(blocks)), dim3(BWD_BLOCK), 0, s,
-                           grad_x, am_g, as_g, v0_g, i0_g, grad_spikes, gvl, gil, x, ckpt_v, ckpt_i, p, p0, p1,
+                           grad_x, am_g, as_g, v0_g, i0_g, grad_spikes, gvl, gil, x, surr, ckpt_v, ckpt_i, p, p0, p1,
                            p0 != 0.f ? 1.f / p0 : 0.f, blocks_per_batch, T, M);
     return static_cast<int>(hipGetLastError());
 }
@@ -906,7 +918,8 @@ EXODUS_API int exodus_layer_lif_forward(float *out_spikes, float *out_vmem_rec, 
                                         const float *isyn_initial, const float *alpha_mem, const float *alpha_syn,
                                         const float *membr_subtract, const float *theta, const float *theta_low,
                                         int apply_theta_low, int max_num_spikes, int decay_early, int norm_input,
-                                        int64_t batch, int64_t t, int64_t neurons, void *stream)
+                                        int record_pre_reset, int64_t batch, int64_t t, int64_t neurons,
+                                        void *stream)
 {
     if (bad3(batch, t, neurons)) return hipErrorInvalidValue;
     if (batch == 0 || t == 0 || neurons == 0) return hipSuccess;
@@ -927,6 +940,7 @@ EXODUS_API int exodus_layer_lif_forward(float *out_spikes, float *out_vmem_rec, 
     p.decay_early = decay_early ? 1 : 0;
     p.norm_input = norm_input ? 1 : 0;
     p.cap = static_cast<unsigned>(max_num_spikes);
+    p.rec_pre = record_pre_reset ? 1 : 0;
     // two neurons per lane at most: with four the spiking kernel needs so many registers for its two
     // load buffers that only two waves fit a SIMD, and it measures slower than two neurons, three waves
     const int npl = pick_neurons_per_lane(
@@ -943,16 +957,17 @@ EXODUS_API int exodus_layer_lif_backward(float *grad_input, float *alpha_mem_gra
                                          const float *isyn_initial, const float *alpha_mem, const float *alpha_syn,
                                          const float *membr_subtract, const float *theta, const float *theta_low,
                                          int apply_theta_low, int max_num_spikes, int decay_early, int norm_input,
-                                         int surrogate_kind, float surr_p0, float surr_p1, int64_t batch, int64_t t,
-                                         int64_t neurons, void *stream)
+                                         int surrogate_kind, float surr_p0, float surr_p1, const float *surr,
+                                         int64_t batch, int64_t t, int64_t neurons, void *stream)
 {
     if (bad3(batch, t, neurons)) return hipErrorInvalidValue;
     if (batch == 0 || t == 0 || neurons == 0) return hipSuccess;
     if (too_wide(neurons)) return hipErrorInvalidValue;
     const bool syn = alpha_syn != nullptr;
     if (!grad_input || !grad_spikes || !input || !ckpt_v || !alpha_mem || !membr_subtract || !theta ||
-        (apply_theta_low && !theta_low) || (syn && !ckpt_i))
+        (apply_theta_low && !theta_low) || (syn && !ckpt_i) || (surrogate_kind == EXODUS_SURR_TENSOR && !surr))
         return hipErrorInvalidValue;
+    if (surrogate_kind != EXODUS_SURR_TENSOR) surr = nullptr;
     if (alpha_mem_grad && !vmem_post_initial) return hipErrorInvalidValue;
     if (syn && alpha_syn_grad && !decay_early && !isyn_initial) return hipErrorInvalidValue;
     LayerConsts p;
@@ -967,12 +982,14 @@ EXODUS_API int exodus_layer_lif_backward(float *grad_input, float *alpha_mem_gra
     p.decay_early = decay_early ? 1 : 0;
     p.norm_input = norm_input ? 1 : 0;
     p.cap = static_cast<unsigned>(max_num_spikes);
+    p.rec_pre = 0;
     hipStream_t s = static_cast<hipStream_t>(stream);
 #define EXODUS_BWD(SYN, K)                                                                                        \
     return dispatch_bwd_cap<SYN, K>(p.cap, grad_input, alpha_mem_grad, alpha_syn_grad, vmem_init_grad,            \
-                                    isyn_init_grad, grad_spikes, grad_v_last, grad_i_last, input, ckpt_v, ckpt_i, \
-                                    p, surr_p0, surr_p1, batch, t, neurons, s)
+                                    isyn_init_grad, grad_spikes, grad_v_last, grad_i_last, input, surr, ckpt_v,   \
+                                    ckpt_i, p, surr_p0, surr_p1, batch, t, neurons, s)
     switch (surrogate_kind) {
+        case EXODUS_SURR_TENSOR: if (syn) EXODUS_BWD(true, EXODUS_SURR_TENSOR); EXODUS_BWD(false, EXODUS_SURR_TENSOR);
         case EXODUS_SURR_SINGLE_EXP: if (syn) EXODUS_BWD(true, EXODUS_SURR_SINGLE_EXP); EXODUS_BWD(false, EXODUS_SURR_SINGLE_EXP);
         case EXODUS_SURR_PERIODIC_EXP: if (syn) EXODUS_BWD(true, EXODUS_SURR_PERIODIC_EXP); EXODUS_BWD(false, EXODUS_SURR_PERIODIC_EXP);
         case EXODUS_SURR_HEAVISIDE: if (syn) EXODUS_BWD(true, EXODUS_SURR_HEAVISIDE); EXODUS_BWD(false, EXODUS_SURR_HEAVISIDE);

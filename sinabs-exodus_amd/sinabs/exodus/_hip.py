@@ -21,7 +21,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("EXODUS_HIP_LIBRARY") or os.path.join(_HERE, "libexodus_hip.so")
 
 SURR_TENSOR, SURR_SINGLE_EXP, SURR_PERIODIC_EXP, SURR_HEAVISIDE = 0, 1, 2, 3
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 _p = ctypes.c_void_p
 _i64 = ctypes.c_int64
@@ -45,8 +45,8 @@ _SIGNATURES = {
     "exodus_spike_backward": ([_p] * 4 + [_f, _f, _i64, _i64, _p], _int),
     "exodus_probe_stream": ([_p, _p, _p, _i64, _p], _int),
     "exodus_layer_checkpoint_interval": ([], _int),
-    "exodus_layer_lif_forward": ([_p] * 16 + [_int, _int, _int, _int, _i64, _i64, _i64, _p], _int),
-    "exodus_layer_lif_backward": ([_p] * 18 + [_int, _int, _int, _int, _int, _f, _f, _i64, _i64, _i64, _p], _int),
+    "exodus_layer_lif_forward": ([_p] * 16 + [_int, _int, _int, _int, _int, _i64, _i64, _i64, _p], _int),
+    "exodus_layer_lif_backward": ([_p] * 18 + [_int, _int, _int, _int, _int, _f, _f, _p, _i64, _i64, _i64, _p], _int),
     "exodus_layer_leaky_forward": ([_p] * 6 + [_int, _int, _i64, _i64, _i64, _p], _int),
     "exodus_layer_leaky_backward": ([_p] * 9 + [_int, _int, _i64, _i64, _i64, _p], _int),
 }
@@ -434,9 +434,14 @@ def _btm(x: torch.Tensor, name: str, like: Optional[torch.Tensor] = None):
 def layerLifForward(input, vmemPostInitial, isynInitial, alphaMem, alphaSyn, membrSubtract, theta, thetaLow,
                     applyThetaLow: bool, maxNumSpikes: int, decayEarly: bool, normInput: bool,
                     wantCheckpoints: bool = True, wantRecords: bool = False, wantSpikeSum: bool = True,
-                    outSpikes: Optional[torch.Tensor] = None, stateShape: Optional[tuple] = None):
+                    outSpikes: Optional[torch.Tensor] = None, stateShape: Optional[tuple] = None,
+                    wantPreReset: bool = False):
     """Returns dict(spikes, v_last, i_last, ckpt_v, ckpt_i, v_rec, i_rec, spike_sum); absent items are None.
-    ``stateShape`` (product = batch*neurons) gives v_last / i_last that shape instead of a flat vector."""
+    ``stateShape`` (product = batch*neurons) gives v_last / i_last that shape instead of a flat vector.
+    ``wantRecords`` records potential (after the reset) and synaptic current of every step;
+    ``wantPreReset`` records only the potential, before the reset (the surrogate function's argument)."""
+    if wantRecords and wantPreReset:
+        raise RuntimeError("wantRecords and wantPreReset exclude each other")
     _btm(input, "input")
     b, t, m = input.shape
     n = b * m
@@ -463,7 +468,8 @@ def layerLifForward(input, vmemPostInitial, isynInitial, alphaMem, alphaSyn, mem
     res = dict(spikes=spikes, v_last=new(*state_shape), i_last=new(*state_shape) if syn else None,
                ckpt_v=new(b, n_ck, m) if wantCheckpoints else None,
                ckpt_i=new(b, n_ck, m) if (wantCheckpoints and syn) else None,
-               v_rec=new(b, t, m) if wantRecords else None, i_rec=new(b, t, m) if (wantRecords and syn) else None,
+               v_rec=new(b, t, m) if (wantRecords or wantPreReset) else None,
+               i_rec=new(b, t, m) if (wantRecords and syn) else None,
                spike_sum=torch.zeros((), dtype=torch.float64, device=input.device) if wantSpikeSum else None)
     if t == 0:                                   # nothing to integrate: the final states are the initial ones
         res["v_last"].copy_(vmemPostInitial.reshape(state_shape))
@@ -475,15 +481,16 @@ def layerLifForward(input, vmemPostInitial, isynInitial, alphaMem, alphaSyn, mem
             _ptr(res["v_last"]), _ptr(res["i_last"]), _ptr(res["spike_sum"]), _ptr(input), _ptr(vmemPostInitial),
             _ptr(isynInitial) if syn else None, _ptr(alphaMem), _ptr(alphaSyn) if syn else None, _ptr(membrSubtract),
             _ptr(theta), _ptr(thetaLow), int(bool(applyThetaLow)), int(maxNumSpikes), int(bool(decayEarly)),
-            int(bool(normInput)), b, t, m, _stream(input)), "exodus_layer_lif_forward")
+            int(bool(normInput)), int(bool(wantPreReset)), b, t, m, _stream(input)), "exodus_layer_lif_forward")
     return res
 
 
 def layerLifBackward(gradSpikes, gradVLast, gradILast, input, ckptV, ckptI, vmemPostInitial, isynInitial, alphaMem,
                      alphaSyn, membrSubtract, theta, thetaLow, applyThetaLow: bool, maxNumSpikes: int,
                      decayEarly: bool, normInput: bool, surrogateKind: int, surrP0: float, surrP1: float,
-                     gradInput: Optional[torch.Tensor] = None):
-    """Returns (gradInput, alphaMemGrad, alphaSynGrad | None, vInitGrad, iInitGrad | None)."""
+                     gradInput: Optional[torch.Tensor] = None, surr: Optional[torch.Tensor] = None):
+    """Returns (gradInput, alphaMemGrad, alphaSynGrad | None, vInitGrad, iInitGrad | None).
+    ``surrogateKind == SURR_TENSOR`` takes the spike function's derivative from ``surr`` (batch, time, neurons)."""
     _btm(input, "input")
     b, t, m = input.shape
     n = b * m
@@ -511,6 +518,11 @@ def layerLifBackward(gradSpikes, gradVLast, gradILast, input, ckptV, ckptI, vmem
         gradInput = torch.empty_like(input)
     elif _btm(gradInput, "gradInput", input).shape != input.shape:
         raise RuntimeError("gradInput must have the shape of input")
+    if surrogateKind == SURR_TENSOR:
+        if surr is None or _btm(surr, "surr", input).shape != input.shape:
+            raise RuntimeError("surr must be given with the shape of input")
+    else:
+        surr = None
     z = lambda: torch.zeros(n, dtype=torch.float32, device=input.device)
     am_g, v0_g = z(), z()
     as_g, i0_g = (z(), z()) if syn else (None, None)
@@ -520,8 +532,8 @@ def layerLifBackward(gradSpikes, gradVLast, gradILast, input, ckptV, ckptI, vmem
             _ptr(gradILast) if syn else None, _ptr(input), _ptr(ckptV), _ptr(ckptI) if syn else None,
             _ptr(vmemPostInitial), _ptr(isynInitial) if syn else None, _ptr(alphaMem), _ptr(alphaSyn) if syn else None,
             _ptr(membrSubtract), _ptr(theta), _ptr(thetaLow), int(bool(applyThetaLow)), int(maxNumSpikes),
-            int(bool(decayEarly)), int(bool(normInput)), int(surrogateKind), float(surrP0), float(surrP1), b, t, m,
-            _stream(input)), "exodus_layer_lif_backward")
+            int(bool(decayEarly)), int(bool(normInput)), int(surrogateKind), float(surrP0), float(surrP1), _ptr(surr),
+            b, t, m, _stream(input)), "exodus_layer_lif_backward")
     return gradInput, am_g, as_g, v0_g, i0_g
 
 

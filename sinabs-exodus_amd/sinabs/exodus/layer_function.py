@@ -7,6 +7,10 @@ the kernels: synaptic current, input normalisation, membrane update, clamp, thre
 final states and the spike total for ``firing_rate``.  The forward keeps only checkpoints; the
 backward re-reads the input and rebuilds membrane potential and synaptic current chunk by chunk,
 so neither is ever written to memory in full.
+
+A surrogate gradient the kernels do not know (any callable, as in the reference,
+sinabs/exodus/spike.py:251) costs one more tensor each way: the forward also records the
+potential before the reset, the backward calls the function on it and hands the result to the kernel.
 """
 from typing import Callable, Optional
 
@@ -40,8 +44,6 @@ class SpikingLayerFunction(torch.autograd.Function):
         of ``spikes``; a gradient arriving at it is added to every element of the gradient of
         ``spikes``).  The final states come as flat vectors, or in ``state_shape`` if given."""
         kind, p0, p1 = classify_surrogate(surrogate_grad_fn)
-        if kind == _hip.SURR_TENSOR:
-            raise ValueError("surrogate_grad_fn is not one the layer kernel can evaluate")
         if inp.ndim != 3:
             raise ValueError("'inp' must be 3D, (batch, time, neurons)")
         if not inp.is_contiguous():
@@ -57,11 +59,15 @@ class SpikingLayerFunction(torch.autograd.Function):
         res = _hip.layerLifForward(
             inp, v_mem_init, i_syn_init, alpha_mem, alpha_syn, membrane_subtract, threshold, min_v_mem, apply_min,
             max_spikes, decay_early, norm_input, wantCheckpoints=need_grad, stateShape=state_shape,
+            wantPreReset=need_grad and kind == _hip.SURR_TENSOR,
         )
         ctx.cfg = (syn, apply_min, max_spikes, bool(decay_early), bool(norm_input), kind, p0, p1)
+        ctx.surrogate_grad_fn = surrogate_grad_fn if kind == _hip.SURR_TENSOR else None
         ctx.set_materialize_grads(False)
         if need_grad:
             saved = [inp, res["ckpt_v"], v_mem_init, alpha_mem, membrane_subtract, threshold]
+            if kind == _hip.SURR_TENSOR:
+                saved.append(res["v_rec"])
             if syn:
                 saved += [res["ckpt_i"], i_syn_init, alpha_syn]
             if apply_min:
@@ -77,6 +83,9 @@ class SpikingLayerFunction(torch.autograd.Function):
         saved = list(ctx.saved_tensors)
         inp, ckpt_v, v_mem_init, alpha_mem, membrane_subtract, threshold = saved[:6]
         rest = saved[6:]
+        v_pre = None
+        if kind == _hip.SURR_TENSOR:
+            v_pre, rest = rest[0], rest[1:]
         ckpt_i = i_syn_init = alpha_syn = None
         if syn:
             ckpt_i, i_syn_init, alpha_syn = rest[:3]
@@ -89,10 +98,17 @@ class SpikingLayerFunction(torch.autograd.Function):
         if grad_total is not None:                  # d(sum of spikes) / d(spike) = 1 for every element
             grad_spikes = grad_spikes + grad_total.to(grad_spikes.dtype)
         cont = lambda x: None if x is None else x.contiguous()
+        surr = None
+        if v_pre is not None:
+            # the function sees (batch, time, neurons) potentials and thresholds that broadcast over time
+            b, _, m = inp.shape
+            with torch.no_grad():
+                surr = ctx.surrogate_grad_fn(v_pre, threshold.view(b, 1, m))
+            surr = torch.as_tensor(surr, device=inp.device).to(torch.float32).expand(inp.shape).contiguous()
         grad_input, g_am, g_as, g_v0, g_i0 = _hip.layerLifBackward(
             cont(grad_spikes), cont(grad_v_last), cont(grad_i_last) if syn else None, inp, ckpt_v, ckpt_i,
             v_mem_init, i_syn_init, alpha_mem, alpha_syn, membrane_subtract, threshold, min_v_mem, apply_min,
-            max_spikes, decay_early, norm_input, kind, p0, p1,
+            max_spikes, decay_early, norm_input, kind, p0, p1, surr=surr,
         )
         return (grad_input, g_am, g_as, g_v0, g_i0, None, None, None, None, None, None, None, None)
 

@@ -222,7 +222,8 @@ class LIF(LIFBase):
             return self.tau_syn_calculated is None
         if not self._needs_grad(input_data):           # inference: any surrogate, with or without records
             return True
-        return not self.record_states and fusable(self.surrogate_grad_fn)
+        # with gradients the recorded states have to stay part of the autograd graph: (rows, time) Functions
+        return not self.record_states
 
     def _needs_grad(self, input_data: torch.Tensor) -> bool:
         if not torch.is_grad_enabled():

@@ -63,18 +63,19 @@ def test_native_equals_rows_path(L, batch, steps, trailing, tau_syn, decay_early
             assert_close(p.grad, q.grad, f"grad {k}", rtol=1e-4, atol=1e-5 * max(1.0, (batch * steps) ** 0.5))
 
 
-def test_native_iaf_squeeze_and_unknown_surrogate_fallback(L):
+def test_native_iaf_squeeze_and_recorded_states_fallback(L):
     el, act, _ = L
     x = torch.rand(6 * 50, 2, 5, 5, generator=gen(3)).cuda()
     native, rows = pair(el, el.IAFSqueeze, batch_size=6, min_v_mem=-1.0)
     assert torch.equal(native(x), rows(x)) and native(x).is_contiguous()
     custom = el.IAF(surrogate_grad_fn=lambda v, th: 1.0 / (1.0 + (v - th) ** 2)).cuda()
-    xg = x.reshape(6, 50, 2, 5, 5).clone().requires_grad_(True)      # with gradients these need the Functions
-    assert not custom._use_native_layout(xg)
+    xg = x.reshape(6, 50, 2, 5, 5).clone().requires_grad_(True)
+    assert custom._use_native_layout(xg)                              # any callable runs on the layer kernels
     rec = el.IAF(record_states=True).cuda()
-    assert not rec._use_native_layout(xg)
-    out = custom(xg); assert out.shape == (6, 50, 2, 5, 5)
-    out.sum().backward(); assert xg.grad is not None and bool(torch.isfinite(xg.grad).all())
+    assert not rec._use_native_layout(xg)                             # differentiable records need the Functions
+    out = rec(xg); assert out.shape == (6, 50, 2, 5, 5)
+    (out.sum() + rec.recordings["v_mem"].sum()).backward()
+    assert xg.grad is not None and bool(torch.isfinite(xg.grad).all())
 
 
 def test_native_forward_against_cpu_oracle(L):
@@ -361,8 +362,40 @@ def test_inference_records_states_and_accepts_any_surrogate(L, tau_syn):
             if tau_syn is not None:
                 assert torch.equal(native.recordings["i_syn"], rows.recordings["i_syn"])
             assert torch.allclose(native.firing_rate, rows.firing_rate, rtol=1e-6, atol=0)
-    assert not native._use_native_layout(x.requires_grad_(True))      # with gradients: the Functions
+    assert not native._use_native_layout(x.requires_grad_(True))      # records with gradients: the Functions
     with pytest.raises(ValueError):
         bad = el.LIF(tau_mem=10.0, min_v_mem=2.0).cuda()
         with torch.no_grad():
             bad(x)
+
+
+@pytest.mark.parametrize("tau_syn", [None, 6.0])
+@pytest.mark.parametrize("shape", [(3, 70, 5, 8), (2, 45, 37)])
+def test_any_callable_surrogate_on_the_layer_kernels(L, tau_syn, shape):
+    """A surrogate gradient the kernels do not know is evaluated by the caller's function on the recorded
+    pre-reset potential and streamed into the backward kernel; gradients equal those of the (rows, time)
+    Functions, which call the same function on the same potentials (reference sinabs/exodus/spike.py:251)."""
+    el, act, _ = L
+    calls = []
+    def custom(v, th):
+        calls.append((tuple(v.shape), tuple(th.shape)))
+        return 0.7 / (1.0 + ((v - th) / (0.4 * th)) ** 2)
+    kw = dict(tau_mem=12.0, tau_syn=tau_syn, min_v_mem=-0.5, train_alphas=True, surrogate_grad_fn=custom,
+              spike_fn=act.MaxSpike(2), spike_threshold=0.8)
+    native, rows = pair(el, el.LIF, **kw)
+    g = gen(17)
+    xa = (torch.rand(*shape, generator=g) * 4 - 1).cuda().requires_grad_(True)
+    xb = xa.detach().clone().requires_grad_(True)
+    assert native._use_native_layout(xa) and not rows._use_native_layout(xb)
+    w = torch.rand(shape, generator=g).cuda()
+    for k in range(2):                                       # the second pass starts from states that carry a graph
+        a = native(xa); b = rows(xb)
+        assert torch.equal(a, b)
+        ((a * w).sum() + native.v_mem.sum()).backward(retain_graph=True)
+        ((b * w).sum() + rows.v_mem.sum()).backward(retain_graph=True)
+    assert calls and len(calls[0][0]) == 3 and calls[0][1][1] == 1     # (batch, time, neurons), (batch, 1, neurons)
+    assert_close(xa.grad, xb.grad, "grad input")
+    for (k, p), (_, q) in zip(native.named_parameters(), rows.named_parameters()):
+        if q.grad is not None:
+            assert_close(p.grad, q.grad, f"grad {k}", rtol=1e-4, atol=1e-5 * max(1.0, (shape[0] * shape[1]) ** 0.5))
+    assert bool((xa.grad != 0).any())

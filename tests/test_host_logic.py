@@ -40,7 +40,7 @@ def test_library_exports_every_declared_symbol():
     extra = [l.split()[-1] for l in exported.splitlines() if " T " in l and not l.split()[-1].startswith("exodus_")]
     assert not extra, f"unexpected exported symbols: {extra}"
     lib.exodus_hip_abi_version.restype = ctypes.c_int
-    assert lib.exodus_hip_abi_version() == 2
+    assert lib.exodus_hip_abi_version() == 3
 
 
 def test_layer_entry_points_reject_too_wide_layers_before_touching_the_device():
@@ -49,11 +49,11 @@ def test_layer_entry_points_reject_too_wide_layers_before_touching_the_device():
     from sinabs.exodus import _hip
     wide = _hip.LAYER_MAX_NEURONS
     null = None
-    rc = _hip.lib.exodus_layer_lif_forward(*([null] * 16), 0, -1, 1, 1, 1, 4, wide, null)
+    rc = _hip.lib.exodus_layer_lif_forward(*([null] * 16), 0, -1, 1, 1, 0, 1, 4, wide, null)
     assert rc == 1
     rc = _hip.lib.exodus_layer_leaky_forward(*([null] * 6), 1, 1, 1, 4, wide, null)
     assert rc == 1
-    assert _hip.lib.exodus_layer_lif_forward(*([null] * 16), 0, -1, 1, 1, 0, 4, 8, null) == 0   # empty batch
+    assert _hip.lib.exodus_layer_lif_forward(*([null] * 16), 0, -1, 1, 1, 0, 0, 4, 8, null) == 0   # empty batch
 
 
 def test_loader_signatures_cover_the_header():
