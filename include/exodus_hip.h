@@ -197,7 +197,10 @@ int exodus_layer_lif_forward(float *out_spikes, float *out_vmem_rec, float *out_
  * vmem_init_grad, isyn_init_grad.  With surrogate_kind == EXODUS_SURR_TENSOR the derivative of
  * the spike function at every step comes from `surr` (batch,t,neurons) — what a caller computes
  * from the pre-reset potential record with any function of its own (the reference evaluates an
- * arbitrary Python callable there, sinabs/exodus/spike.py:251); otherwise `surr` is ignored. */
+ * arbitrary Python callable there, sinabs/exodus/spike.py:251); otherwise `surr` is ignored.
+ * grad_v_rec / grad_i_rec (batch,t,neurons, optional; with synapse both or none) are gradients
+ * arriving at the forward's per-step records of the post-reset potential and the synaptic current
+ * (the layer's `recordings` are differentiable, reference sinabs/exodus/layers/lif.py:256,290-293). */
 int exodus_layer_lif_backward(float *grad_input, float *alpha_mem_grad, float *alpha_syn_grad,
                               float *vmem_init_grad, float *isyn_init_grad, const float *grad_spikes,
                               const float *grad_v_last, const float *grad_i_last, const float *input,
@@ -206,7 +209,8 @@ int exodus_layer_lif_backward(float *grad_input, float *alpha_mem_grad, float *a
                               const float *membr_subtract, const float *theta, const float *theta_low,
                               int apply_theta_low, int max_num_spikes, int decay_early, int norm_input,
                               int surrogate_kind, float surr_p0, float surr_p1, const float *surr,
-                              int64_t batch, int64_t t, int64_t neurons, void *stream);
+                              const float *grad_v_rec, const float *grad_i_rec, int64_t batch, int64_t t,
+                              int64_t neurons, void *stream);
 
 /* Forward of the non-spiking leaky-integrator layer (ExpLeak) on (batch,t,neurons): per neuron
  *   xin = norm_input ? (1 - alpha) * input : input;  xin = decay_early ? xin * alpha : xin;

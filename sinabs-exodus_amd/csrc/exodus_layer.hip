@@ -389,16 +389,18 @@ __global__ void __launch_bounds__(BLOCK) layer_lif_forward(
 // KIND == EXODUS_SURR_TENSOR reads the surrogate derivative of every step from `surr` (a third
 // streamed tensor, whose register buffer costs the kernel one wave per SIMD); the other kinds
 // evaluate it from the rebuilt potential and ignore `surr`.
-template <bool SYN, int KIND, int CAPK, bool NT>
+// EXTRA: gradients also arrive at the per-step state records of the forward (grad_v_rec on the potential
+// after each reset, with synapse grad_i_rec on each synaptic current): two more streamed inputs.
+template <bool SYN, int KIND, int CAPK, bool NT, bool EXTRA>
 __global__ void __launch_bounds__(BWD_BLOCK)
-    __attribute__((amdgpu_waves_per_eu(KIND == EXODUS_SURR_TENSOR ? 2 : EXODUS_LAYER_BWD_WAVES,
-                                       KIND == EXODUS_SURR_TENSOR ? 2 : EXODUS_LAYER_BWD_WAVES)))
+    __attribute__((amdgpu_waves_per_eu((KIND == EXODUS_SURR_TENSOR || EXTRA) ? 2 : EXODUS_LAYER_BWD_WAVES,
+                                       (KIND == EXODUS_SURR_TENSOR || EXTRA) ? 2 : EXODUS_LAYER_BWD_WAVES)))
 layer_lif_backward(
     float *__restrict__ grad_x, float *__restrict__ alpha_mem_grad, float *__restrict__ alpha_syn_grad,
     float *__restrict__ v_init_grad, float *__restrict__ i_init_grad, const float *__restrict__ grad_spikes,
     const float *__restrict__ grad_v_last, const float *__restrict__ grad_i_last, const float *__restrict__ x,
-    const float *__restrict__ surr, const float *__restrict__ ckpt_v, const float *__restrict__ ckpt_i,
-    const LayerConsts p, const float p0,
+    const float *__restrict__ surr, const float *__restrict__ grad_v_rec, const float *__restrict__ grad_i_rec,
+    const float *__restrict__ ckpt_v, const float *__restrict__ ckpt_i, const LayerConsts p, const float p0,
     const float p1, const float inv_p0, const int64_t blocks_per_batch, const int64_t T, const int64_t M)
 {
     typedef BufIO<1, NT> IO;
@@ -414,6 +416,8 @@ layer_lif_backward(
     float *op = grad_x + (b * T) * M + m0;
     constexpr bool FROM_TENSOR = KIND == EXODUS_SURR_TENSOR;
     const float *srp = FROM_TENSOR ? surr + (b * T) * M + m0 : nullptr;
+    const float *qvp = EXTRA ? grad_v_rec + (b * T) * M + m0 : nullptr;
+    const float *qip = (EXTRA && SYN) ? grad_i_rec + (b * T) * M + m0 : nullptr;
     const float *cvp = ckpt_v + (b * n_ck) * M + m0;
     const float *cip = SYN ? ckpt_i + (b * n_ck) * M + m0 : nullptr;
     const unsigned voff = lane_off * 4u;
@@ -449,11 +453,14 @@ layer_lif_backward(
         const int64_t t0 = j * CKPT;
         const int len = GUARD ? static_cast<int>(T - t0) : CKPT;
         float xr[CKPT], gr[CKPT], vr[CKPT], sr[FROM_TENSOR ? CKPT : 1];
+        float qv[EXTRA ? CKPT : 1], qi[(EXTRA && SYN) ? CKPT : 1];
         {
             // always CKPT loads per tensor (steps past the end re-read the last step): a constant number
             // of loads in flight lets each use wait for its own load only
             const Rsrc rx = make_rsrc(xp + t0 * M), rg = make_rsrc(gp + t0 * M);
             const Rsrc rs = make_rsrc(FROM_TENSOR ? srp + t0 * M : nullptr);
+            const Rsrc rqv = make_rsrc(EXTRA ? qvp + t0 * M : nullptr);
+            const Rsrc rqi = make_rsrc((EXTRA && SYN) ? qip + t0 * M : nullptr);
             const unsigned last = static_cast<unsigned>(len - 1);
 #pragma unroll
             for (int k = 0; k < CKPT; ++k) {
@@ -461,6 +468,8 @@ layer_lif_backward(
                 xr[k] = IO::load(rx, voff, so);
                 gr[k] = IO::load(rg, voff, so);
                 if (FROM_TENSOR) sr[k] = IO::load(rs, voff, so);
+                if (EXTRA) qv[k] = IO::load(rqv, voff, so);
+                if (EXTRA && SYN) qi[k] = IO::load(rqi, voff, so);
             }
         }
         nr.vpost = ld_stream(cvp + j * M + lane_off);
@@ -487,7 +496,9 @@ layer_lif_backward(
                 const float vpost = __fsub_rn(v, __fmul_rn(nr.c, spike_count_fast<CAPK>(v, nr, cc)));
                 acc_m.add(lam, vpost);                          // lambda_{t+1} * vpost_t
                 const float through = __fsub_rn(1.0f, __fmul_rn(nr.c, sg));   // d vpost_t / d v_t
-                const float l = __fadd_rn(__fmul_rn(sg, gr[k]), __fmul_rn(through, h));
+                // a gradient on the recorded vpost_t joins what the next step sends down to vpost_t
+                const float below = EXTRA ? __fadd_rn(h, qv[EXTRA ? k : 0]) : h;
+                const float l = __fadd_rn(__fmul_rn(sg, gr[k]), __fmul_rn(through, below));
                 lam = v > nr.lo ? l : 0.f;                      // clamped (or NaN) steps pass nothing on
                 h = __fmul_rn(nr.am, lam);
                 acc_n.add(lam, cur_i);                          // lambda_t * i_t
@@ -495,6 +506,7 @@ layer_lif_backward(
                 if (SYN) {
                     const float mu_next = mu;
                     mu = __fadd_rn(hm, du);
+                    if (EXTRA) mu = __fadd_rn(mu, qi[(EXTRA && SYN) ? k : 0]);
                     hm = __fmul_rn(nr.as, mu);
                     acc_s.add(pair_new ? mu : mu_next, cur_i);
                     gr[k] = __fmul_rn(mu, xg);
@@ -801,21 +813,26 @@ inline bool bad3(int64_t b, int64_t t, int64_t m)
 
 template <bool SYN, int KIND, int CAPK>
 int launch_bwd(float *grad_x, float *am_g, float *as_g, float *v0_g, float *i0_g, const float *grad_spikes,
-               const float *gvl, const float *gil, const float *x, const float *surr, const float *ckpt_v,
-               const float *ckpt_i, const LayerConsts &p, float p0, float p1, int64_t B, int64_t T, int64_t M,
-               hipStream_t s)
+               const float *gvl, const float *gil, const float *x, const float *surr, const float *gvr,
+               const float *gir, const float *ckpt_v, const float *ckpt_i, const LayerConsts &p, float p0, float p1,
+               int64_t B, int64_t T, int64_t M, hipStream_t s)
 {
     const int64_t blocks_per_batch = (M + BWD_BLOCK - 1) / BWD_BLOCK;
     if (blocks_per_batch > 0x7fffffffLL / B) return hipErrorInvalidValue;
     const int64_t blocks = blocks_per_batch * B;
-    if (whole_lines(M, {grad_x, grad_spikes, x, surr}))
-        hipLaunchKernelGGL((layer_lif_backward<SYN, KIND, CAPK, true>), dim3(static_cast<unsigned>(blocks)), dim3(BWD_BLOCK), 0, s,
-                           grad_x, am_g, as_g, v0_g, i0_g, grad_spikes, gvl, gil, x, surr, ckpt_v, ckpt_i, p, p0, p1,
-                           p0 != 0.f ? 1.f / p0 : 0.f, blocks_per_batch, T, M);
-    else
-        hipLaunchKernelGGL((layer_lif_backward<SYN, KIND, CAPK, false>), dim3(static_cast<unsigned>(blocks)), dim3(BWD_BLOCK), 0, s,
-                           grad_x, am_g, as_g, v0_g, i0_g, grad_spikes, gvl, gil, x, surr, ckpt_v, ckpt_i, p, p0, p1,
-                           p0 != 0.f ? 1.f / p0 : 0.f, blocks_per_batch, T, M);
+#define EXODUS_LAUNCH(CK, NT, EX)                                                                                  \
+    hipLaunchKernelGGL((layer_lif_backward<SYN, KIND, CK, NT, EX>), dim3(static_cast<unsigned>(blocks)),          \
+                       dim3(BWD_BLOCK), 0, s, grad_x, am_g, as_g, v0_g, i0_g, grad_spikes, gvl, gil, x, surr, gvr, \
+                       gir, ckpt_v, ckpt_i, p, p0, p1, p0 != 0.f ? 1.f / p0 : 0.f, blocks_per_batch, T, M)
+    if (gvr) {
+        // gradients on the state records: one general instance per surrogate kind
+        EXODUS_LAUNCH(0, false, true);
+    } else if (whole_lines(M, {grad_x, grad_spikes, x, surr})) {
+        EXODUS_LAUNCH(CAPK, true, false);
+    } else {
+        EXODUS_LAUNCH(CAPK, false, false);
+    }
+#undef EXODUS_LAUNCH
     return static_cast<int>(hipGetLastError());
 }
 
@@ -958,7 +975,8 @@ EXODUS_API int exodus_layer_lif_backward(float *grad_input, float *alpha_mem_gra
                                          const float *membr_subtract, const float *theta, const float *theta_low,
                                          int apply_theta_low, int max_num_spikes, int decay_early, int norm_input,
                                          int surrogate_kind, float surr_p0, float surr_p1, const float *surr,
-                                         int64_t batch, int64_t t, int64_t neurons, void *stream)
+                                         const float *grad_v_rec, const float *grad_i_rec, int64_t batch, int64_t t,
+                                         int64_t neurons, void *stream)
 {
     if (bad3(batch, t, neurons)) return hipErrorInvalidValue;
     if (batch == 0 || t == 0 || neurons == 0) return hipSuccess;
@@ -968,6 +986,7 @@ EXODUS_API int exodus_layer_lif_backward(float *grad_input, float *alpha_mem_gra
         (apply_theta_low && !theta_low) || (syn && !ckpt_i) || (surrogate_kind == EXODUS_SURR_TENSOR && !surr))
         return hipErrorInvalidValue;
     if (surrogate_kind != EXODUS_SURR_TENSOR) surr = nullptr;
+    if (syn ? ((grad_v_rec != nullptr) != (grad_i_rec != nullptr)) : grad_i_rec != nullptr) return hipErrorInvalidValue;
     if (alpha_mem_grad && !vmem_post_initial) return hipErrorInvalidValue;
     if (syn && alpha_syn_grad && !decay_early && !isyn_initial) return hipErrorInvalidValue;
     LayerConsts p;
@@ -986,8 +1005,9 @@ EXODUS_API int exodus_layer_lif_backward(float *grad_input, float *alpha_mem_gra
     hipStream_t s = static_cast<hipStream_t>(stream);
 #define EXODUS_BWD(SYN, K)                                                                                        \
     return dispatch_bwd_cap<SYN, K>(p.cap, grad_input, alpha_mem_grad, alpha_syn_grad, vmem_init_grad,            \
-                                    isyn_init_grad, grad_spikes, grad_v_last, grad_i_last, input, surr, ckpt_v,   \
-                                    ckpt_i, p, surr_p0, surr_p1, batch, t, neurons, s)
+                                    isyn_init_grad, grad_spikes, grad_v_last, grad_i_last, input, surr,           \
+                                    grad_v_rec, grad_i_rec, ckpt_v, ckpt_i, p, surr_p0, surr_p1, batch, t,        \
+                                    neurons, s)
     switch (surrogate_kind) {
         case EXODUS_SURR_TENSOR: if (syn) EXODUS_BWD(true, EXODUS_SURR_TENSOR); EXODUS_BWD(false, EXODUS_SURR_TENSOR);
         case EXODUS_SURR_SINGLE_EXP: if (syn) EXODUS_BWD(true, EXODUS_SURR_SINGLE_EXP); EXODUS_BWD(false, EXODUS_SURR_SINGLE_EXP);

@@ -46,7 +46,7 @@ _SIGNATURES = {
     "exodus_probe_stream": ([_p, _p, _p, _i64, _p], _int),
     "exodus_layer_checkpoint_interval": ([], _int),
     "exodus_layer_lif_forward": ([_p] * 16 + [_int, _int, _int, _int, _int, _i64, _i64, _i64, _p], _int),
-    "exodus_layer_lif_backward": ([_p] * 18 + [_int, _int, _int, _int, _int, _f, _f, _p, _i64, _i64, _i64, _p], _int),
+    "exodus_layer_lif_backward": ([_p] * 18 + [_int, _int, _int, _int, _int, _f, _f, _p, _p, _p, _i64, _i64, _i64, _p], _int),
     "exodus_layer_leaky_forward": ([_p] * 6 + [_int, _int, _i64, _i64, _i64, _p], _int),
     "exodus_layer_leaky_backward": ([_p] * 9 + [_int, _int, _i64, _i64, _i64, _p], _int),
 }
@@ -488,9 +488,12 @@ def layerLifForward(input, vmemPostInitial, isynInitial, alphaMem, alphaSyn, mem
 def layerLifBackward(gradSpikes, gradVLast, gradILast, input, ckptV, ckptI, vmemPostInitial, isynInitial, alphaMem,
                      alphaSyn, membrSubtract, theta, thetaLow, applyThetaLow: bool, maxNumSpikes: int,
                      decayEarly: bool, normInput: bool, surrogateKind: int, surrP0: float, surrP1: float,
-                     gradInput: Optional[torch.Tensor] = None, surr: Optional[torch.Tensor] = None):
+                     gradInput: Optional[torch.Tensor] = None, surr: Optional[torch.Tensor] = None,
+                     gradVRec: Optional[torch.Tensor] = None, gradIRec: Optional[torch.Tensor] = None):
     """Returns (gradInput, alphaMemGrad, alphaSynGrad | None, vInitGrad, iInitGrad | None).
-    ``surrogateKind == SURR_TENSOR`` takes the spike function's derivative from ``surr`` (batch, time, neurons)."""
+    ``surrogateKind == SURR_TENSOR`` takes the spike function's derivative from ``surr`` (batch, time, neurons).
+    ``gradVRec`` / ``gradIRec`` (batch, time, neurons) are gradients on the forward's state records; one that is
+    missing while the other is given counts as zero."""
     _btm(input, "input")
     b, t, m = input.shape
     n = b * m
@@ -523,6 +526,16 @@ def layerLifBackward(gradSpikes, gradVLast, gradILast, input, ckptV, ckptI, vmem
             raise RuntimeError("surr must be given with the shape of input")
     else:
         surr = None
+    if not syn:
+        gradIRec = None
+    if gradVRec is not None or gradIRec is not None:
+        if gradVRec is None:
+            gradVRec = torch.zeros_like(input)
+        if syn and gradIRec is None:
+            gradIRec = torch.zeros_like(input)
+        for nm, x in (("gradVRec", gradVRec), ("gradIRec", gradIRec)):
+            if x is not None and _btm(x, nm, input).shape != input.shape:
+                raise RuntimeError(f"{nm} must have the shape of input")
     z = lambda: torch.zeros(n, dtype=torch.float32, device=input.device)
     am_g, v0_g = z(), z()
     as_g, i0_g = (z(), z()) if syn else (None, None)
@@ -533,7 +546,7 @@ def layerLifBackward(gradSpikes, gradVLast, gradILast, input, ckptV, ckptI, vmem
             _ptr(vmemPostInitial), _ptr(isynInitial) if syn else None, _ptr(alphaMem), _ptr(alphaSyn) if syn else None,
             _ptr(membrSubtract), _ptr(theta), _ptr(thetaLow), int(bool(applyThetaLow)), int(maxNumSpikes),
             int(bool(decayEarly)), int(bool(normInput)), int(surrogateKind), float(surrP0), float(surrP1), _ptr(surr),
-            b, t, m, _stream(input)), "exodus_layer_lif_backward")
+            _ptr(gradVRec), _ptr(gradIRec), b, t, m, _stream(input)), "exodus_layer_lif_backward")
     return gradInput, am_g, as_g, v0_g, i0_g
 
 

@@ -38,11 +38,15 @@ class SpikingLayerFunction(torch.autograd.Function):
         decay_early: bool,
         norm_input: bool,
         state_shape: Optional[tuple] = None,
+        record_states: bool = False,
     ):
-        """Returns ``(spikes (batch,time,neurons), v_mem_last, i_syn_last | None, spike_total)``;
-        ``v_mem_last`` is the potential after the last reset, ``spike_total`` a float64 scalar (the sum
-        of ``spikes``; a gradient arriving at it is added to every element of the gradient of
-        ``spikes``).  The final states come as flat vectors, or in ``state_shape`` if given."""
+        """Returns ``(spikes (batch,time,neurons), v_mem_last, i_syn_last | None, spike_total, v_mem_record |
+        None, i_syn_record | None)``; ``v_mem_last`` is the potential after the last reset, ``spike_total`` a
+        float64 scalar (the sum of ``spikes``; a gradient arriving at it is added to every element of the
+        gradient of ``spikes``).  The final states come as flat vectors, or in ``state_shape`` if given.
+        With ``record_states`` the potential after each reset and the synaptic current of every step come
+        back as (batch,time,neurons) tensors, differentiable like every other output (what the layer keeps
+        in ``recordings``, reference sinabs/exodus/layers/lif.py:256,290-293)."""
         kind, p0, p1 = classify_surrogate(surrogate_grad_fn)
         if inp.ndim != 3:
             raise ValueError("'inp' must be 3D, (batch, time, neurons)")
@@ -59,7 +63,8 @@ class SpikingLayerFunction(torch.autograd.Function):
         res = _hip.layerLifForward(
             inp, v_mem_init, i_syn_init, alpha_mem, alpha_syn, membrane_subtract, threshold, min_v_mem, apply_min,
             max_spikes, decay_early, norm_input, wantCheckpoints=need_grad, stateShape=state_shape,
-            wantPreReset=need_grad and kind == _hip.SURR_TENSOR,
+            wantPreReset=need_grad and kind == _hip.SURR_TENSOR and not record_states,
+            wantRecords=bool(record_states),
         )
         ctx.cfg = (syn, apply_min, max_spikes, bool(decay_early), bool(norm_input), kind, p0, p1)
         ctx.surrogate_grad_fn = surrogate_grad_fn if kind == _hip.SURR_TENSOR else None
@@ -67,18 +72,22 @@ class SpikingLayerFunction(torch.autograd.Function):
         if need_grad:
             saved = [inp, res["ckpt_v"], v_mem_init, alpha_mem, membrane_subtract, threshold]
             if kind == _hip.SURR_TENSOR:
-                saved.append(res["v_rec"])
+                # the function's argument is the potential before the reset; a post-reset record plus
+                # what the reset took away gives it back (up to one rounding)
+                v_pre = res["v_rec"]
+                if record_states:
+                    v_pre = torch.addcmul(v_pre, res["spikes"], membrane_subtract.view(inp.shape[0], 1, inp.shape[2]))
+                saved.append(v_pre)
             if syn:
                 saved += [res["ckpt_i"], i_syn_init, alpha_syn]
             if apply_min:
                 saved.append(min_v_mem)
             ctx.save_for_backward(*saved)
-        if syn:
-            return res["spikes"], res["v_last"], res["i_last"], res["spike_sum"]
-        return res["spikes"], res["v_last"], None, res["spike_sum"]
+        return (res["spikes"], res["v_last"], res["i_last"] if syn else None, res["spike_sum"],
+                res["v_rec"] if record_states else None, res["i_rec"] if (record_states and syn) else None)
 
     @staticmethod
-    def backward(ctx, grad_spikes, grad_v_last, grad_i_last, grad_total):
+    def backward(ctx, grad_spikes, grad_v_last, grad_i_last, grad_total, grad_v_rec=None, grad_i_rec=None):
         syn, apply_min, max_spikes, decay_early, norm_input, kind, p0, p1 = ctx.cfg
         saved = list(ctx.saved_tensors)
         inp, ckpt_v, v_mem_init, alpha_mem, membrane_subtract, threshold = saved[:6]
@@ -91,8 +100,8 @@ class SpikingLayerFunction(torch.autograd.Function):
             ckpt_i, i_syn_init, alpha_syn = rest[:3]
             rest = rest[3:]
         min_v_mem = rest[0] if apply_min else None
-        if grad_spikes is None and grad_v_last is None and grad_i_last is None and grad_total is None:
-            return (None,) * 13
+        if all(g is None for g in (grad_spikes, grad_v_last, grad_i_last, grad_total, grad_v_rec, grad_i_rec)):
+            return (None,) * 14
         if grad_spikes is None:
             grad_spikes = torch.zeros_like(inp)
         if grad_total is not None:                  # d(sum of spikes) / d(spike) = 1 for every element
@@ -109,8 +118,9 @@ class SpikingLayerFunction(torch.autograd.Function):
             cont(grad_spikes), cont(grad_v_last), cont(grad_i_last) if syn else None, inp, ckpt_v, ckpt_i,
             v_mem_init, i_syn_init, alpha_mem, alpha_syn, membrane_subtract, threshold, min_v_mem, apply_min,
             max_spikes, decay_early, norm_input, kind, p0, p1, surr=surr,
+            gradVRec=cont(grad_v_rec), gradIRec=cont(grad_i_rec) if syn else None,
         )
-        return (grad_input, g_am, g_as, g_v0, g_i0, None, None, None, None, None, None, None, None)
+        return (grad_input, g_am, g_as, g_v0, g_i0) + (None,) * 9
 
 
 class LeakyLayerFunction(torch.autograd.Function):

@@ -220,10 +220,7 @@ class LIF(LIFBase):
             return False
         if self.spike_fn is None:                      # leaky integrator: the output is the state record
             return self.tau_syn_calculated is None
-        if not self._needs_grad(input_data):           # inference: any surrogate, with or without records
-            return True
-        # with gradients the recorded states have to stay part of the autograd graph: (rows, time) Functions
-        return not self.record_states
+        return True
 
     def _needs_grad(self, input_data: torch.Tensor) -> bool:
         if not torch.is_grad_enabled():
@@ -290,7 +287,7 @@ class LIF(LIFBase):
                 self.i_syn = res["i_last"]
             self.firing_rate = (res["spike_sum"] / max(flat_input.numel(), 1)).float()
             return res["spikes"].reshape(input_data.shape)
-        spikes, v_last, i_last, spike_total = SpikingLayerFunction.apply(
+        spikes, v_last, i_last, spike_total, v_rec, i_rec = SpikingLayerFunction.apply(
             flat_input,
             alpha_mem,
             alpha_syn,
@@ -304,8 +301,13 @@ class LIF(LIFBase):
             self.decay_early,
             self.norm_input,
             state_shape,
+            self.record_states,
         )
         self.recordings = dict()
+        if self.record_states:
+            self.recordings["v_mem"] = v_rec.reshape(input_data.shape)
+            if has_syn:
+                self.recordings["i_syn"] = i_rec.reshape(input_data.shape)
         self.v_mem = v_last
         if has_syn:
             self.i_syn = i_last

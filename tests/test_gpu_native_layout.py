@@ -63,7 +63,7 @@ def test_native_equals_rows_path(L, batch, steps, trailing, tau_syn, decay_early
             assert_close(p.grad, q.grad, f"grad {k}", rtol=1e-4, atol=1e-5 * max(1.0, (batch * steps) ** 0.5))
 
 
-def test_native_iaf_squeeze_and_recorded_states_fallback(L):
+def test_native_iaf_squeeze_callable_surrogate_and_records(L):
     el, act, _ = L
     x = torch.rand(6 * 50, 2, 5, 5, generator=gen(3)).cuda()
     native, rows = pair(el, el.IAFSqueeze, batch_size=6, min_v_mem=-1.0)
@@ -72,7 +72,7 @@ def test_native_iaf_squeeze_and_recorded_states_fallback(L):
     xg = x.reshape(6, 50, 2, 5, 5).clone().requires_grad_(True)
     assert custom._use_native_layout(xg)                              # any callable runs on the layer kernels
     rec = el.IAF(record_states=True).cuda()
-    assert not rec._use_native_layout(xg)                             # differentiable records need the Functions
+    assert rec._use_native_layout(xg)                                 # and so do differentiable state records
     out = rec(xg); assert out.shape == (6, 50, 2, 5, 5)
     (out.sum() + rec.recordings["v_mem"].sum()).backward()
     assert xg.grad is not None and bool(torch.isfinite(xg.grad).all())
@@ -362,7 +362,6 @@ def test_inference_records_states_and_accepts_any_surrogate(L, tau_syn):
             if tau_syn is not None:
                 assert torch.equal(native.recordings["i_syn"], rows.recordings["i_syn"])
             assert torch.allclose(native.firing_rate, rows.firing_rate, rtol=1e-6, atol=0)
-    assert not native._use_native_layout(x.requires_grad_(True))      # records with gradients: the Functions
     with pytest.raises(ValueError):
         bad = el.LIF(tau_mem=10.0, min_v_mem=2.0).cuda()
         with torch.no_grad():
@@ -398,4 +397,46 @@ def test_any_callable_surrogate_on_the_layer_kernels(L, tau_syn, shape):
     for (k, p), (_, q) in zip(native.named_parameters(), rows.named_parameters()):
         if q.grad is not None:
             assert_close(p.grad, q.grad, f"grad {k}", rtol=1e-4, atol=1e-5 * max(1.0, (shape[0] * shape[1]) ** 0.5))
+    assert bool((xa.grad != 0).any())
+
+
+@pytest.mark.parametrize("tau_syn", [None, 6.0])
+@pytest.mark.parametrize("surrogate", ["single_exp", "callable"])
+@pytest.mark.parametrize("shape", [(3, 70, 5, 8), (2, 45, 37)])
+def test_recorded_states_are_differentiable_on_the_layer_kernels(L, tau_syn, surrogate, shape):
+    """``record_states=True`` while training: the records are outputs of the layer Function, and a loss on
+    them reaches input and parameters as it does through the (rows, time) Functions
+    (reference sinabs/exodus/layers/lif.py:256,290-293)."""
+    el, act, _ = L
+    kw = dict(tau_mem=12.0, tau_syn=tau_syn, min_v_mem=-0.5, train_alphas=True, record_states=True,
+              spike_fn=act.MaxSpike(2), spike_threshold=0.8)
+    if surrogate == "callable":
+        kw["surrogate_grad_fn"] = lambda v, th: 0.7 / (1.0 + ((v - th) / (0.4 * th)) ** 2)
+    native, rows = pair(el, el.LIF, **kw)
+    g = gen(23)
+    xa = (torch.rand(*shape, generator=g) * 4 - 1).cuda().requires_grad_(True)
+    xb = xa.detach().clone().requires_grad_(True)
+    assert native._use_native_layout(xa) and not rows._use_native_layout(xb)
+    w = [torch.rand(shape, generator=g).cuda() for _ in range(3)]
+    def loss(layer, out):
+        total = (out * w[0]).sum() + (layer.recordings["v_mem"] * w[1]).sum() + layer.v_mem.sum()
+        if tau_syn is not None:
+            total = total + (layer.recordings["i_syn"] * w[2]).sum()
+        return total
+    for k in range(2):
+        a = native(xa); b = rows(xb)
+        assert torch.equal(a, b)
+        assert torch.equal(native.recordings["v_mem"], rows.recordings["v_mem"])
+        if tau_syn is not None:
+            assert torch.equal(native.recordings["i_syn"], rows.recordings["i_syn"])
+        loss(native, a).backward(retain_graph=True); loss(rows, b).backward(retain_graph=True)
+    assert_close(xa.grad, xb.grad, "grad input")
+    for (k, p), (_, q) in zip(native.named_parameters(), rows.named_parameters()):
+        if q.grad is not None:
+            assert_close(p.grad, q.grad, f"grad {k}", rtol=1e-4, atol=1e-5 * max(1.0, (shape[0] * shape[1]) ** 0.5))
+    # a loss on the records alone (no gradient on the spikes at all)
+    native.reset_states(); rows.reset_states(); xa.grad = None; xb.grad = None
+    native(xa); rows(xb)
+    (native.recordings["v_mem"] * w[1]).sum().backward(); (rows.recordings["v_mem"] * w[1]).sum().backward()
+    assert_close(xa.grad, xb.grad, "grad input from the records alone")
     assert bool((xa.grad != 0).any())
