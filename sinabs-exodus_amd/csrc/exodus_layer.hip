@@ -80,9 +80,12 @@ typedef __amdgpu_buffer_rsrc_t Rsrc;
 // is marked non-temporal, which measures a few percent faster; but when a step's neurons do not start
 // and end on 128-byte lines (neuron count not a multiple of 32, or a view at an odd offset) neighbouring
 // waves and blocks share lines, and a non-temporal line is dropped before the neighbour gets to it:
-// reads from memory grow by a third and partial writes appear.  Such layers use NT = false, and their
-// kernels also put a workgroup barrier in front of every group of loads: waves that ask for the two halves
-// of a line at the same moment are served by one fetch, waves that have drifted apart are not.
+// reads from memory grow by a third and partial writes appear.  Such layers use NT = false.
+// All kernels put a workgroup barrier in front of every group of loads (the waves of a block share no
+// data; the barrier only keeps them at the same step): waves that ask for the two halves of a line at
+// the same moment are served by one fetch, waves that have drifted apart are not (+10-15 % where lines
+// are shared), and neighbouring pieces requested together also suit the memory better when nothing is
+// shared (+1-2 %).
 template <bool NT> struct Aux {
     static constexpr int load = (NT && EXODUS_NT_LOAD) ? 2 : 0;
     static constexpr int store = (NT && EXODUS_NT_STORE) ? 2 : 0;
@@ -274,7 +277,7 @@ __global__ void __launch_bounds__(BLOCK) layer_lif_forward(
         // FWD_UNROLL steps from t0; steps past the end re-read the last step (also when t0 itself lies
         // past the end), so every call issues exactly FWD_UNROLL loads
         auto fetch = [&](V(&dst)[FWD_UNROLL], int64_t t0) {
-            if (!NT) __syncthreads();                          // shared lines: keep the block's waves together
+            __syncthreads();                                   // keeps the block's waves at the same step
             if (t0 + FWD_UNROLL <= T) {
                 const Rsrc r = make_rsrc(xp + t0 * M);
 #pragma unroll
@@ -457,7 +460,7 @@ layer_lif_backward(
         const int len = GUARD ? static_cast<int>(T - t0) : CKPT;
         float xr[CKPT], gr[CKPT], vr[CKPT], sr[FROM_TENSOR ? CKPT : 1];
         float qv[EXTRA ? CKPT : 1], qi[(EXTRA && SYN) ? CKPT : 1];
-        if (!NT) __syncthreads();                              // shared lines: keep the block's waves together
+        __syncthreads();                                   // keeps the block's waves at the same step
         {
             // always CKPT loads per tensor (steps past the end re-read the last step): a constant number
             // of loads in flight lets each use wait for its own load only
@@ -614,7 +617,7 @@ __global__ void __launch_bounds__(BLOCK) layer_leaky_forward(float *__restrict__
     };
     // `spread` = step_bytes, or 0 for a fetch whose data will not be used (same count of loads, one step)
     auto fetch = [&](V(&dst)[U], int64_t t0, unsigned spread) {
-        if (!NT) __syncthreads();                              // shared lines: keep the block's waves together
+        __syncthreads();                                   // keeps the block's waves at the same step
         const Rsrc r = make_rsrc(xp + t0 * M);
 #pragma unroll
         for (int u = 0; u < U; ++u) dst[u] = IO::load(r, voff, u * spread);
@@ -714,7 +717,7 @@ __global__ void __launch_bounds__(BLOCK) layer_leaky_backward(
     };
     // steps t0 .. t0 + U - 1; `spread` = step_bytes, or 0 for a fetch whose data will not be used
     auto fetch = [&](Stage &s, int64_t t0, unsigned spread) {
-        if (!NT) __syncthreads();                              // shared lines: keep the block's waves together
+        __syncthreads();                                   // keeps the block's waves at the same step
         const Rsrc rg = make_rsrc(gp + t0 * M);
 #pragma unroll
         for (int u = 0; u < U; ++u) s.g[u] = IO::load(rg, voff, u * spread);
