@@ -489,8 +489,11 @@ def layerLifBackward(gradSpikes, gradVLast, gradILast, input, ckptV, ckptI, vmem
                      alphaSyn, membrSubtract, theta, thetaLow, applyThetaLow: bool, maxNumSpikes: int,
                      decayEarly: bool, normInput: bool, surrogateKind: int, surrP0: float, surrP1: float,
                      gradInput: Optional[torch.Tensor] = None, surr: Optional[torch.Tensor] = None,
-                     gradVRec: Optional[torch.Tensor] = None, gradIRec: Optional[torch.Tensor] = None):
-    """Returns (gradInput, alphaMemGrad, alphaSynGrad | None, vInitGrad, iInitGrad | None).
+                     gradVRec: Optional[torch.Tensor] = None, gradIRec: Optional[torch.Tensor] = None,
+                     wantAlphaMemGrad: bool = True, wantAlphaSynGrad: bool = True, wantVInitGrad: bool = True,
+                     wantIInitGrad: bool = True):
+    """Returns (gradInput, alphaMemGrad, alphaSynGrad | None, vInitGrad, iInitGrad | None); a per-neuron
+    gradient that is not wanted is neither computed nor allocated and comes back as None.
     ``surrogateKind == SURR_TENSOR`` takes the spike function's derivative from ``surr`` (batch, time, neurons).
     ``gradVRec`` / ``gradIRec`` (batch, time, neurons) are gradients on the forward's state records; one that is
     missing while the other is given counts as zero."""
@@ -536,9 +539,10 @@ def layerLifBackward(gradSpikes, gradVLast, gradILast, input, ckptV, ckptI, vmem
         for nm, x in (("gradVRec", gradVRec), ("gradIRec", gradIRec)):
             if x is not None and _btm(x, nm, input).shape != input.shape:
                 raise RuntimeError(f"{nm} must have the shape of input")
-    z = lambda: torch.zeros(n, dtype=torch.float32, device=input.device)
-    am_g, v0_g = z(), z()
-    as_g, i0_g = (z(), z()) if syn else (None, None)
+    # the kernel writes every neuron's entry of each vector it is given
+    z = lambda want: torch.empty(n, dtype=torch.float32, device=input.device) if want else None
+    am_g, v0_g = z(wantAlphaMemGrad), z(wantVInitGrad)
+    as_g, i0_g = z(syn and wantAlphaSynGrad), z(syn and wantIInitGrad)
     with torch.cuda.device(input.device):
         _check(lib.exodus_layer_lif_backward(
             _ptr(gradInput), _ptr(am_g), _ptr(as_g), _ptr(v0_g), _ptr(i0_g), _ptr(gradSpikes), _ptr(gradVLast),

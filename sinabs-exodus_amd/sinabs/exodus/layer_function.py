@@ -39,6 +39,7 @@ class SpikingLayerFunction(torch.autograd.Function):
         norm_input: bool,
         state_shape: Optional[tuple] = None,
         record_states: bool = False,
+        check_values: bool = True,
     ):
         """Returns ``(spikes (batch,time,neurons), v_mem_last, i_syn_last | None, spike_total, v_mem_record |
         None, i_syn_record | None)``; ``v_mem_last`` is the potential after the last reset, ``spike_total`` a
@@ -46,7 +47,8 @@ class SpikingLayerFunction(torch.autograd.Function):
         gradient of ``spikes``).  The final states come as flat vectors, or in ``state_shape`` if given.
         With ``record_states`` the potential after each reset and the synaptic current of every step come
         back as (batch,time,neurons) tensors, differentiable like every other output (what the layer keeps
-        in ``recordings``, reference sinabs/exodus/layers/lif.py:256,290-293)."""
+        in ``recordings``, reference sinabs/exodus/layers/lif.py:256,290-293).  ``check_values=False`` skips
+        the range checks of ``alpha`` / ``threshold`` (for a caller that knows they passed already)."""
         kind, p0, p1 = classify_surrogate(surrogate_grad_fn)
         if inp.ndim != 3:
             raise ValueError("'inp' must be 3D, (batch, time, neurons)")
@@ -56,7 +58,8 @@ class SpikingLayerFunction(torch.autograd.Function):
             membrane_subtract = threshold
         syn = alpha_syn is not None
         apply_min = min_v_mem is not None
-        check_parameters([alpha_mem, alpha_syn] if syn else [alpha_mem], threshold, min_v_mem)
+        if check_values:
+            check_parameters([alpha_mem, alpha_syn] if syn else [alpha_mem], threshold, min_v_mem)
 
         max_spikes = -1 if max_num_spikes_per_bin is None else int(max_num_spikes_per_bin)
         need_grad = any(ctx.needs_input_grad)
@@ -100,8 +103,9 @@ class SpikingLayerFunction(torch.autograd.Function):
             ckpt_i, i_syn_init, alpha_syn = rest[:3]
             rest = rest[3:]
         min_v_mem = rest[0] if apply_min else None
+        need = ctx.needs_input_grad
         if all(g is None for g in (grad_spikes, grad_v_last, grad_i_last, grad_total, grad_v_rec, grad_i_rec)):
-            return (None,) * 14
+            return (None,) * 15
         if grad_spikes is None:
             grad_spikes = torch.zeros_like(inp)
         if grad_total is not None:                  # d(sum of spikes) / d(spike) = 1 for every element
@@ -119,8 +123,9 @@ class SpikingLayerFunction(torch.autograd.Function):
             v_mem_init, i_syn_init, alpha_mem, alpha_syn, membrane_subtract, threshold, min_v_mem, apply_min,
             max_spikes, decay_early, norm_input, kind, p0, p1, surr=surr,
             gradVRec=cont(grad_v_rec), gradIRec=cont(grad_i_rec) if syn else None,
+            wantAlphaMemGrad=need[1], wantAlphaSynGrad=need[2], wantVInitGrad=need[3], wantIInitGrad=need[4],
         )
-        return (grad_input, g_am, g_as, g_v0, g_i0) + (None,) * 9
+        return (grad_input if need[0] else None, g_am, g_as, g_v0, g_i0) + (None,) * 10
 
 
 class LeakyLayerFunction(torch.autograd.Function):

@@ -222,6 +222,21 @@ class LIF(LIFBase):
             return self.tau_syn_calculated is None
         return True
 
+    def _value_stamp(self, state_shape):
+        """Identity and version of everything the range checks depend on.  The checks of decay factors,
+        threshold and lower bound make the host wait for the device (reference sinabs/exodus/spike.py:183-191
+        does so on every call).  The layer's own parameters only change between calls when somebody writes
+        to them, which their version counters show, so a layer whose parameters passed once skips the
+        checks until one of them is modified, replaced or moved (a write through ``tensor.data`` bypasses
+        the counter and is only seen together with the next ordinary write)."""
+        def stamp(name):
+            v = getattr(self, name, None)
+            if isinstance(v, torch.Tensor):
+                return (id(v), v._version, v.data_ptr(), tuple(v.shape))
+            return v
+        names = ("tau_mem", "alpha_mem", "tau_syn", "alpha_syn", "spike_threshold", "min_v_mem")
+        return tuple(stamp(n) for n in names) + (tuple(state_shape),)
+
     def _needs_grad(self, input_data: torch.Tensor) -> bool:
         if not torch.is_grad_enabled():
             return False
@@ -266,10 +281,15 @@ class LIF(LIFBase):
         else:
             membrane_subtract = expand_to_1d_contiguous(membrane_subtract, state_shape, dev)
         flat_input = input_data.reshape(batch_size, time_steps, int(np.prod(trailing_dim))).contiguous()
+        stamp = self._value_stamp(state_shape)
+        check_values = getattr(self, "_checked_values", None) != stamp
         if not self._needs_grad(input_data):
             # nothing to differentiate: no checkpoints, and the per-step states can be written along the way
             with torch.no_grad():
-                check_parameters([alpha_mem, alpha_syn] if has_syn else [alpha_mem], spike_threshold, min_v_mem)
+                if check_values:
+                    check_parameters([alpha_mem, alpha_syn] if has_syn else [alpha_mem], spike_threshold, min_v_mem)
+                    if not torch.cuda.is_current_stream_capturing():
+                        self._checked_values = stamp
                 res = _hip.layerLifForward(
                     flat_input, self.v_mem.flatten().contiguous(),
                     self.i_syn.flatten().contiguous() if has_syn else None, alpha_mem, alpha_syn, membrane_subtract,
@@ -302,7 +322,10 @@ class LIF(LIFBase):
             self.norm_input,
             state_shape,
             self.record_states,
+            check_values,
         )
+        if check_values and not torch.cuda.is_current_stream_capturing():
+            self._checked_values = stamp
         self.recordings = dict()
         if self.record_states:
             self.recordings["v_mem"] = v_rec.reshape(input_data.shape)

@@ -440,3 +440,45 @@ def test_recorded_states_are_differentiable_on_the_layer_kernels(L, tau_syn, sur
     (native.recordings["v_mem"] * w[1]).sum().backward(); (rows.recordings["v_mem"] * w[1]).sum().backward()
     assert_close(xa.grad, xb.grad, "grad input from the records alone")
     assert bool((xa.grad != 0).any())
+
+
+def test_value_checks_follow_parameter_versions(L, monkeypatch):
+    """The range checks wait for the device, so a layer repeats them only after one of its parameters was
+    written to; an invalid value is reported at the first call after the write and at every later one."""
+    el, act, _ = L
+    import sinabs.exodus.layer_function as lf
+    import sinabs.exodus.layers.neurons as nm
+    calls = []
+    real = lf.check_parameters
+    def counting(*a, **k):
+        calls.append(1)
+        return real(*a, **k)
+    monkeypatch.setattr(lf, "check_parameters", counting)
+    monkeypatch.setattr(nm, "check_parameters", counting)
+    layer = el.LIF(tau_mem=10.0, min_v_mem=-1.0, train_alphas=True).cuda()
+    x = torch.rand(2, 20, 16, generator=gen(2)).cuda()
+    layer(x); layer(x)
+    with torch.no_grad():
+        layer(x)
+    assert len(calls) == 1
+    with torch.no_grad():
+        layer.alpha_mem.fill_(1.5)
+    for _ in range(2):
+        with pytest.raises(ValueError):
+            layer(x)
+    with torch.no_grad():
+        with pytest.raises(ValueError):
+            layer(x)
+    assert len(calls) == 4
+    with torch.no_grad():
+        layer.alpha_mem.fill_(0.9)
+    layer(x); layer(x)
+    assert len(calls) == 5
+    with torch.no_grad():
+        layer.min_v_mem.fill_(3.0)                          # not below the threshold any more
+    with pytest.raises(ValueError):
+        layer(x)
+    with torch.no_grad():
+        layer.min_v_mem.fill_(-1.0)
+    layer(torch.rand(3, 20, 16, generator=gen(3)).cuda())   # new state shape: checked again
+    assert len(calls) == 7
