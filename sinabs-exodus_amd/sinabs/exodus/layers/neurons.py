@@ -98,9 +98,9 @@ class LIF(LIFBase):
         # layers with synapses run synapse and membrane in one kernel when the surrogate gradient
         # is one the kernels can evaluate; set to False to force the two separate Functions
         self.fuse_synapse = True
-        # spiking layers that do not record states run one kernel per direction on the input's own
-        # (batch, time, neurons) layout (no transposing copies, no stored v_mem / i_syn); set to False
-        # to force the (rows, time) Functions
+        # float32 device inputs run one kernel per direction on the input's own (batch, time, neurons)
+        # layout (no transposing copies, no stored v_mem / i_syn); set to False to force the
+        # (rows, time) Functions
         self.native_layout = True
 
     def _parse_activation_fn(self, spike_fn, reset_fn):
