@@ -243,6 +243,42 @@ def test_single_layer_compare_grads(L, train_alphas, norm_input, tau_syn, decay_
         assert abs(corr - 1) < 1e-5 and abs(scale - 1) < 1e-3
 
 
+@pytest.mark.parametrize("tau_syn", [None, 30.0])
+@pytest.mark.parametrize("train_alphas", [True, False])
+def test_loss_on_recorded_states_against_the_step_loop(L, tau_syn, train_alphas):
+    """A loss on ``recordings`` (potential after each reset, synaptic current) and on the spikes: gradients of
+    the layer kernels against torch autograd through the plain per-step loop (the records are differentiable
+    in the reference too, sinabs/exodus/layers/lif.py:256,290-293)."""
+    el, sl, _ = L
+    n_ch = 12
+    kw = dict(tau_mem=torch.linspace(10.0, 30.0, n_ch), tau_syn=tau_syn, spike_threshold=1.0, min_v_mem=-1.0,
+              norm_input=True, train_alphas=train_alphas, record_states=True)
+    plain = sl.LIF(**kw); plain.clip_mode = "max"
+    fast = el.LIF(**kw).cuda()
+    g = gen(31)
+    x = torch.rand((3, 40, n_ch), generator=g) * 8.0
+    w = [torch.rand((3, 40, n_ch), generator=g) for _ in range(3)]
+    v0 = torch.rand(3, n_ch, generator=g)
+    plain.v_mem = v0.clone(); fast.v_mem = v0.clone().cuda()
+    xa = x.clone().requires_grad_(True); xb = x.clone().cuda().requires_grad_(True)
+    def loss(layer, out, dev):
+        total = (out * w[0].to(dev)).sum() + (layer.recordings["v_mem"] * w[1].to(dev)).sum()
+        if tau_syn is not None:
+            total = total + (layer.recordings["i_syn"] * w[2].to(dev)).sum()
+        return total
+    a = plain(xa); loss(plain, a, "cpu").backward()
+    b = fast(xb); loss(fast, b, "cuda").backward()
+    assert fast._use_native_layout(xb)
+    assert torch.equal(a, b.cpu())
+    assert_close(fast.recordings["v_mem"].cpu(), plain.recordings["v_mem"], "recorded v_mem")
+    assert_close(xb.grad.cpu(), xa.grad, "grad input", rtol=1e-4, atol=1e-5)
+    gp = {k: p.grad for k, p in plain.named_parameters() if p.grad is not None}
+    gf = {k: p.grad.cpu() for k, p in fast.named_parameters() if p.grad is not None}
+    assert set(gp) == set(gf) and len(gp) > 0
+    for k in gp:
+        assert_close(gf[k], gp[k], f"grad {k}", rtol=1e-3, atol=1e-5)
+
+
 def test_alpha_grad_trace_per_timestep(L):
     """reference tests/test_lif.py:426-485: d out[t] / d alpha_mem for every t, lower bound 0, synapses."""
     el, sl, _ = L
