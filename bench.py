@@ -300,6 +300,10 @@ def measure_ceilings(args, torch, hip, dev):
         return e0.elapsed_time(e1) / args.steps
 
     res = {"workload": w["name"], "tensor_GB": n * 4 / 1e9, "peak_GBs": HBM_PEAK_GBS}
+    ms = timed(lambda: hip.probeRead(a))
+    res["flat_read_only"] = {"ms": ms, "GBs": n * 4 / ms / 1e6}
+    ms = timed(lambda: hip.probeWrite(out))
+    res["flat_write_only"] = {"ms": ms, "GBs": n * 4 / ms / 1e6}
     ms = timed(lambda: hip.probeStream(out, a))
     res["flat_copy_1r1w"] = {"ms": ms, "GBs": n * 8 / ms / 1e6}
     ms = timed(lambda: hip.probeStream(out, a, b))

@@ -260,6 +260,11 @@ int exodus_spike_backward(float *input_grad, const float *surr, const float *out
  * exactly known traffic to scale hardware counters by. */
 int exodus_probe_stream(float *dst, const float *a, const float *b, int64_t n, void *stream);
 
+/* The same accesses in one direction only: read n floats of `a` (nothing is written), or write n
+ * zeros to `dst`.  What the memory gives reads alone and writes alone, next to the mixed figure. */
+int exodus_probe_read(const float *a, int64_t n, void *stream);
+int exodus_probe_write(float *dst, int64_t n, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

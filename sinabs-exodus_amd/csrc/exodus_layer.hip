@@ -930,6 +930,27 @@ __global__ void __launch_bounds__(256) probe_stream(f32x4 *__restrict__ dst, con
     }
 }
 
+// one direction only: READ loads and hands every value to an empty asm statement (so the loads stay
+// although nothing is done with them), !READ writes zeros
+template <bool READ>
+__global__ void __launch_bounds__(256) probe_one_way(f32x4 *__restrict__ dst, const f32x4 *__restrict__ a,
+                                                     const int64_t n_chunks)
+{
+    const int64_t base = (static_cast<int64_t>(blockIdx.x) * PROBE_PER_THREAD) * 256 + threadIdx.x;
+#pragma unroll
+    for (int k = 0; k < PROBE_PER_THREAD; ++k) {
+        const int64_t i = base + k * 256;
+        if (i < n_chunks) {
+            if (READ) {
+                const f32x4 v = ld_stream(a + i);
+                asm volatile("" : : "v"(v));
+            } else {
+                st_stream(f32x4{0.f, 0.f, 0.f, 0.f}, dst + i);
+            }
+        }
+    }
+}
+
 }  // namespace
 
 extern "C" {
@@ -1124,6 +1145,32 @@ EXODUS_API int exodus_probe_stream(float *dst, const float *a, const float *b, i
         hipLaunchKernelGGL((probe_stream<false>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s,
                            reinterpret_cast<f32x4 *>(dst), reinterpret_cast<const f32x4 *>(a),
                            static_cast<const f32x4 *>(nullptr), n_chunks);
+    return static_cast<int>(hipGetLastError());
+}
+
+EXODUS_API int exodus_probe_read(const float *a, int64_t n, void *stream)
+{
+    if (n < 0 || (n % 4) != 0 || !a || (reinterpret_cast<uintptr_t>(a) & 15u)) return hipErrorInvalidValue;
+    if (n == 0) return hipSuccess;
+    const int64_t n_chunks = n / 4;
+    const int64_t blocks = (n_chunks + 256 * PROBE_PER_THREAD - 1) / (256 * PROBE_PER_THREAD);
+    if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
+    hipLaunchKernelGGL((probe_one_way<true>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), static_cast<f32x4 *>(nullptr),
+                       reinterpret_cast<const f32x4 *>(a), n_chunks);
+    return static_cast<int>(hipGetLastError());
+}
+
+EXODUS_API int exodus_probe_write(float *dst, int64_t n, void *stream)
+{
+    if (n < 0 || (n % 4) != 0 || !dst || (reinterpret_cast<uintptr_t>(dst) & 15u)) return hipErrorInvalidValue;
+    if (n == 0) return hipSuccess;
+    const int64_t n_chunks = n / 4;
+    const int64_t blocks = (n_chunks + 256 * PROBE_PER_THREAD - 1) / (256 * PROBE_PER_THREAD);
+    if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
+    hipLaunchKernelGGL((probe_one_way<false>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), reinterpret_cast<f32x4 *>(dst),
+                       static_cast<const f32x4 *>(nullptr), n_chunks);
     return static_cast<int>(hipGetLastError());
 }
 

@@ -44,6 +44,8 @@ _SIGNATURES = {
     "exodus_spike_forward": ([_p, _p, _f, _f, _f, _f, _int, _int, _i64, _i64, _p], _int),
     "exodus_spike_backward": ([_p] * 4 + [_f, _f, _i64, _i64, _p], _int),
     "exodus_probe_stream": ([_p, _p, _p, _i64, _p], _int),
+    "exodus_probe_read": ([_p, _i64, _p], _int),
+    "exodus_probe_write": ([_p, _i64, _p], _int),
     "exodus_layer_checkpoint_interval": ([], _int),
     "exodus_layer_lif_forward": ([_p] * 16 + [_int, _int, _int, _int, _int, _i64, _i64, _i64, _p], _int),
     "exodus_layer_lif_backward": ([_p] * 18 + [_int, _int, _int, _int, _int, _f, _f, _p, _p, _p, _i64, _i64, _i64, _p], _int),
@@ -414,6 +416,20 @@ def probeStream(dst, a, b=None) -> None:
         raise RuntimeError("dst, a and b must have the same number of elements")
     with torch.cuda.device(a.device):
         _check(lib.exodus_probe_stream(_ptr(dst), _ptr(a), _ptr(b), a.numel(), _stream(a)), "exodus_probe_stream")
+
+
+def probeRead(a) -> None:
+    """Read all of ``a`` with flat streaming accesses and write nothing."""
+    _dev(a, "a")
+    with torch.cuda.device(a.device):
+        _check(lib.exodus_probe_read(_ptr(a), a.numel(), _stream(a)), "exodus_probe_read")
+
+
+def probeWrite(dst) -> None:
+    """Fill ``dst`` with zeros with flat streaming accesses."""
+    _dev(dst, "dst")
+    with torch.cuda.device(dst.device):
+        _check(lib.exodus_probe_write(_ptr(dst), dst.numel(), _stream(dst)), "exodus_probe_write")
 
 
 # neurons per batch element the layer-layout entry points accept (they return invalid-value beyond)

@@ -216,3 +216,15 @@ def test_argument_errors(hip):
         hip.leakyForward(x.double(), r.double(), r.double())
     with pytest.raises(RuntimeError):            # raw ABI: bad surrogate kind is rejected on the host
         hip.lifBackwardFused(x, None, x, None, r, r, r, None, False, -1, 17)
+
+
+def test_one_way_streaming_probes():
+    """The measurement probes: the write probe zeroes exactly its range, the read probe writes nothing."""
+    from sinabs.exodus import _hip
+    n = 4 * 1000 + 4
+    buf = torch.full((n + 8,), 3.0, device="cuda")
+    _hip.probeWrite(buf[4:4 + n])
+    assert bool((buf[4:4 + n] == 0).all()) and bool((buf[:4] == 3).all()) and bool((buf[4 + n:] == 3).all())
+    a = torch.randn(n, device="cuda"); keep = a.clone()
+    _hip.probeRead(a)
+    assert torch.equal(a, keep)
