@@ -222,6 +222,11 @@ class LIF(LIFBase):
             return self.tau_syn_calculated is None
         return True
 
+    def _decay_source(self, which: str):
+        """The parameter a decay factor derives from: the factor itself or its time constant (None for a
+        layer without leak, whose factor is the constant 1)."""
+        return getattr(self, ("alpha_" if self.train_alphas else "tau_") + which, None)
+
     def _value_stamp(self, state_shape):
         """Identity and version of everything the range checks depend on.  The checks of decay factors,
         threshold and lower bound make the host wait for the device (reference sinabs/exodus/spike.py:183-191
@@ -237,6 +242,36 @@ class LIF(LIFBase):
         names = ("tau_mem", "alpha_mem", "tau_syn", "alpha_syn", "spike_threshold", "min_v_mem")
         return tuple(stamp(n) for n in names) + (tuple(state_shape),)
 
+    def _per_neuron(self, name: str, source, state_shape, dev, value=None) -> torch.Tensor:
+        """One float32 entry per neuron of ``state_shape`` for the layer quantity ``name``
+        (``expand_to_1d_contiguous``).  ``source`` is the parameter or number it derives from and ``value`` a
+        callable giving the quantity itself when it is not the source (a decay factor computed from a time
+        constant).  Quantities that take no part in differentiation are kept until their source is written
+        to, replaced or moved: a layer call then launches no kernels for them."""
+        compute = (lambda: source) if value is None else value
+        if isinstance(source, torch.Tensor):
+            if (source.requires_grad and torch.is_grad_enabled()) or torch.cuda.is_current_stream_capturing():
+                return expand_to_1d_contiguous(compute(), state_shape, dev)
+            key = (id(source), source._version, source.data_ptr(), tuple(source.shape), tuple(state_shape), str(dev))
+        else:
+            if torch.cuda.is_current_stream_capturing():
+                return expand_to_1d_contiguous(compute(), state_shape, dev)
+            key = (source, tuple(state_shape), str(dev))
+        cache = self.__dict__.setdefault("_per_neuron_cache", {})
+        hit = cache.get(name)
+        if hit is not None and hit[0] == key:
+            return hit[1]
+        out = expand_to_1d_contiguous(compute(), state_shape, dev).detach()
+        cache[name] = (key, out)
+        return out
+
+    def _set_state(self, name: str, value: torch.Tensor) -> None:
+        """Replace a state buffer (``nn.Module.__setattr__`` does the same after a longer search)."""
+        if name in self._buffers:
+            self._buffers[name] = value
+        else:
+            setattr(self, name, value)
+
     def _needs_grad(self, input_data: torch.Tensor) -> bool:
         if not torch.is_grad_enabled():
             return False
@@ -248,7 +283,8 @@ class LIF(LIFBase):
         state_shape = (batch_size, *trailing_dim)
         if not self.is_state_initialised() or not self.state_has_shape(state_shape):
             self.init_state_with_shape(state_shape)
-        alpha_mem = expand_to_1d_contiguous(self.alpha_mem_calculated, state_shape, self.v_mem.device)
+        alpha_mem = self._per_neuron("alpha_mem", self._decay_source("mem"), state_shape, self.v_mem.device,
+                                     lambda: self.alpha_mem_calculated)
         out, v_last, total = LeakyLayerFunction.apply(
             input_data.reshape(batch_size, time_steps, int(np.prod(trailing_dim))).contiguous(),
             alpha_mem,
@@ -259,7 +295,7 @@ class LIF(LIFBase):
         )
         out = out.reshape(input_data.shape)
         self.recordings = {"v_mem": out} if self.record_states else dict()
-        self.v_mem = v_last
+        self._set_state("v_mem", v_last)
         self.firing_rate = (total / max(out.numel(), 1)).float()
         return out
 
@@ -271,15 +307,17 @@ class LIF(LIFBase):
             self.init_state_with_shape(state_shape)
         dev = self.v_mem.device
         has_syn = self.tau_syn_calculated is not None
-        alpha_mem = expand_to_1d_contiguous(self.alpha_mem_calculated, state_shape, dev)
-        alpha_syn = expand_to_1d_contiguous(self.alpha_syn_calculated, state_shape, dev) if has_syn else None
-        spike_threshold = expand_to_1d_contiguous(self.spike_threshold, state_shape, dev)
-        min_v_mem = None if self.min_v_mem is None else expand_to_1d_contiguous(self.min_v_mem, state_shape, dev)
+        alpha_mem = self._per_neuron("alpha_mem", self._decay_source("mem"), state_shape, dev,
+                                     lambda: self.alpha_mem_calculated)
+        alpha_syn = self._per_neuron("alpha_syn", self._decay_source("syn"), state_shape, dev,
+                                     lambda: self.alpha_syn_calculated) if has_syn else None
+        spike_threshold = self._per_neuron("spike_threshold", self.spike_threshold, state_shape, dev)
+        min_v_mem = None if self.min_v_mem is None else self._per_neuron("min_v_mem", self.min_v_mem, state_shape, dev)
         membrane_subtract = self.reset_fn.subtract_value
         if membrane_subtract is None:
             membrane_subtract = spike_threshold
         else:
-            membrane_subtract = expand_to_1d_contiguous(membrane_subtract, state_shape, dev)
+            membrane_subtract = self._per_neuron("membrane_subtract", membrane_subtract, state_shape, dev)
         flat_input = input_data.reshape(batch_size, time_steps, int(np.prod(trailing_dim))).contiguous()
         stamp = self._value_stamp(state_shape)
         check_values = getattr(self, "_checked_values", None) != stamp
@@ -302,9 +340,9 @@ class LIF(LIFBase):
                 self.recordings["v_mem"] = res["v_rec"].reshape(input_data.shape)
                 if has_syn:
                     self.recordings["i_syn"] = res["i_rec"].reshape(input_data.shape)
-            self.v_mem = res["v_last"]
+            self._set_state("v_mem", res["v_last"])
             if has_syn:
-                self.i_syn = res["i_last"]
+                self._set_state("i_syn", res["i_last"])
             self.firing_rate = (res["spike_sum"] / max(flat_input.numel(), 1)).float()
             return res["spikes"].reshape(input_data.shape)
         spikes, v_last, i_last, spike_total, v_rec, i_rec = SpikingLayerFunction.apply(
@@ -331,9 +369,9 @@ class LIF(LIFBase):
             self.recordings["v_mem"] = v_rec.reshape(input_data.shape)
             if has_syn:
                 self.recordings["i_syn"] = i_rec.reshape(input_data.shape)
-        self.v_mem = v_last
+        self._set_state("v_mem", v_last)
         if has_syn:
-            self.i_syn = i_last
+            self._set_state("i_syn", i_last)
         self.firing_rate = (spike_total / max(spikes.numel(), 1)).float()
         return spikes.reshape(input_data.shape)
 

@@ -482,3 +482,42 @@ def test_value_checks_follow_parameter_versions(L, monkeypatch):
         layer.min_v_mem.fill_(-1.0)
     layer(torch.rand(3, 20, 16, generator=gen(3)).cuda())   # new state shape: checked again
     assert len(calls) == 7
+
+
+def test_kept_parameter_vectors_follow_writes_to_the_parameters(L):
+    """Per-neuron vectors of parameters that are not differentiated are kept between calls; a write to the
+    parameter, a replacement or a new state shape must show in the very next call."""
+    el, act, _ = L
+    x = (torch.rand(2, 40, 24, generator=gen(5)) * 3).cuda()
+    def fresh(**kw):
+        layer = el.LIF(**kw).cuda()
+        with torch.no_grad():
+            return layer(x), layer.v_mem
+    layer = el.LIF(tau_mem=10.0, min_v_mem=-1.0, spike_threshold=1.0).cuda()
+    with torch.no_grad():
+        for _ in range(2):
+            layer.reset_states(); a = layer(x)
+        want, _ = fresh(tau_mem=10.0, min_v_mem=-1.0, spike_threshold=1.0)
+        assert torch.equal(a, want)
+        layer.spike_threshold.fill_(0.5)                      # in-place write
+        layer.reset_states(); a = layer(x)
+        want, _ = fresh(tau_mem=10.0, min_v_mem=-1.0, spike_threshold=0.5)
+        assert torch.equal(a, want)
+        layer.tau_mem.fill_(4.0)
+        layer.reset_states(); a = layer(x)
+        want, _ = fresh(tau_mem=4.0, min_v_mem=-1.0, spike_threshold=0.5)
+        assert torch.equal(a, want)
+        layer.min_v_mem = torch.nn.Parameter(torch.tensor(-0.2).cuda(), requires_grad=False)   # replacement
+        layer.reset_states(); a = layer(x)
+        want, _ = fresh(tau_mem=4.0, min_v_mem=-0.2, spike_threshold=0.5)
+        assert torch.equal(a, want)
+        b = layer(x[:1])                                       # other state shape
+        other = el.LIF(tau_mem=4.0, min_v_mem=-0.2, spike_threshold=0.5).cuda()
+        assert torch.equal(b, other(x[:1]))
+    # with gradients the decay factor is rebuilt from the time constant in every call
+    layer = el.LIF(tau_mem=10.0).cuda()
+    assert layer.tau_mem.requires_grad
+    layer(x).sum().backward()
+    g1 = layer.tau_mem.grad.clone(); layer.tau_mem.grad = None
+    layer.reset_states(); layer(x).sum().backward()
+    assert torch.equal(layer.tau_mem.grad, g1) and bool(g1.abs() > 0)
