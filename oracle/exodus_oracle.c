@@ -23,6 +23,11 @@
  *                               the O(T) reverse recurrence, torch autograd BPTT
  *   oracle_lif_backward_alpha   torch autograd BPTT (only where step 0 is not clipped or
  *                               v_init == 0, see the note at the function)
+ *   oracle_spike_forward        notebook cells 2/4/6 on cumsum(input); bit-equality with
+ *                               oracle_lif_forward on a dyadic grid where all arithmetic is exact
+ *   oracle_spike_backward       equality with oracle_lif_backward at alpha == 1; quadratic sum ==
+ *                               reverse recurrence in fp64.  For alpha != 1 and for clipped steps
+ *                               nothing else holds it: parity unpinned there
  */
 #include <math.h>
 #include <stdint.h>
