@@ -367,6 +367,19 @@ def measure_conv_snn(args, torch, dev):
     return res
 
 
+def without_cycle_option(argv):
+    """The command line without ``--after-hbm-cycle [N]`` (for the child process that measures)."""
+    rest, skip = [], False
+    for k, a in enumerate(argv):
+        if skip:
+            skip = False
+        elif a == "--after-hbm-cycle":
+            skip = k + 1 < len(argv) and argv[k + 1].isdigit()
+        elif not a.startswith("--after-hbm-cycle="):
+            rest.append(a)
+    return rest
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -407,15 +420,7 @@ def main():
                  "torch.cuda.synchronize(); print(f'[hbm cycle] {n} x 4 GiB allocated, released on exit', flush=True)")
         for _ in range(args.after_hbm_cycle):
             subprocess.run([sys.executable, "-c", cycle], check=True, stdout=sys.stderr)
-        rest, skip = [], False
-        for k, a in enumerate(sys.argv[1:]):
-            if skip:
-                skip = False
-            elif a == "--after-hbm-cycle":
-                nxt = sys.argv[k + 2] if k + 2 < len(sys.argv) else ""
-                skip = nxt.isdigit()
-            elif not a.startswith("--after-hbm-cycle="):
-                rest.append(a)
+        rest = without_cycle_option(sys.argv[1:])
         env = dict(os.environ, EXODUS_BENCH_AFTER_HBM_CYCLE=str(args.after_hbm_cycle))
         sys.exit(subprocess.run([sys.executable, os.path.abspath(__file__)] + rest, env=env).returncode)
 

@@ -179,6 +179,18 @@ def test_bench_refuses_more_than_one_gpu():
     assert out.returncode != 0 and "one GPU" in (out.stderr + out.stdout)
 
 
+def test_bench_child_command_line_drops_the_cycle_option():
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("bench", os.path.join(ROOT, "bench.py"))
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    f = bench.without_cycle_option
+    assert f(["--steps", "5", "--after-hbm-cycle", "3", "--workload", "c2"]) == ["--steps", "5", "--workload", "c2"]
+    assert f(["--after-hbm-cycle", "--ceilings"]) == ["--ceilings"]
+    assert f(["--after-hbm-cycle=4", "--path", "rows"]) == ["--path", "rows"]
+    assert f(["--workload", "c3"]) == ["--workload", "c3"]
+
+
 def test_parameter_validation_modes():
     from sinabs.exodus import _validate as val
     good, bad = torch.tensor([0.0, 0.5, 1.0]), torch.tensor([0.5, 1.5])
