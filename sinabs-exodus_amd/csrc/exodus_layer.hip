@@ -299,8 +299,13 @@ __global__ void __launch_bounds__(BLOCK) layer_lif_forward(
                     lane_put<NPL>(cv, e, nr[e].vpost);
                     lane_put<NPL>(ci, e, nr[e].i);
                 }
-                st_stream(cv, reinterpret_cast<V *>(cvp + j * M + lane_off));
-                if (cip) st_stream(ci, reinterpret_cast<V *>(cip + j * M + lane_off));
+                // checkpoints follow the hint of the other streamed tensors (their rows share lines alike)
+                V *cvq = reinterpret_cast<V *>(cvp + j * M + lane_off);
+                if (NT) st_stream(cv, cvq); else *cvq = cv;
+                if (cip) {
+                    V *ciq = reinterpret_cast<V *>(cip + j * M + lane_off);
+                    if (NT) st_stream(ci, ciq); else *ciq = ci;
+                }
             }
             my_spikes += static_cast<double>(part);
             part = 0.f;
@@ -479,8 +484,8 @@ layer_lif_backward(
                 if (EXTRA && SYN) qi[k] = IO::load(rqi, voff, so);
             }
         }
-        nr.vpost = ld_stream(cvp + j * M + lane_off);
-        nr.i = SYN ? ld_stream(cip + j * M + lane_off) : 0.f;
+        nr.vpost = NT ? ld_stream(cvp + j * M + lane_off) : cvp[j * M + lane_off];
+        nr.i = SYN ? (NT ? ld_stream(cip + j * M + lane_off) : cip[j * M + lane_off]) : 0.f;
 
         // rebuild the block: vr[k] = pre-reset potential, xr[k] = synaptic current (the value that
         // was normalised and fed to the membrane; without synapse that is the input itself)
