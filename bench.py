@@ -389,6 +389,10 @@ def main():
     ap.add_argument("--path", default="layer", choices=["layer", "rows"],
                     help="layer: kernels on the layer's (batch, time, neurons) layout (what the layers run); "
                          "rows: the (rows, time) kernels behind the autograd Functions")
+    ap.add_argument("--shape", default=None, metavar="B,T,M",
+                    help="run the chosen workload's layer type and options at another (batch, steps, neurons) shape, "
+                         "e.g. a neuron count that does not fill 128-byte memory lines; such a run is a measurement "
+                         "aid, not the benchmark (roofline.traffic is then null)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also launch one plain elementwise kernel (torch.neg) over exactly 1 GiB before the timed region, so that a "
@@ -413,6 +417,11 @@ def main():
         sys.exit("bench.py: this build measures one GPU only (rows shard across GPUs without exchange; "
                  "no multi-GPU figure is produced). Run with --gpus 1.")
 
+    if args.shape:
+        b_, t_, m_ = (int(v) for v in args.shape.split(","))
+        w_ = WORKLOADS[args.workload]
+        WORKLOADS[args.workload] = dict(w_, batch=b_, steps=t_, neurons=m_,
+                                        name=w_["name"] + f" -- at shape ({b_},{t_},{m_})")
     if args.after_hbm_cycle:
         import subprocess
         cycle = ("import torch; free, _ = torch.cuda.mem_get_info(); n = int((free - 6 * 2**30) // (4 * 2**30)); "
@@ -496,7 +505,8 @@ def main():
                       if os.environ.get("EXODUS_BENCH_AFTER_HBM_CYCLE") else {})},
         "roofline": {
             "bound": "hbm", "kernel": dom_name, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC.get((args.workload, dom_name)),
+            "frac": achieved / HBM_PEAK_GBS,
+            "traffic": None if args.shape else MEASURED_TRAFFIC.get((args.workload, dom_name)),
             "kernel_ms": dom_ms, "algorithmic_bytes_per_launch": N * T * dom_bytes,
             "other_kernel": {"kernel": other_name, "kernel_ms": other_ms,
                              "achieved": N * T * other_bytes / (other_ms * 1e-3) / 1e9},
