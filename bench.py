@@ -41,19 +41,23 @@ WORKLOADS = {
                batch=8, steps=100, neurons=256, mean=None, std=None, bytes=(12, 12)),
 }
 
-# HBM traffic per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by the
-# reading of a plain copy of known size); bytes per launch of the dominant kernel, or None.
+# HBM traffic per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (FETCH_SIZE x2 + WRITE_SIZE
+# x1 KiB, factors from a plain elementwise kernel over exactly 1 GiB in the same runs): bytes per launch
+# and the committed summary the figure comes from.  These are measurements of the kernels as they were
+# when the summary was made; a kernel that changes needs its counters taken again.
 MEASURED_TRAFFIC = {
-    # FETCH_SIZE x2 + WRITE_SIZE x1 (KiB), factors from the 1 GiB probe kernel
-    ("c5", "exodus_layer_lif_backward"): 25.74e9,
-    ("c5", "exodus_layer_lif_forward"): 17.34e9,
-    ("c5", "exodus_synlif_backward"): 33.79e9,
-    ("c5", "exodus_synlif_forward"): 33.64e9,
-    ("c2", "exodus_layer_lif_backward"): 15.37e9,
-    ("c2", "exodus_layer_lif_forward"): 10.30e9,
-    ("c3", "exodus_layer_leaky_backward"): 3.15e9,
-    ("c3", "exodus_layer_leaky_forward"): 2.10e9,
+    ("c5", "exodus_layer_lif_backward"): (25.74e9, "profiles/layer_lif_c5_pmc.md"),
+    ("c5", "exodus_layer_lif_forward"): (17.34e9, "profiles/layer_lif_c5_pmc.md"),
+    ("c5", "exodus_synlif_backward"): (33.79e9, "profiles/rows_synlif_c5_pmc.md"),
+    ("c5", "exodus_synlif_forward"): (33.64e9, "profiles/rows_synlif_c5_pmc.md"),
+    ("c2", "exodus_layer_lif_backward"): (15.37e9, "profiles/layer_lif_c2_kernel_stats_pmc.md"),
+    ("c2", "exodus_layer_lif_forward"): (10.30e9, "profiles/layer_lif_c2_kernel_stats_pmc.md"),
+    ("c3", "exodus_layer_leaky_backward"): (3.15e9, "profiles/layer_leaky_c3_kernel_stats_pmc.md"),
+    ("c3", "exodus_layer_leaky_forward"): (2.10e9, "profiles/layer_leaky_c3_kernel_stats_pmc.md"),
 }
+
+# what the default run reports next to its headline workload: (workload, path)
+OTHERS = [("c2", "layer"), ("c3", "layer"), ("c5", "rows"), ("c2", "rows"), ("c3", "rows")]
 
 
 def build_layer_workload(key, torch, hip, act, dev):
@@ -278,6 +282,45 @@ def parity_on_sample(key, torch, m, x, out_cpu, grad_cpu, alphas):
             "grad_input_error_in_tolerances (rtol 1e-4, atol 1e-5)": float(err.max()) if same.any() else None}
 
 
+class Probes:
+    """ctypes face of libexodus_bench_probes.so: flat streaming kernels (copy / add, read only, write
+    only) that only this script uses, as bandwidth yardsticks next to the recurrence kernels."""
+
+    PATH = os.path.join(ROOT, "sinabs-exodus_amd", "libexodus_bench_probes.so")
+
+    def __init__(self, torch):
+        import ctypes
+        if not os.path.exists(self.PATH):
+            raise ImportError(f"{self.PATH} not found; build it with `python sinabs-exodus_amd/build_hip.py`")
+        self.torch, self.c = torch, ctypes
+        self.lib = ctypes.CDLL(self.PATH)
+        p, i64 = ctypes.c_void_p, ctypes.c_int64
+        for name, argtypes in (("exodus_probe_stream", [p, p, p, i64, p]), ("exodus_probe_read", [p, i64, p]),
+                               ("exodus_probe_write", [p, i64, p])):
+            fn = getattr(self.lib, name)
+            fn.argtypes, fn.restype = argtypes, ctypes.c_int
+
+    def _call(self, name, *args):
+        stream = self.c.c_void_p(self.torch.cuda.current_stream().cuda_stream)
+        rc = getattr(self.lib, name)(*args, stream)
+        if rc:
+            raise RuntimeError(f"{name} failed with hipError {rc}")
+
+    def _ptr(self, x):
+        assert x is None or (x.is_cuda and x.dtype == self.torch.float32 and x.is_contiguous())
+        return None if x is None else self.c.c_void_p(x.data_ptr())
+
+    def stream(self, dst, a, b=None):
+        assert dst.numel() == a.numel() and (b is None or b.numel() == a.numel())
+        self._call("exodus_probe_stream", self._ptr(dst), self._ptr(a), self._ptr(b), a.numel())
+
+    def read(self, a):
+        self._call("exodus_probe_read", self._ptr(a), a.numel())
+
+    def write(self, dst):
+        self._call("exodus_probe_write", self._ptr(dst), dst.numel())
+
+
 def measure_ceilings(args, torch, hip, dev):
     """GB/s of data-movement-only kernels on tensors of the chosen workload's shape."""
     w = WORKLOADS[args.workload]
@@ -300,13 +343,14 @@ def measure_ceilings(args, torch, hip, dev):
         return e0.elapsed_time(e1) / args.steps
 
     res = {"workload": w["name"], "tensor_GB": n * 4 / 1e9, "peak_GBs": HBM_PEAK_GBS}
-    ms = timed(lambda: hip.probeRead(a))
+    probes = Probes(torch)
+    ms = timed(lambda: probes.read(a))
     res["flat_read_only"] = {"ms": ms, "GBs": n * 4 / ms / 1e6}
-    ms = timed(lambda: hip.probeWrite(out))
+    ms = timed(lambda: probes.write(out))
     res["flat_write_only"] = {"ms": ms, "GBs": n * 4 / ms / 1e6}
-    ms = timed(lambda: hip.probeStream(out, a))
+    ms = timed(lambda: probes.stream(out, a))
     res["flat_copy_1r1w"] = {"ms": ms, "GBs": n * 8 / ms / 1e6}
-    ms = timed(lambda: hip.probeStream(out, a, b))
+    ms = timed(lambda: probes.stream(out, a, b))
     res["flat_add_2r1w"] = {"ms": ms, "GBs": n * 12 / ms / 1e6}
     ms = timed(lambda: hip.layerLeakyForward(a, zeros, alpha, False, False))
     res["time_strided_1r1w (leaky layer forward)"] = {"ms": ms, "GBs": n * 8 / ms / 1e6}
@@ -367,6 +411,47 @@ def measure_conv_snn(args, torch, dev):
     return res
 
 
+def measure(wl, steps, warmup, torch):
+    """`warmup` untimed and `steps` timed forward + backward passes of a built workload: wall time per
+    step and the mean duration of each direction from events on the launch stream."""
+    fwd, bwd = wl["fwd"], wl["bwd"]
+    for _ in range(warmup):
+        fwd(); bwd()
+    torch.cuda.synchronize()
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for k in range(steps):
+        ev[k][0].record()
+        fwd()
+        ev[k][1].record()
+        bwd()
+        ev[k][2].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    return {"steps": steps, "ms_per_step": wall * 1e3 / steps,
+            "fwd_ms": sum(e[0].elapsed_time(e[1]) for e in ev) / steps,
+            "bwd_ms": sum(e[1].elapsed_time(e[2]) for e in ev) / steps}
+
+
+def roofline(key, wl, fwd_ms, bwd_ms, bf, bb, traffic_known=True):
+    """HBM roofline of the slower of the two kernels: algorithmic bytes per launch / mean duration."""
+    n_t = wl["N"] * wl["T"]
+    dom = "bwd" if bwd_ms >= fwd_ms else "fwd"
+    dom_ms, dom_bytes, dom_name = (bwd_ms, bb, wl["bwd_name"]) if dom == "bwd" else (fwd_ms, bf, wl["fwd_name"])
+    other_ms, other_bytes, other_name = (fwd_ms, bf, wl["fwd_name"]) if dom == "bwd" else (bwd_ms, bb, wl["bwd_name"])
+    achieved = n_t * dom_bytes / (dom_ms * 1e-3) / 1e9
+    traffic, source = MEASURED_TRAFFIC.get((key, dom_name), (None, None)) if traffic_known else (None, None)
+    return {
+        "bound": "hbm", "kernel": dom_name, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+        "frac": achieved / HBM_PEAK_GBS, "traffic": traffic, "traffic_source": source,
+        "kernel_ms": dom_ms, "algorithmic_bytes_per_launch": n_t * dom_bytes,
+        "other_kernel": {"kernel": other_name, "kernel_ms": other_ms,
+                         "achieved": n_t * other_bytes / (other_ms * 1e-3) / 1e9},
+        "fwd_bwd_combined_frac": n_t * (bf + bb) / ((fwd_ms + bwd_ms) * 1e-3) / 1e9 / HBM_PEAK_GBS,
+    }
+
+
 def without_cycle_option(argv):
     """The command line without ``--after-hbm-cycle [N]`` (for the child process that measures)."""
     rest, skip = [], False
@@ -394,6 +479,9 @@ def main():
                          "e.g. a neuron count that does not fill 128-byte memory lines; such a run is a measurement "
                          "aid, not the benchmark (roofline.traffic is then null)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-others", dest="others", action="store_false",
+                    help="report only the chosen workload (the default run also times the other configurations "
+                         "and the (rows, time) kernels for a few steps each and lists them under \"others\")")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also launch one plain elementwise kernel (torch.neg) over exactly 1 GiB before the timed region, so that a "
                          "counter run (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE) has a kernel of known traffic "
@@ -461,30 +549,17 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    for _ in range(args.warmup):
-        fwd(); bwd()
-    torch.cuda.synchronize()
-
-    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for k in range(args.steps):
-        ev[k][0].record()
-        fwd()
-        ev[k][1].record()
-        bwd()
-        ev[k][2].record()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-
-    ms_step = wall * 1e3 / args.steps
-    fwd_ms = sum(e[0].elapsed_time(e[1]) for e in ev) / args.steps
-    bwd_ms = sum(e[1].elapsed_time(e[2]) for e in ev) / args.steps
+    m = measure(wl, args.steps, args.warmup, torch)
+    ms_step, fwd_ms, bwd_ms = m["ms_per_step"], m["fwd_ms"], m["bwd_ms"]
     bf, bb = wl.get("bytes", WORKLOADS[args.workload]["bytes"])
-    dom = "bwd" if bwd_ms >= fwd_ms else "fwd"
-    dom_ms, dom_bytes, dom_name = (bwd_ms, bb, wl["bwd_name"]) if dom == "bwd" else (fwd_ms, bf, wl["fwd_name"])
-    achieved = N * T * dom_bytes / (dom_ms * 1e-3) / 1e9
-    other_ms, other_bytes, other_name = (fwd_ms, bf, wl["fwd_name"]) if dom == "bwd" else (bwd_ms, bb, wl["bwd_name"])
+    roof = roofline(args.workload, wl, fwd_ms, bwd_ms, bf, bb, traffic_known=not args.shape)
+    # the same durations priced with the bytes of a kernel pair that stores and re-reads the states (the
+    # figure the workload description quotes); "frac" uses what this design has to move, which is less
+    # because the backward pass recomputes the states
+    roof["priced_at_stored_state_bytes"] = {
+        "bytes_per_neuron_timestep": sum(WORKLOADS[args.workload]["bytes"]),
+        "fwd_bwd_combined_frac": N * T * sum(WORKLOADS[args.workload]["bytes"])
+        / ((fwd_ms + bwd_ms) * 1e-3) / 1e9 / HBM_PEAK_GBS}
 
     result = {
         "metric": "neuron-timesteps/sec fwd+bwd (LIF, fp32) + % of HBM peak, 1 MI355X",
@@ -503,23 +578,27 @@ def main():
                    "algorithmic_bytes_per_neuron_timestep": bf + bb,
                    **({"after_hbm_cycles": int(os.environ["EXODUS_BENCH_AFTER_HBM_CYCLE"])}
                       if os.environ.get("EXODUS_BENCH_AFTER_HBM_CYCLE") else {})},
-        "roofline": {
-            "bound": "hbm", "kernel": dom_name, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": achieved / HBM_PEAK_GBS,
-            "traffic": None if args.shape else MEASURED_TRAFFIC.get((args.workload, dom_name)),
-            "kernel_ms": dom_ms, "algorithmic_bytes_per_launch": N * T * dom_bytes,
-            "other_kernel": {"kernel": other_name, "kernel_ms": other_ms,
-                             "achieved": N * T * other_bytes / (other_ms * 1e-3) / 1e9},
-            "fwd_bwd_combined_frac": N * T * (bf + bb) / ((fwd_ms + bwd_ms) * 1e-3) / 1e9 / HBM_PEAK_GBS,
-            # the same durations priced with the bytes of a kernel pair that stores and re-reads the
-            # states (the figure the workload description quotes); "frac" above uses what this
-            # design has to move, which is less because the backward pass recomputes the states
-            "priced_at_stored_state_bytes": {
-                "bytes_per_neuron_timestep": sum(WORKLOADS[args.workload]["bytes"]),
-                "fwd_bwd_combined_frac": N * T * sum(WORKLOADS[args.workload]["bytes"])
-                / ((fwd_ms + bwd_ms) * 1e-3) / 1e9 / HBM_PEAK_GBS},
-        },
+        "roofline": roof,
     }
+    if args.others and not args.shape:
+        # the other configurations and the (rows, time) kernels behind the autograd Functions, a few
+        # steps each: same measurement, reported beside the headline workload
+        del wl, fwd, bwd
+        result["others"] = []
+        for key, path in OTHERS:
+            if (key, path) == (args.workload, args.path):
+                continue
+            torch.cuda.empty_cache()
+            other = (build_layer_workload if path == "layer" else build_workload)(key, torch, hip, act, dev)
+            mo = measure(other, max(3, args.steps // 2), max(2, args.warmup // 2), torch)
+            obf, obb = other.get("bytes", WORKLOADS[key]["bytes"])
+            result["others"].append({
+                "workload": WORKLOADS[key]["name"], "path": path, "rows": other["N"], "time_steps": other["T"],
+                "steps": mo["steps"], "ms_per_step": mo["ms_per_step"],
+                "value": other["N"] * other["T"] / (mo["ms_per_step"] * 1e-3), "unit": "neuron-timesteps/s",
+                "algorithmic_bytes_per_neuron_timestep": obf + obb,
+                "roofline": roofline(key, other, mo["fwd_ms"], mo["bwd_ms"], obf, obb)})
+            del other
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(args.workload, torch)
     print(json.dumps(result))

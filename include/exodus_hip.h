@@ -29,7 +29,7 @@ extern "C" {
 #endif
 
 /* ABI version of this header; bumped on any signature change. */
-#define EXODUS_HIP_ABI_VERSION 3
+#define EXODUS_HIP_ABI_VERSION 4
 
 int exodus_hip_abi_version(void);
 const char *exodus_hip_error_string(int status);
@@ -252,18 +252,6 @@ int exodus_spike_forward(float *out_spikes, float *vmem, float alpha, float memb
 int exodus_spike_backward(float *input_grad, const float *surr, const float *output_grad,
                           const float *not_clipped, float alpha, float membr_subtract, int64_t n,
                           int64_t t, void *stream);
-
-/* ---- measurement aid, no counterpart in the reference ------------------------------------------
- * dst[i] = a[i] (b == NULL) or a[i] + b[i], n floats (multiple of 4, 16-byte aligned pointers),
- * with the same non-temporal 16-byte accesses the recurrence kernels use but consecutive addresses
- * per block: the bandwidth this machine gives a kernel that only moves data, and a kernel of
- * exactly known traffic to scale hardware counters by. */
-int exodus_probe_stream(float *dst, const float *a, const float *b, int64_t n, void *stream);
-
-/* The same accesses in one direction only: read n floats of `a` (nothing is written), or write n
- * zeros to `dst`.  What the memory gives reads alone and writes alone, next to the mixed figure. */
-int exodus_probe_read(const float *a, int64_t n, void *stream);
-int exodus_probe_write(float *dst, int64_t n, void *stream);
 
 #ifdef __cplusplus
 }

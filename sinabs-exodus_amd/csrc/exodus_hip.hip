@@ -682,6 +682,7 @@ int launch(const Op &op, int64_t n, int64_t t, void *stream)
     bool vec = (t % 4) == 0;
     for (int j = 0; j < Op::NIN; ++j) vec = vec && aligned16(op.in[j]);
     for (int j = 0; j < Op::NOUT; ++j) vec = vec && aligned16(op.out[j]);
+    if constexpr (Op::NDER > 0) vec = vec && aligned16(op.der);   // the derived output leaves through the same stores
     // Tiles are aligned to the first tensor's address (allocators hand out >= 256-byte aligned
     // blocks, so in practice every tensor shares this alignment).  Row shifts are
     // (base_shift + r*t) mod TT, i.e. base_shift plus multiples of g = gcd(t, TT); the largest one

@@ -249,8 +249,12 @@ __global__ void __launch_bounds__(BLOCK) layer_lif_forward(
     const int64_t m0 = static_cast<int64_t>(blockIdx.x - b * blocks_per_batch) * (BLOCK * NPL);
     const unsigned lane_off = threadIdx.x * NPL;
     const int64_t first = b * M + m0 + lane_off;              // first neuron (row) of this lane
+    // Lanes past the end of the layer (only the last block of a batch element has any) walk the same
+    // loops and meet every barrier, but touch no memory and compute nothing: all work sits behind
+    // `active`, all barriers in front of it.
+    const bool active = m0 + lane_off < M;
     double my_spikes = 0.0;
-    if (m0 + lane_off < M) {
+    {
         const int64_t n_ck = (T + CKPT - 1) / CKPT;
         const float *xp = x + (b * T) * M + m0;
         float *sp = spikes + (b * T) * M + m0;
@@ -265,12 +269,14 @@ __global__ void __launch_bounds__(BLOCK) layer_lif_forward(
         cc.cap = p.cap;
         cc.one = p.cap >= 1u ? 1.f : 0.f;
         cc.two = p.cap >= 2u ? 2.f : cc.one;
-        Neuron nr[NPL];
+        Neuron nr[NPL] = {};
+        if (active) {
 #pragma unroll
-        for (int e = 0; e < NPL; ++e) {
-            neuron_load<SYN, CAPK>(nr[e], p, first + e);
-            nr[e].vpost = p.v_init[first + e];
-            nr[e].i = SYN ? p.i_init[first + e] : 0.f;
+            for (int e = 0; e < NPL; ++e) {
+                neuron_load<SYN, CAPK>(nr[e], p, first + e);
+                nr[e].vpost = p.v_init[first + e];
+                nr[e].i = SYN ? p.i_init[first + e] : 0.f;
+            }
         }
 
         V bufa[FWD_UNROLL], bufb[FWD_UNROLL];
@@ -278,6 +284,7 @@ __global__ void __launch_bounds__(BLOCK) layer_lif_forward(
         // past the end), so every call issues exactly FWD_UNROLL loads
         auto fetch = [&](V(&dst)[FWD_UNROLL], int64_t t0) {
             __syncthreads();                                   // keeps the block's waves at the same step
+            if (!active) return;
             if (t0 + FWD_UNROLL <= T) {
                 const Rsrc r = make_rsrc(xp + t0 * M);
 #pragma unroll
@@ -292,6 +299,7 @@ __global__ void __launch_bounds__(BLOCK) layer_lif_forward(
         };
         float part = 0.f;                                     // spike count since the last checkpoint (exact in fp32)
         auto checkpoint = [&](int64_t j) {
+            if (!active) return;
             if (cvp) {
                 V cv, ci;
 #pragma unroll
@@ -312,6 +320,7 @@ __global__ void __launch_bounds__(BLOCK) layer_lif_forward(
         };
         auto compute = [&](const V(&buf)[FWD_UNROLL], int64_t t0, auto guard) {
             constexpr bool GUARD = decltype(guard)::value;
+            if (!active) return;
             const Rsrc rs = make_rsrc(sp + t0 * M);
             const Rsrc rv = make_rsrc(REC ? vrp + t0 * M : nullptr);
             const Rsrc ri = make_rsrc(REC ? irp + t0 * M : nullptr);
@@ -368,10 +377,12 @@ __global__ void __launch_bounds__(BLOCK) layer_lif_forward(
             }
         }
         my_spikes += static_cast<double>(part);
+        if (active) {
 #pragma unroll
-        for (int e = 0; e < NPL; ++e) {
-            v_last[first + e] = nr[e].vpost;
-            if (SYN && i_last) i_last[first + e] = nr[e].i;
+            for (int e = 0; e < NPL; ++e) {
+                v_last[first + e] = nr[e].vpost;
+                if (SYN && i_last) i_last[first + e] = nr[e].i;
+            }
         }
     }
     if (spike_sum) {
@@ -418,7 +429,9 @@ layer_lif_backward(
     const int64_t b = blockIdx.x / blocks_per_batch;
     const int64_t m0 = static_cast<int64_t>(blockIdx.x - b * blocks_per_batch) * BWD_BLOCK;
     const unsigned lane_off = threadIdx.x;
-    if (m0 + lane_off >= M) return;
+    // lanes past the end of the layer walk the same loops and meet every barrier, but all memory
+    // accesses and all arithmetic sit behind `active`
+    const bool active = m0 + lane_off < M;
     const int64_t row = b * M + m0 + lane_off;
     const int64_t n_ck = (T + CKPT - 1) / CKPT;
     // block-uniform bases; lane and step offsets are added by the buffer instructions
@@ -438,8 +451,8 @@ layer_lif_backward(
     cc.cap = p.cap;
     cc.one = p.cap >= 1u ? 1.f : 0.f;
     cc.two = p.cap >= 2u ? 2.f : cc.one;
-    Neuron nr;
-    neuron_load<SYN, CAPK>(nr, p, row);
+    Neuron nr = {};
+    if (active) neuron_load<SYN, CAPK>(nr, p, row);
     const float xg = (SYN && p.decay_early) ? nr.as : 1.0f;   // factor between mu and grad_x
     const bool pair_new = p.decay_early != 0;                  // the synapse sum pairs i_t with mu_t (else mu_{t+1})
     const SurrConst sk = surrogate_consts<KIND>(nr.th, p0, p1);
@@ -450,8 +463,8 @@ layer_lif_backward(
     // gradient enters v_{T-1} with the same factor 1 - c s_{T-1} as a_mem lambda_T would), and no step
     // needs a special case.
     float lam = 0.f, mu = 0.f;
-    float h = grad_v_last ? grad_v_last[row] : 0.f;
-    float hm = (SYN && grad_i_last) ? grad_i_last[row] : 0.f;
+    float h = (active && grad_v_last) ? grad_v_last[row] : 0.f;
+    float hm = (active && SYN && grad_i_last) ? grad_i_last[row] : 0.f;
     TileSum acc_m, acc_n, acc_s;                               // sums of lambda_{t+1} vpost_t, lambda_t i_t, mu i
     acc_m.clear();
     acc_n.clear();
@@ -466,6 +479,7 @@ layer_lif_backward(
         float xr[CKPT], gr[CKPT], vr[CKPT], sr[FROM_TENSOR ? CKPT : 1];
         float qv[EXTRA ? CKPT : 1], qi[(EXTRA && SYN) ? CKPT : 1];
         __syncthreads();                                   // keeps the block's waves at the same step
+        if (!active) return;
         {
             // always CKPT loads per tensor (steps past the end re-read the last step): a constant number
             // of loads in flight lets each use wait for its own load only
@@ -545,6 +559,7 @@ layer_lif_backward(
     }
     for (; j >= 0; --j) block(j, std::false_type{});
 
+    if (!active) return;                                       // no barrier follows
     if (v_init_grad) v_init_grad[row] = h;
     if (SYN && i_init_grad) i_init_grad[row] = hm;
     if (alpha_mem_grad) {
@@ -594,20 +609,25 @@ __global__ void __launch_bounds__(BLOCK) layer_leaky_forward(float *__restrict__
     const int64_t m0 = static_cast<int64_t>(blockIdx.x - b * blocks_per_batch) * (BLOCK * NPL);
     const unsigned lane_off = threadIdx.x * NPL;
     double my_sum = 0.0;                                       // sum of this lane's outputs (for the layer's mean)
-    if (m0 + lane_off < M) {
+    // lanes past the end of the layer walk the same loops and meet every barrier, but all memory
+    // accesses and all arithmetic sit behind `active`
+    const bool active = m0 + lane_off < M;
+    {
     const int64_t first = b * M + m0 + lane_off;
     const float *xp = x + (b * T) * M + m0;
     float *op = out + (b * T) * M + m0;
     const unsigned voff = lane_off * 4u;
     const unsigned step_bytes = static_cast<unsigned>(M) * 4u;
-    float a[NPL], kn[NPL], kd[NPL], v[NPL];
+    float a[NPL] = {}, kn[NPL] = {}, kd[NPL] = {}, v[NPL] = {};
     float part = 0.f;                                          // outputs of one stage, then folded into my_sum
+    if (active) {
 #pragma unroll
-    for (int e = 0; e < NPL; ++e) {
-        a[e] = p.alpha[first + e];
-        kn[e] = p.norm_input ? __fsub_rn(1.0f, a[e]) : 1.0f;
-        kd[e] = p.decay_early ? a[e] : 1.0f;
-        v[e] = p.v_init[first + e];
+        for (int e = 0; e < NPL; ++e) {
+            a[e] = p.alpha[first + e];
+            kn[e] = p.norm_input ? __fsub_rn(1.0f, a[e]) : 1.0f;
+            kd[e] = p.decay_early ? a[e] : 1.0f;
+            v[e] = p.v_init[first + e];
+        }
     }
     auto advance = [&](const V &xv) {
         V o;
@@ -623,11 +643,13 @@ __global__ void __launch_bounds__(BLOCK) layer_leaky_forward(float *__restrict__
     // `spread` = step_bytes, or 0 for a fetch whose data will not be used (same count of loads, one step)
     auto fetch = [&](V(&dst)[U], int64_t t0, unsigned spread) {
         __syncthreads();                                   // keeps the block's waves at the same step
+        if (!active) return;
         const Rsrc r = make_rsrc(xp + t0 * M);
 #pragma unroll
         for (int u = 0; u < U; ++u) dst[u] = IO::load(r, voff, u * spread);
     };
     auto compute = [&](const V(&buf)[U], int64_t t0) {
+        if (!active) return;
         const Rsrc r = make_rsrc(op + t0 * M);
 #pragma unroll
         for (int u = 0; u < U; ++u) IO::store(advance(buf[u]), r, voff, u * step_bytes);
@@ -645,13 +667,15 @@ __global__ void __launch_bounds__(BLOCK) layer_leaky_forward(float *__restrict__
         fetch(bufa, more ? t0 + 2 * U : t0, more ? step_bytes : 0u);
         compute(bufb, t0 + U);
     }
-    for (int64_t t = pairs * 2 * U; t < T; ++t) {
-        const V xv = IO::load(make_rsrc(xp + t * M), voff, 0u);
-        IO::store(advance(xv), make_rsrc(op + t * M), voff, 0u);
-    }
-    my_sum += static_cast<double>(part);
+    if (active) {
+        for (int64_t t = pairs * 2 * U; t < T; ++t) {
+            const V xv = IO::load(make_rsrc(xp + t * M), voff, 0u);
+            IO::store(advance(xv), make_rsrc(op + t * M), voff, 0u);
+        }
+        my_sum += static_cast<double>(part);
 #pragma unroll
-    for (int e = 0; e < NPL; ++e) v_last[first + e] = v[e];
+        for (int e = 0; e < NPL; ++e) v_last[first + e] = v[e];
+    }
     }
     if (out_sum) {
         // wave reduction, then one atomic per wave
@@ -677,7 +701,9 @@ __global__ void __launch_bounds__(BLOCK) layer_leaky_backward(
     const int64_t b = blockIdx.x / blocks_per_batch;
     const int64_t m0 = static_cast<int64_t>(blockIdx.x - b * blocks_per_batch) * (BLOCK * NPL);
     const unsigned lane_off = threadIdx.x * NPL;
-    if (m0 + lane_off >= M) return;
+    // lanes past the end of the layer walk the same loops and meet every barrier, but all memory
+    // accesses and all arithmetic sit behind `active`
+    const bool active = m0 + lane_off < M;
     const int64_t first = b * M + m0 + lane_off;
     const float *gp = grad_out + (b * T) * M + m0;
     const float *outp = ALPHA ? out + (b * T) * M + m0 : nullptr;
@@ -685,15 +711,17 @@ __global__ void __launch_bounds__(BLOCK) layer_leaky_backward(
     float *op = grad_x + (b * T) * M + m0;
     const unsigned voff = lane_off * 4u;
     const unsigned step_bytes = static_cast<unsigned>(M) * 4u;
-    float a[NPL], k[NPL], h[NPL], g[NPL];
+    float a[NPL] = {}, k[NPL] = {}, h[NPL] = {}, g[NPL] = {};
     TileSum acc[NPL];
 #pragma unroll
-    for (int e = 0; e < NPL; ++e) {
-        a[e] = p.alpha[first + e];
-        k[e] = __fsub_rn(1.0f, a[e]);
-        h[e] = grad_v_last ? grad_v_last[first + e] : 0.f;     // what reaches step t from later steps: alpha g_{t+1}
-        g[e] = 0.f;
-        acc[e].clear();
+    for (int e = 0; e < NPL; ++e) acc[e].clear();
+    if (active) {
+#pragma unroll
+        for (int e = 0; e < NPL; ++e) {
+            a[e] = p.alpha[first + e];
+            k[e] = __fsub_rn(1.0f, a[e]);
+            h[e] = grad_v_last ? grad_v_last[first + e] : 0.f; // what reaches step t from later steps: alpha g_{t+1}
+        }
     }
     // one step; `ov` = out_{t-1} (ignored at t = 0, where the initial state takes its place)
     auto advance = [&](int64_t t, const V &gv, const V &ov, const V &xv) {
@@ -723,6 +751,7 @@ __global__ void __launch_bounds__(BLOCK) layer_leaky_backward(
     // steps t0 .. t0 + U - 1; `spread` = step_bytes, or 0 for a fetch whose data will not be used
     auto fetch = [&](Stage &s, int64_t t0, unsigned spread) {
         __syncthreads();                                   // keeps the block's waves at the same step
+        if (!active) return;
         const Rsrc rg = make_rsrc(gp + t0 * M);
 #pragma unroll
         for (int u = 0; u < U; ++u) s.g[u] = IO::load(rg, voff, u * spread);
@@ -740,6 +769,7 @@ __global__ void __launch_bounds__(BLOCK) layer_leaky_backward(
         }
     };
     auto compute = [&](const Stage &s, int64_t t0) {          // newest step first
+        if (!active) return;
         const Rsrc r = make_rsrc(op + t0 * M);
 #pragma unroll
         for (int uu = 0; uu < U; ++uu) {
@@ -749,7 +779,7 @@ __global__ void __launch_bounds__(BLOCK) layer_leaky_backward(
     };
     const int64_t pairs = T / (2 * U);
     // the steps that do not fill a pair are the newest ones: one at a time
-    for (int64_t t = T - 1; t >= pairs * 2 * U; --t) {
+    for (int64_t t = T - 1; active && t >= pairs * 2 * U; --t) {
         const V gv = IO::load(make_rsrc(gp + t * M), voff, 0u);
         V ov = gv, xv = gv;
         if (ALPHA && t >= 1) ov = IO::load(make_rsrc(outp + (t - 1) * M), voff, 0u);
@@ -773,6 +803,7 @@ __global__ void __launch_bounds__(BLOCK) layer_leaky_backward(
             for (int e = 0; e < NPL; ++e) acc[e].fold();
         }
     }
+    if (!active) return;                                       // no barrier follows
 #pragma unroll
     for (int e = 0; e < NPL; ++e) {
         if (v_init_grad) v_init_grad[first + e] = h[e];
@@ -906,55 +937,6 @@ int dispatch_fwd(const FwdArgs &a, int npl)
 
 // step offsets inside a block of CKPT steps are 32-bit byte offsets
 inline bool too_wide(int64_t neurons) { return neurons >= (int64_t{1} << 25); }
-
-// ---------------------------------------------------------------------------------------------
-// streaming probes: what the memory system gives a kernel that does nothing but move floats,
-// flat (consecutive addresses per block).  Used to calibrate counters and to put the recurrence
-// kernels' bandwidth next to a ceiling measured on the same machine.
-// ---------------------------------------------------------------------------------------------
-constexpr int PROBE_PER_THREAD = 4;                            // 16-byte chunks per thread
-
-template <bool TWO_INPUTS>
-__global__ void __launch_bounds__(256) probe_stream(f32x4 *__restrict__ dst, const f32x4 *__restrict__ a,
-                                                    const f32x4 *__restrict__ b, const int64_t n_chunks)
-{
-    const int64_t base = (static_cast<int64_t>(blockIdx.x) * PROBE_PER_THREAD) * 256 + threadIdx.x;
-    f32x4 va[PROBE_PER_THREAD], vb[PROBE_PER_THREAD];
-#pragma unroll
-    for (int k = 0; k < PROBE_PER_THREAD; ++k) {
-        const int64_t i = base + k * 256;
-        if (i < n_chunks) {
-            va[k] = ld_stream(a + i);
-            if (TWO_INPUTS) vb[k] = ld_stream(b + i);
-        }
-    }
-#pragma unroll
-    for (int k = 0; k < PROBE_PER_THREAD; ++k) {
-        const int64_t i = base + k * 256;
-        if (i < n_chunks) st_stream(TWO_INPUTS ? va[k] + vb[k] : va[k], dst + i);
-    }
-}
-
-// one direction only: READ loads and hands every value to an empty asm statement (so the loads stay
-// although nothing is done with them), !READ writes zeros
-template <bool READ>
-__global__ void __launch_bounds__(256) probe_one_way(f32x4 *__restrict__ dst, const f32x4 *__restrict__ a,
-                                                     const int64_t n_chunks)
-{
-    const int64_t base = (static_cast<int64_t>(blockIdx.x) * PROBE_PER_THREAD) * 256 + threadIdx.x;
-#pragma unroll
-    for (int k = 0; k < PROBE_PER_THREAD; ++k) {
-        const int64_t i = base + k * 256;
-        if (i < n_chunks) {
-            if (READ) {
-                const f32x4 v = ld_stream(a + i);
-                asm volatile("" : : "v"(v));
-            } else {
-                st_stream(f32x4{0.f, 0.f, 0.f, 0.f}, dst + i);
-            }
-        }
-    }
-}
 
 }  // namespace
 
@@ -1129,53 +1111,6 @@ EXODUS_API int exodus_layer_leaky_backward(float *grad_input, float *alpha_grad,
     }
 #undef EXODUS_LK
 #undef EXODUS_LK1
-    return static_cast<int>(hipGetLastError());
-}
-
-EXODUS_API int exodus_probe_stream(float *dst, const float *a, const float *b, int64_t n, void *stream)
-{
-    if (n < 0 || (n % 4) != 0 || !dst || !a) return hipErrorInvalidValue;
-    for (const void *q : {static_cast<const void *>(dst), static_cast<const void *>(a), static_cast<const void *>(b)})
-        if (reinterpret_cast<uintptr_t>(q) & 15u) return hipErrorInvalidValue;
-    if (n == 0) return hipSuccess;
-    const int64_t n_chunks = n / 4;
-    const int64_t blocks = (n_chunks + 256 * PROBE_PER_THREAD - 1) / (256 * PROBE_PER_THREAD);
-    if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    if (b)
-        hipLaunchKernelGGL((probe_stream<true>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s,
-                           reinterpret_cast<f32x4 *>(dst), reinterpret_cast<const f32x4 *>(a),
-                           reinterpret_cast<const f32x4 *>(b), n_chunks);
-    else
-        hipLaunchKernelGGL((probe_stream<false>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s,
-                           reinterpret_cast<f32x4 *>(dst), reinterpret_cast<const f32x4 *>(a),
-                           static_cast<const f32x4 *>(nullptr), n_chunks);
-    return static_cast<int>(hipGetLastError());
-}
-
-EXODUS_API int exodus_probe_read(const float *a, int64_t n, void *stream)
-{
-    if (n < 0 || (n % 4) != 0 || !a || (reinterpret_cast<uintptr_t>(a) & 15u)) return hipErrorInvalidValue;
-    if (n == 0) return hipSuccess;
-    const int64_t n_chunks = n / 4;
-    const int64_t blocks = (n_chunks + 256 * PROBE_PER_THREAD - 1) / (256 * PROBE_PER_THREAD);
-    if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
-    hipLaunchKernelGGL((probe_one_way<true>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0,
-                       static_cast<hipStream_t>(stream), static_cast<f32x4 *>(nullptr),
-                       reinterpret_cast<const f32x4 *>(a), n_chunks);
-    return static_cast<int>(hipGetLastError());
-}
-
-EXODUS_API int exodus_probe_write(float *dst, int64_t n, void *stream)
-{
-    if (n < 0 || (n % 4) != 0 || !dst || (reinterpret_cast<uintptr_t>(dst) & 15u)) return hipErrorInvalidValue;
-    if (n == 0) return hipSuccess;
-    const int64_t n_chunks = n / 4;
-    const int64_t blocks = (n_chunks + 256 * PROBE_PER_THREAD - 1) / (256 * PROBE_PER_THREAD);
-    if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
-    hipLaunchKernelGGL((probe_one_way<false>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0,
-                       static_cast<hipStream_t>(stream), reinterpret_cast<f32x4 *>(dst),
-                       static_cast<const f32x4 *>(nullptr), n_chunks);
     return static_cast<int>(hipGetLastError());
 }
 

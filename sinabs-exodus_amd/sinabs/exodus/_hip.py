@@ -21,7 +21,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("EXODUS_HIP_LIBRARY") or os.path.join(_HERE, "libexodus_hip.so")
 
 SURR_TENSOR, SURR_SINGLE_EXP, SURR_PERIODIC_EXP, SURR_HEAVISIDE = 0, 1, 2, 3
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 _p = ctypes.c_void_p
 _i64 = ctypes.c_int64
@@ -43,9 +43,6 @@ _SIGNATURES = {
     "exodus_synlif_backward": ([_p] * 17 + [_int, _int, _int, _int, _int, _f, _f, _i64, _i64, _p], _int),
     "exodus_spike_forward": ([_p, _p, _f, _f, _f, _f, _int, _int, _i64, _i64, _p], _int),
     "exodus_spike_backward": ([_p] * 4 + [_f, _f, _i64, _i64, _p], _int),
-    "exodus_probe_stream": ([_p, _p, _p, _i64, _p], _int),
-    "exodus_probe_read": ([_p, _i64, _p], _int),
-    "exodus_probe_write": ([_p, _i64, _p], _int),
     "exodus_layer_checkpoint_interval": ([], _int),
     "exodus_layer_lif_forward": ([_p] * 16 + [_int, _int, _int, _int, _int, _i64, _i64, _i64, _p], _int),
     "exodus_layer_lif_backward": ([_p] * 18 + [_int, _int, _int, _int, _int, _f, _f, _p, _p, _p, _i64, _i64, _i64, _p], _int),
@@ -81,7 +78,7 @@ class ExodusHipError(RuntimeError):
 def _check(status: int, what: str) -> None:
     if status != 0:
         msg = lib.exodus_hip_error_string(status)
-        raise ExodusHipError(f"{what} failed: {msg.decode() if msg else status} (hipError {status})")
+        raise ExodusHipError(f"{what} failed: {msg.decode() if msg else status} (status {status})")
 
 
 def _dev(x: torch.Tensor, name: str, like: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -406,32 +403,6 @@ def synLifBackward(gradSpikes, gradVmem, gradIsyn, vmem, isyn, vmemPostInitial, 
 # layer-layout kernels: (batch, time, neurons) tensors, no transposition
 # ------------------------------------------------------------------------------------------
 
-def probeStream(dst, a, b=None) -> None:
-    """dst = a (b is None) or a + b with flat streaming accesses: a bandwidth yardstick."""
-    _dev(a, "a")
-    _dev(dst, "dst", a)
-    if b is not None:
-        _dev(b, "b", a)
-    if dst.numel() != a.numel() or (b is not None and b.numel() != a.numel()):
-        raise RuntimeError("dst, a and b must have the same number of elements")
-    with torch.cuda.device(a.device):
-        _check(lib.exodus_probe_stream(_ptr(dst), _ptr(a), _ptr(b), a.numel(), _stream(a)), "exodus_probe_stream")
-
-
-def probeRead(a) -> None:
-    """Read all of ``a`` with flat streaming accesses and write nothing."""
-    _dev(a, "a")
-    with torch.cuda.device(a.device):
-        _check(lib.exodus_probe_read(_ptr(a), a.numel(), _stream(a)), "exodus_probe_read")
-
-
-def probeWrite(dst) -> None:
-    """Fill ``dst`` with zeros with flat streaming accesses."""
-    _dev(dst, "dst")
-    with torch.cuda.device(dst.device):
-        _check(lib.exodus_probe_write(_ptr(dst), dst.numel(), _stream(dst)), "exodus_probe_write")
-
-
 # neurons per batch element the layer-layout entry points accept (they return invalid-value beyond)
 LAYER_MAX_NEURONS = 1 << 25
 
@@ -555,18 +526,29 @@ def layerLifBackward(gradSpikes, gradVLast, gradILast, input, ckptV, ckptI, vmem
         for nm, x in (("gradVRec", gradVRec), ("gradIRec", gradIRec)):
             if x is not None and _btm(x, nm, input).shape != input.shape:
                 raise RuntimeError(f"{nm} must have the shape of input")
-    # the kernel writes every neuron's entry of each vector it is given
-    z = lambda want: torch.empty(n, dtype=torch.float32, device=input.device) if want else None
+    # the kernel writes every neuron's entry of each vector it is given -- unless there is no step to
+    # walk: then nothing is launched, the decay factors have no influence and a gradient on a final
+    # state is the gradient of the initial state it equals
+    if t == 0:
+        z = lambda want: torch.zeros(n, dtype=torch.float32, device=input.device) if want else None
+    else:
+        z = lambda want: torch.empty(n, dtype=torch.float32, device=input.device) if want else None
     am_g, v0_g = z(wantAlphaMemGrad), z(wantVInitGrad)
     as_g, i0_g = z(syn and wantAlphaSynGrad), z(syn and wantIInitGrad)
-    with torch.cuda.device(input.device):
-        _check(lib.exodus_layer_lif_backward(
-            _ptr(gradInput), _ptr(am_g), _ptr(as_g), _ptr(v0_g), _ptr(i0_g), _ptr(gradSpikes), _ptr(gradVLast),
-            _ptr(gradILast) if syn else None, _ptr(input), _ptr(ckptV), _ptr(ckptI) if syn else None,
-            _ptr(vmemPostInitial), _ptr(isynInitial) if syn else None, _ptr(alphaMem), _ptr(alphaSyn) if syn else None,
+    if t == 0:
+        if v0_g is not None and gradVLast is not None:
+            v0_g.copy_(gradVLast.reshape(-1))
+        if i0_g is not None and gradILast is not None:
+            i0_g.copy_(gradILast.reshape(-1))
+    head = (_ptr(gradInput), _ptr(am_g), _ptr(as_g), _ptr(v0_g), _ptr(i0_g), _ptr(gradSpikes), _ptr(gradVLast),
+            _ptr(gradILast) if syn else None, _ptr(input))
+    tail = (_ptr(vmemPostInitial), _ptr(isynInitial) if syn else None, _ptr(alphaMem), _ptr(alphaSyn) if syn else None,
             _ptr(membrSubtract), _ptr(theta), _ptr(thetaLow), int(bool(applyThetaLow)), int(maxNumSpikes),
             int(bool(decayEarly)), int(bool(normInput)), int(surrogateKind), float(surrP0), float(surrP1), _ptr(surr),
-            _ptr(gradVRec), _ptr(gradIRec), b, t, m, _stream(input)), "exodus_layer_lif_backward")
+            _ptr(gradVRec), _ptr(gradIRec), b, t, m, _stream(input))
+    with torch.cuda.device(input.device):
+        _check(lib.exodus_layer_lif_backward(*head, _ptr(ckptV), _ptr(ckptI) if syn else None, *tail),
+               "exodus_layer_lif_backward")
     return gradInput, am_g, as_g, v0_g, i0_g
 
 

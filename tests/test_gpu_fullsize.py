@@ -233,3 +233,157 @@ def test_identical_batch_elements_give_identical_results_at_full_size(mods):
     gir, gar, ginit = hip.lifBackwardFused(gor, None, v, full(0.0), full(am), full(1.0), full(1.0), full(-1.0), True, 2,
                                            hip.SURR_SINGLE_EXP, 0.5, 1.0, needAlphaGrad=True)
     assert repeats(gir) and repeats(gar) and repeats(ginit)
+
+
+def test_c3_expleak_full_size(mods):
+    """ExpLeak with one trainable decay factor per channel, tau ~ U[5, 50], input ~ N(0, 1), at
+    (64, 1000, 4096) (the reference's counterpart at small size: tests/test_exp_leak.py:100-136).
+    The output and the input gradient of 768 sampled (batch, channel) rows and the batch-summed
+    per-channel alpha gradient of 48 whole channels against the oracle's restatement of the reference
+    kernels; both input options of the layer, weighted output gradients."""
+    hip, ref = mods
+    from _util import note_scaled, worst
+    need_gib(8)
+    B, T, M = 64, 1000, 4096
+    dev = "cuda"
+    g = torch.Generator(device=dev).manual_seed(2)
+    x = torch.randn(B, T, M, generator=g, device=dev)
+    go = torch.randn(B, T, M, generator=g, device=dev)
+    tau = 5.0 + 45.0 * torch.rand(M, generator=g, device=dev)
+    alpha_c = torch.exp(-1.0 / tau)                               # (M,)
+    alpha = alpha_c.expand(B, M).flatten().contiguous()
+    v0 = torch.randn(B * M, generator=g, device=dev) * 0.2
+    cg = gen(9)
+    ib = torch.randint(0, B, (768,), generator=cg); im = torch.randint(0, M, (768,), generator=cg)
+    chans = torch.randperm(M, generator=cg)[:48]
+    for decay_early, norm_input in ((False, False), (True, True)):
+        out, v_last = hip.layerLeakyForward(x, v0, alpha, decay_early, norm_input)
+        gi, ga, gv0 = hip.layerLeakyBackward(go, None, out, x, v0, alpha, decay_early, norm_input, True)
+
+        def oracle(xs, gos, a, v0s):
+            """rows through the oracle: scaled input -> leaky forward -> backward, chain rule for the scalings"""
+            k = (1.0 - a) if norm_input else torch.ones_like(a)
+            xin = k[:, None] * xs
+            if decay_early:
+                xin = xin * a[:, None]
+            o = ref.leaky_forward(xin.contiguous(), v0s, a)
+            g_in, g_a, g_v0 = ref.leaky_integrator_backward(gos.contiguous(), o, v0s, a, True)
+            gx = g_in * k[:, None] * (a[:, None] if decay_early else 1.0)
+            # d xin / d alpha = -x (norm) * (alpha if decay) + k x (decay)
+            dxin = torch.zeros_like(xs)
+            if norm_input:
+                dxin = dxin - xs * (a[:, None] if decay_early else 1.0)
+            if decay_early:
+                dxin = dxin + k[:, None] * xs
+            g_a = g_a + (g_in.double() * dxin.double()).sum(1).float()
+            # natural size of the alpha gradient's rounding error: it is a sum over time of products
+            # g_t * (out_{t-1} + d xin_t / d alpha) with both signs, whose terms are far from 1 here (outputs
+            # and adjoints of a slow integrator driven by N(0, 1) reach +-10), so the absolute tolerance
+            # scales with the root of the sum of squared terms (= sqrt(T) for terms of size 1)
+            prev = torch.cat([v0s[:, None], o[:, :-1]], 1)
+            spread = ((g_in.double() * (prev.double() + dxin.double())) ** 2).sum(1).sqrt().float()
+            return o, gx, g_a, g_v0, spread
+
+        # sampled rows
+        a_s = alpha_c.cpu()[im]; flat = ib * M + im
+        o, gx, g_a, g_v0, spread = oracle(sample_columns(x, ib.to(dev), im.to(dev)),
+                                          sample_columns(go, ib.to(dev), im.to(dev)), a_s, v0.cpu()[flat])
+        got_o = sample_columns(out, ib.to(dev), im.to(dev))
+        if not (decay_early or norm_input):
+            assert torch.equal(got_o, o)                              # same operations in the same order
+        assert_close(got_o, o, "output of sampled rows")
+        assert torch.equal(v_last.cpu()[flat], got_o[:, -1])
+        assert_close(sample_columns(gi, ib.to(dev), im.to(dev)), gx, "grad_x of sampled rows")
+        assert_close(gv0.cpu()[flat], g_v0, "grad v_init of sampled rows")
+        print(f"per-row alpha grad of sampled rows: {worst(ga.cpu()[flat], g_a)}")
+        note_scaled("C3 per-row alpha gradient (atol 1e-5 x root of the summed squared terms)", ga.cpu()[flat], g_a, 1e-4,
+                    float(1e-5 * spread.max()))
+        err = (ga.cpu()[flat].double() - g_a.double()).abs() / (1e-5 * spread.clamp(min=1.0) + 1e-4 * g_a.abs()).double()
+        assert float(err.max()) <= 1.0, f"grad alpha of sampled rows: {float(err.max()):.3g} x tolerance"
+        # whole channels: the per-channel gradient is the sum over the batch (what autograd's expand does)
+        xs = x[:, :, chans.to(dev)].permute(2, 0, 1).reshape(-1, T).cpu()      # (48 * B, T), channel-major
+        gos = go[:, :, chans.to(dev)].permute(2, 0, 1).reshape(-1, T).cpu()
+        a_rows = alpha_c.cpu()[chans].repeat_interleave(B)
+        v0_rows = v0.view(B, M)[:, chans.to(dev)].T.reshape(-1).cpu()
+        _, _, g_a, _, spread = oracle(xs, gos, a_rows, v0_rows)
+        want = g_a.double().view(48, B).sum(1)
+        spread = (spread.double().view(48, B) ** 2).sum(1).sqrt()
+        got = ga.view(B, M).double().sum(0).cpu()[chans]
+        print(f"per-channel alpha grad: {worst(got, want)}")
+        note_scaled("C3 per-channel alpha gradient (atol 1e-5 x root of the summed squared terms)", got, want, 1e-4,
+                    float(1e-5 * spread.max()))
+        err = (got - want).abs() / (1e-5 * spread.clamp(min=1.0) + 1e-4 * want.abs())
+        assert float(err.max()) <= 1.0, f"per-channel alpha gradient: {float(err.max()):.3g} x tolerance"
+
+
+def test_c1_iaf_full_shape():
+    """The smallest configuration exactly as described: IAF layer, input (8, 100, 256) ~ U[0, 0.5],
+    threshold 1, membrane subtract, SingleExponential surrogate, loss = sum of spikes -- the whole
+    tensor against the CPU step loop with autograd, and against the closed form floor(cumsum(x))."""
+    import sinabs.exodus.layers as el
+    from oracle import sinabs_layers as sl
+    x = torch.rand(8, 100, 256, generator=gen(0)) * 0.5
+    fast = el.IAF().cuda(); plain = sl.IAF()
+    xa = x.clone().requires_grad_(True); xb = x.clone().cuda().requires_grad_(True)
+    a = plain(xa); b = fast(xb)
+    assert torch.equal(b.cpu(), a) and a.sum() > 0
+    # integrate-and-fire identity for non-negative input: spikes up to t = floor(cumsum(x) / theta)
+    steps = torch.cumsum(x.double(), 1)
+    total = b.detach().cpu().double().cumsum(1)
+    assert float((total - steps.floor()).abs().max().item()) <= 1.0          # fp32 sums vs fp64: ties at most one step apart
+    assert torch.equal(b.cpu().sum(1), a.sum(1))
+    assert torch.equal(fast.v_mem.cpu(), plain.v_mem)
+    a.sum().backward(); b.sum().backward()
+    assert bool((xa.grad != 0).any())
+    assert_close(xb.grad, xa.grad, "grad input")
+
+
+def test_c4_conv_snn_full_shape():
+    """The convolutional configuration at its full shape (batch 64, 300 steps, 2 x 34 x 34 Bernoulli(0.02)
+    input, cross-entropy on spike counts): this package's layers against plain step-loop layers with
+    autograd, both on the GPU with identical weights -- spikes of all three neuron layers bit for bit,
+    loss and weight gradients within tolerance."""
+    import torch.nn as nn
+    import sinabs.exodus.layers as el
+    from oracle import sinabs_layers as sl
+    need_gib(120)
+    batch, steps = 64, 300
+
+    def net(mod):
+        return nn.Sequential(
+            nn.Conv2d(2, 32, 3), mod.IAFSqueeze(batch_size=batch), nn.AvgPool2d(2),
+            nn.Conv2d(32, 64, 3), mod.IAFSqueeze(batch_size=batch), nn.Flatten(),
+            nn.Linear(64 * 14 * 14, 10), mod.IAFSqueeze(batch_size=batch))
+
+    torch.manual_seed(4)
+    fast = net(el).cuda(); plain = net(sl).cuda()
+    for i in (0, 3, 6):
+        with torch.no_grad():
+            fast[i].weight.mul_(3.0)
+        plain[i].load_state_dict(fast[i].state_dict())
+    x = (torch.rand(batch, steps, 2, 34, 34, generator=gen(30)) < 0.02).float().cuda()
+    labels = torch.randint(0, 10, (batch,), generator=gen(31)).cuda()
+    taps = {}
+
+    def run(model, name):
+        hooks = [model[i].register_forward_hook(lambda m, a, o, i=i: taps.__setitem__((name, i), o.detach()))
+                 for i in (1, 4, 7)]
+        out = model(x.flatten(0, 1)).reshape(batch, steps, 10)
+        loss = nn.functional.cross_entropy(out.sum(1), labels)
+        loss.backward()
+        for h in hooks:
+            h.remove()
+        return out, loss
+
+    out_f, loss_f = run(fast, "fast")
+    out_p, loss_p = run(plain, "plain")
+    for i in (1, 4, 7):
+        assert taps[("plain", i)].sum() > 0 and torch.equal(taps[("fast", i)], taps[("plain", i)]), f"spikes of layer {i}"
+    assert torch.equal(fast[1].v_mem, plain[1].v_mem) and torch.equal(fast[4].v_mem, plain[4].v_mem)
+    assert_close(loss_f, loss_p, "loss", rtol=1e-6, atol=1e-7)
+    from _util import worst
+    for (k, p), (_, q) in zip(plain.named_parameters(), fast.named_parameters()):
+        if p.grad is not None:
+            print(f"grad {k}: {worst(q.grad, p.grad)}")
+            # sums over 64 x 300 x positions of products: judged relative to the gradient's own scale
+            assert_close(q.grad, p.grad, f"grad {k}", rtol=1e-4, atol=1e-5 * max(1.0, float(p.grad.abs().max())))

@@ -134,16 +134,23 @@ def evolve_steploop(sc, data, alpha, v_mem_init, threshold, min_v_mem, surrogate
 SURR = ["periodic", "single", "heaviside", "custom"]
 
 
-@pytest.mark.parametrize("surr_name", SURR)
-@pytest.mark.parametrize(argnames + ",backward_var",
-                         list(product(v_mem_initials, alphas, thresholds, min_v_mems[:-1], membrane_subtracts,
-                                      ("spikes", "vmem", "sum"))))
+def _integratefire_cases():
+    """The reference's grid (tests/test_spike_functions.py) in full for the surrogate its test uses; for the
+    other surrogates every configuration with a loss on spikes and potential together, and every fifth
+    configuration with a loss on the spikes alone and on the potential alone."""
+    grid = list(product(v_mem_initials, alphas, thresholds, min_v_mems[:-1], membrane_subtracts))
+    cases = [("periodic", *cfg, var) for cfg in grid for var in ("spikes", "vmem", "sum")]
+    for name in SURR[1:]:
+        cases += [(name, *cfg, "sum") for cfg in grid]
+        cases += [(name, *cfg, var) for cfg in grid[SURR.index(name)::5] for var in ("spikes", "vmem")]
+    return cases
+
+
+@pytest.mark.parametrize("surr_name," + argnames + ",backward_var", _integratefire_cases())
 def test_compare_integratefire(fns, oracle, surr_name, v_mem_initial, alpha, threshold, min_v_mem, membrane_subtract,
                                backward_var):
     IntegrateAndFire, _ = fns
     ref, sc = oracle
-    if surr_name != "periodic" and backward_var != "sum":
-        pytest.skip("full grid only for the surrogate the reference test uses")
     fn = {"periodic": ref.PeriodicExponential(), "single": ref.SingleExponential(), "heaviside": ref.Heaviside(0.6),
           "custom": CustomSurrogate()}[surr_name]
     if surr_name != "custom":

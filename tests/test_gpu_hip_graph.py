@@ -4,6 +4,8 @@ given, so the recording holds the hand-written kernels themselves and a replay s
 
 Each replay is compared with the same step run eagerly; between replays the program does ordinary eager
 work and waits for the device, so that a node that only works on the first replay is caught."""
+import warnings
+
 import pytest
 import torch
 import torch.nn as nn
@@ -52,21 +54,34 @@ def test_replays_equal_eager_steps(el, tau_syn):
     weight = torch.rand(batch, steps, 10, generator=gen(39)).cuda()
     x_static = inputs[0].clone()
 
-    # the usual recipe: a few eager passes on a side stream, gradients released, then the capture
+    # The usual recipe: a few eager passes on a side stream, gradients released, then the capture -- on the
+    # same stream.  Two things keep autograd's per-parameter gradient accumulators from being bound to another
+    # stream than the one that is captured (PyTorch warns about such a mismatch, and with the default stream on
+    # the other side it makes the engine wait on a stream outside the capture, which ends the capture with an
+    # error): (1) the capture runs on the warm-up's stream; (2) the layers' states, which carry the autograd
+    # graph of the last warm-up pass and with it every accumulator that pass created, are detached first
+    # (``layer.zero_grad()`` does that), so the capture creates its own.
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):
         for _ in range(3):
             step(recorded, x_static, weight)
             recorded.zero_grad(set_to_none=True)
+        for m in recorded:
+            if hasattr(m, "reset_states"):
+                m.zero_grad()                                  # detaches v_mem / i_syn from the warm-up's graph
     torch.cuda.current_stream().wait_stream(side)
 
     # the recording zeroes and reads the state tensors that exist now; the layers replace them by new ones
     # during the pass, so the program has to keep these alive for as long as it replays the graph
     held = [buf for buf in recorded.buffers()]
     graph = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(graph):
-        out_static = step(recorded, x_static, weight)
+    with warnings.catch_warnings(record=True) as caught:
+        warnings.simplefilter("always")
+        with torch.cuda.graph(graph, stream=side):
+            out_static = step(recorded, x_static, weight)
+    stream_warnings = [str(w.message) for w in caught if "AccumulateGrad" in str(w.message)]
+    assert not stream_warnings, stream_warnings
     grads_static = {k: p.grad for k, p in recorded.named_parameters() if p.grad is not None}
     assert {"0.weight", "1.alpha_mem", "2.weight"} <= set(grads_static)
 

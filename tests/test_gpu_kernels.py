@@ -219,12 +219,19 @@ def test_argument_errors(hip):
 
 
 def test_one_way_streaming_probes():
-    """The measurement probes: the write probe zeroes exactly its range, the read probe writes nothing."""
-    from sinabs.exodus import _hip
+    """bench.py's measurement probes (a library of their own, not part of libexodus_hip.so): the copy
+    copies, the write probe zeroes exactly its range, the read probe writes nothing."""
+    import bench
+    probes = bench.Probes(torch)
     n = 4 * 1000 + 4
     buf = torch.full((n + 8,), 3.0, device="cuda")
-    _hip.probeWrite(buf[4:4 + n])
+    probes.write(buf[4:4 + n])
     assert bool((buf[4:4 + n] == 0).all()) and bool((buf[:4] == 3).all()) and bool((buf[4 + n:] == 3).all())
     a = torch.randn(n, device="cuda"); keep = a.clone()
-    _hip.probeRead(a)
+    probes.read(a)
     assert torch.equal(a, keep)
+    b = torch.randn(n, device="cuda"); dst = torch.empty(n, device="cuda")
+    probes.stream(dst, a)
+    assert torch.equal(dst, a)
+    probes.stream(dst, a, b)
+    assert torch.equal(dst, a + b)

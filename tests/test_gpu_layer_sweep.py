@@ -12,7 +12,7 @@ import random
 import pytest
 import torch
 
-from _util import gen
+from _util import gen, note_scaled
 
 pytestmark = pytest.mark.gpu
 
@@ -77,12 +77,14 @@ def test_random_layers_native_equals_rows_path():
                 la = la + native.v_mem.sum() * 0.3; lc = lc + rows.v_mem.sum() * 0.3
             la.backward(retain_graph=True); lc.backward(retain_graph=True)
         e = excess(xa.grad, xb.grad)
+        note_scaled("layer sweep: grad input", xa.grad, xb.grad, 1e-4, 1e-5, e)
         assert e <= 1, f"{what}: grad input {e:.3g} x tolerance"
         worst = max(worst, e)
         for (k, p), (_, q) in zip(native.named_parameters(), rows.named_parameters()):
             assert (p.grad is None) == (q.grad is None), f"{what}: grad {k}"
             if q.grad is not None:
                 e = excess(p.grad, q.grad, atol=1e-5 * max(1.0, (b * t) ** 0.5))
+                note_scaled(f"layer sweep: grad {k}", p.grad, q.grad, 1e-4, 1e-5 * max(1.0, (b * t) ** 0.5), e)
                 assert e <= 1, f"{what}: grad {k} {e:.3g} x tolerance"
                 worst = max(worst, e)
         assert excess(native.v_mem, rows.v_mem, 1e-5, 1e-6, 0.0) <= 1, what

@@ -174,6 +174,47 @@ def test_native_membrane_against_cpu_oracle_all_caps(L, cap, b, t, m, theta_sign
     assert_close(got[1].cpu(), ga, "grad alpha", rtol=2e-4, atol=2e-5 * max(1.0, ga.abs().max().item()))
 
 
+@pytest.mark.parametrize("cap", [1, 2, -1])
+@pytest.mark.parametrize("b,t,m", [(2, 31, 6), (3, 32, 10), (2, 33, 7), (2, 97, 67), (1, 64, 260), (3, 97, 1030)])
+@pytest.mark.parametrize("decay_early,norm_input", list(product((True, False), (True, False))))
+def test_native_synaptic_against_cpu_oracle(L, cap, b, t, m, decay_early, norm_input):
+    """The synaptic layer kernels (the benchmark's kernels) directly against the CPU oracle, composed the
+    way the reference layer composes its Functions: both input options, the three spike-count
+    specialisations, sequences that end inside / at / just after a checkpoint block, ragged widths,
+    random per-neuron parameters and initial states, gradients arriving at spikes and at both final
+    states.  Forward bit for bit; gradients of input, both decay factors and both initial states within
+    rtol 1e-4 / atol 1e-5 (sums over time: atol scaled by sqrt(t), worst error printed in plain units)."""
+    _, _, hip = L
+    from oracle import exodus_ref as ref
+    from oracle import sinabs_cpu as sc
+    from _util import synaptic_layer_oracle, worst
+    n = b * m
+    g = gen(7000 + cap * 100 + t * 10 + m + 2 * decay_early + norm_input)
+    scale = (6.0 if norm_input else 0.7) * 0.5
+    x = torch.randn(b, t, m, generator=g) * scale + 0.3 * scale
+    am = 0.5 + 0.5 * torch.rand(n, generator=g); asn = 0.3 + 0.6 * torch.rand(n, generator=g)
+    v0 = torch.randn(n, generator=g) * 0.3; i0 = torch.randn(n, generator=g) * 0.3
+    th = 0.5 + torch.rand(n, generator=g); c = th * (0.4 + 0.6 * torch.rand(n, generator=g))
+    lo = -0.2 - torch.rand(n, generator=g)
+    go = torch.randn(b, t, m, generator=g); gvl = torch.randn(n, generator=g); gil = torch.randn(n, generator=g)
+    want = synaptic_layer_oracle(ref, sc.bt_to_rows(x), sc.bt_to_rows(go), am, asn, v0, i0, th, c, lo, cap, decay_early,
+                                 norm_input, ref.SingleExponential(), gvl, gil)
+    D = lambda z: z.cuda()
+    f = hip.layerLifForward(D(x), D(v0), D(i0), D(am), D(asn), D(c), D(th), D(lo), True, cap, decay_early, norm_input)
+    assert want["spikes"].sum() > 0
+    assert torch.equal(f["spikes"].cpu(), sc.rows_to_bt(want["spikes"], b))
+    assert torch.equal(f["v_last"].cpu(), want["v_last"]) and torch.equal(f["i_last"].cpu(), want["i_last"])
+    got = hip.layerLifBackward(D(go), D(gvl), D(gil), D(x), f["ckpt_v"], f["ckpt_i"], D(v0), D(i0), D(am), D(asn), D(c),
+                               D(th), D(lo), True, cap, decay_early, norm_input, hip.SURR_SINGLE_EXP, 0.5, 1.0)
+    gx, g_am, g_as, g_v0, g_i0 = (z.cpu() for z in got)
+    assert_close(sc.bt_to_rows(gx), want["g_x"], "grad input")
+    assert_close(g_v0, want["g_v_init"], "grad v_init")
+    assert_close(g_i0, want["g_i_init"], "grad i_init")
+    print(f"alpha_mem grad {worst(g_am, want['g_alpha_mem'])}; alpha_syn grad {worst(g_as, want['g_alpha_syn'])}")
+    assert_close(g_am, want["g_alpha_mem"], "grad alpha_mem", atol=1e-5 * t ** 0.5)
+    assert_close(g_as, want["g_alpha_syn"], "grad alpha_syn", atol=1e-5 * t ** 0.5)
+
+
 @pytest.mark.parametrize("kind", ["lif", "synaptic", "expleak"])
 def test_firing_rate_carries_gradient_like_the_reference(L, kind):
     """The reference computes ``firing_rate = output.sum() / output.numel()`` with autograd
@@ -313,6 +354,28 @@ def test_empty_sequences_and_batches(L):
         assert res["spikes"].shape == shape and res["v_last"].numel() == 0
     layer = el.IAF().cuda()
     assert layer(torch.empty(2, 0, 4).cuda()).shape == (2, 0, 4)
+    # backward over zero steps: a gradient on a final state is the gradient of the initial state,
+    # the decay factors get zero (nothing is launched, so nothing may be left uninitialised)
+    gv = torch.tensor([1.0, -2.0, 3.0]); gi = torch.tensor([0.5, 0.25, -1.0])
+    ck = torch.empty(1, 0, 3)
+    for _ in range(3):                                         # fresh allocations each time
+        torch.full((1 << 16,), float("nan")).cuda()            # dirty memory for the allocator to hand out again
+        got = hip.layerLifBackward(D(x), D(gv), D(gi), D(x), D(ck), D(ck), D(v0), D(i0), D(one * 0.9), D(one * 0.8),
+                                   D(one), D(one), None, False, -1, True, True, hip.SURR_SINGLE_EXP, 0.5, 1.0)
+        assert got[0].shape == (1, 0, 3)
+        assert torch.equal(got[1].cpu(), torch.zeros(3)) and torch.equal(got[2].cpu(), torch.zeros(3))
+        assert torch.equal(got[3].cpu(), gv) and torch.equal(got[4].cpu(), gi)
+    got = hip.layerLifBackward(D(x), None, None, D(x), D(ck), None, D(v0), None, D(one * 0.9), None, D(one), D(one),
+                               None, False, -1, True, True, hip.SURR_SINGLE_EXP, 0.5, 1.0)
+    assert torch.equal(got[3].cpu(), torch.zeros(3)) and got[2] is None and got[4] is None
+    # through the layer: a loss on the state after an empty sequence reaches the state before it
+    lif = el.LIF(tau_mem=10.0, tau_syn=5.0, train_alphas=True).cuda()
+    warm = (torch.rand(2, 5, 4, generator=gen(1)) * 3).cuda().requires_grad_(True)
+    lif(warm)                                                  # states now carry a graph
+    lif(torch.empty(2, 0, 4).cuda())
+    (lif.v_mem.sum() + 2.0 * lif.i_syn.sum()).backward()
+    assert warm.grad is not None and bool(torch.isfinite(warm.grad).all()) and bool((warm.grad != 0).any())
+    assert bool(torch.isfinite(lif.alpha_mem.grad).all()) and bool(torch.isfinite(lif.alpha_syn.grad).all())
 
 
 @pytest.mark.parametrize("mode", ["no_grad", "inference_mode", "non_contiguous", "half_input"])

@@ -8,7 +8,7 @@ import random
 import pytest
 import torch
 
-from _util import gen
+from _util import gen, note_scaled
 
 pytestmark = pytest.mark.gpu
 
@@ -62,6 +62,7 @@ def test_random_rows_against_the_c_oracle():
         for name, a, b, atol in zip(("grad input", "grad alpha", "grad init"), got, want,
                                     (1e-5, 1e-5 * max(1, t) ** 0.5, 1e-5)):
             e = excess(a, b, atol=atol)
+            note_scaled(f"rows sweep: {name}", a, b, 1e-4, atol, e)   # also in units of the plain rtol 1e-4 / atol 1e-5
             assert e <= 1, f"{what}: {name} {e:.3g} x tolerance"
             worst = max(worst, e)
         want_o = ref.leaky_forward(x, v0, alpha)
@@ -72,6 +73,7 @@ def test_random_rows_against_the_c_oracle():
         for name, a, b, atol in zip(("leaky grad input", "leaky grad alpha", "leaky grad init"), got, want,
                                     (1e-5, 1e-5 * max(1, t) ** 0.5, 1e-5)):
             e = excess(a, b, atol=atol)
+            note_scaled(f"rows sweep: {name}", a, b, 1e-4, atol, e)   # also in units of the plain rtol 1e-4 / atol 1e-5
             assert e <= 1, f"{what}: {name} {e:.3g} x tolerance"
             worst = max(worst, e)
     print(f"largest gradient difference: {worst:.3g} x tolerance")

@@ -98,5 +98,5 @@ def test_fused_against_cpu_step_loop(mods, capsys):
     if tie == 0:
         assert_close(v, sc.bt_to_rows(rec["v_mem"]), "v_mem", rtol=1e-4, atol=1e-5)
         assert_close(xd.grad, sc.bt_to_rows(xo.grad), "grad input", rtol=1e-4, atol=1e-5)
-        assert_close(asd.grad, aso.grad, "grad alpha_syn", rtol=2e-4, atol=1e-3)
-        assert_close(amd.grad, amo.grad, "grad alpha_mem", rtol=2e-4, atol=1e-3)
+        assert_close(asd.grad, aso.grad, "grad alpha_syn", rtol=1e-4, atol=1e-5)
+        assert_close(amd.grad, amo.grad, "grad alpha_mem", rtol=1e-4, atol=1e-5)
