@@ -12,7 +12,7 @@
  *   - Return value: 0 on success, otherwise a hipError_t value (1 = invalid value for a bad
  *     argument detected on the host before any launch).  exodus_hip_error_string() names it.
  *   - n == 0 or t == 0 is a successful no-op (per-row outputs are then left untouched).
- *   - Thread safe: no global state.
+ *   - Thread safe: no global state (one exception, stated there: exodus_layer_lif_backward_from_input).
  *
  * The first six entry points map one-to-one onto the six production functions the reference
  * exports from its CUDA extension (reference cuda/bindings.cu:362-373), so that the same unit
@@ -29,10 +29,13 @@ extern "C" {
 #endif
 
 /* ABI version of this header; bumped on any signature change. */
-#define EXODUS_HIP_ABI_VERSION 4
+#define EXODUS_HIP_ABI_VERSION 5
 
 int exodus_hip_abi_version(void);
 const char *exodus_hip_error_string(int status);
+
+/* Status values of this library's own (negative, so that they cannot collide with a hipError_t). */
+#define EXODUS_ERROR_SCRATCH_TOO_SMALL (-2)
 
 /* ---------------------------------------------------------------------------------------------
  * One-to-one counterparts of the reference bindings
@@ -211,6 +214,32 @@ int exodus_layer_lif_backward(float *grad_input, float *alpha_mem_grad, float *a
                               int surrogate_kind, float surr_p0, float surr_p1, const float *surr,
                               const float *grad_v_rec, const float *grad_i_rec, int64_t batch, int64_t t,
                               int64_t neurons, void *stream);
+
+/* exodus_layer_lif_backward for callers that cannot allocate device memory -- code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the
+ * reference.  Same arguments, outputs and arithmetic as exodus_layer_lif_backward, except that no
+ * checkpoints are passed: the checkpoints live in a fixed array of exodus_layer_scratch_floats()
+ * floats (2^24 = 64 MiB) inside the library's device image, and this call first runs the forward
+ * recurrence once more over `input` to fill them (so vmem_post_initial, and isyn_initial with synapse,
+ * are always required), then the backward pass.  A forward that was run without checkpoints
+ * (ckpt_v == NULL) therefore suffices.  The batch is walked in slices of as many batch elements as
+ * fit the array; if a single batch element does not fit -- ceil(t / interval) * neurons floats, twice
+ * that with synapse, more than the array holds -- nothing is launched and
+ * EXODUS_ERROR_SCRATCH_TOO_SMALL is returned.  The call allocates and frees nothing and does not
+ * synchronise.  Every GPU holds one such array for the life of the process and all calls on a GPU
+ * share it: calls on different streams of one GPU that may overlap race on it and must be ordered by
+ * the caller. */
+int64_t exodus_layer_scratch_floats(void);
+int exodus_layer_lif_backward_from_input(float *grad_input, float *alpha_mem_grad, float *alpha_syn_grad,
+                                         float *vmem_init_grad, float *isyn_init_grad, const float *grad_spikes,
+                                         const float *grad_v_last, const float *grad_i_last, const float *input,
+                                         const float *vmem_post_initial, const float *isyn_initial,
+                                         const float *alpha_mem, const float *alpha_syn, const float *membr_subtract,
+                                         const float *theta, const float *theta_low, int apply_theta_low,
+                                         int max_num_spikes, int decay_early, int norm_input, int surrogate_kind,
+                                         float surr_p0, float surr_p1, const float *surr, const float *grad_v_rec,
+                                         const float *grad_i_rec, int64_t batch, int64_t t, int64_t neurons,
+                                         void *stream);
 
 /* Forward of the non-spiking leaky-integrator layer (ExpLeak) on (batch,t,neurons): per neuron
  *   xin = norm_input ? (1 - alpha) * input : input;  xin = decay_early ? xin * alpha : xin;

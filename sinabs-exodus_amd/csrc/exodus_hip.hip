@@ -805,6 +805,10 @@ EXODUS_API int exodus_hip_abi_version(void) { return EXODUS_HIP_ABI_VERSION; }
 
 EXODUS_API const char *exodus_hip_error_string(int status)
 {
+    if (status == EXODUS_ERROR_SCRATCH_TOO_SMALL)
+        return "one batch element needs more checkpoint memory than the library's fixed scratch array holds "
+               "(see exodus_layer_scratch_floats); use exodus_layer_lif_forward / exodus_layer_lif_backward with "
+               "caller-allocated checkpoints";
     return hipGetErrorString(static_cast<hipError_t>(status));
 }
 

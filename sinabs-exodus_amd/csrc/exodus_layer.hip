@@ -18,6 +18,7 @@
 #include <stdint.h>
 
 #include <initializer_list>
+#include <mutex>
 #include <type_traits>
 
 #include "exodus_common.hpp"
@@ -233,7 +234,9 @@ __device__ __forceinline__ float spike_count_fast(float v, const Neuron &n, cons
 // the same number of loads (past the end it re-reads the last step), so the number of outstanding
 // loads at each wait is a compile-time constant.  A last, partial block runs through a guarded copy
 // of the same code.
-template <bool SYN, int NPL, int CAPK, bool REC, bool NT>
+// OUT = false keeps only the checkpoints: no spike raster, no final states, no spike total (what a
+// backward pass that was handed no checkpoints runs first).
+template <bool SYN, int NPL, int CAPK, bool REC, bool NT, bool OUT = true>
 __global__ void __launch_bounds__(BLOCK) layer_lif_forward(
     float *__restrict__ spikes, float *__restrict__ v_rec, float *__restrict__ i_rec, float *__restrict__ ckpt_v,
     float *__restrict__ ckpt_i, float *__restrict__ v_last, float *__restrict__ i_last, double *spike_sum,
@@ -349,7 +352,7 @@ __global__ void __launch_bounds__(BLOCK) layer_lif_forward(
                         lane_put<NPL>(vr, e, (REC && p.rec_pre) ? v[e] : nr[e].vpost);
                         lane_put<NPL>(ir, e, nr[e].i);
                     }
-                    IO::store(s, rs, voff, u * step_bytes);
+                    if (OUT) IO::store(s, rs, voff, u * step_bytes);
                     if (REC && vrp) IO::store(vr, rv, voff, u * step_bytes);
                     if (REC && irp) IO::store(ir, ri, voff, u * step_bytes);
                 }
@@ -377,7 +380,7 @@ __global__ void __launch_bounds__(BLOCK) layer_lif_forward(
             }
         }
         my_spikes += static_cast<double>(part);
-        if (active) {
+        if (active && OUT) {
 #pragma unroll
             for (int e = 0; e < NPL; ++e) {
                 v_last[first + e] = nr[e].vpost;
@@ -385,7 +388,7 @@ __global__ void __launch_bounds__(BLOCK) layer_lif_forward(
             }
         }
     }
-    if (spike_sum) {
+    if (OUT && spike_sum) {
         // wave reduction, then one atomic per wave
 #pragma unroll
         for (int off = WAVE / 2; off > 0; off >>= 1) my_spikes += __shfl_xor(my_spikes, off, WAVE);
@@ -935,8 +938,64 @@ int dispatch_fwd(const FwdArgs &a, int npl)
     return dispatch_fwd_cap<SYN, 1>(a);
 }
 
+// the forward pass again, keeping nothing but the checkpoints (one neuron per lane, general spike count:
+// the values do not depend on either choice)
+template <bool SYN>
+int launch_checkpoints_only(float *ckpt_v, float *ckpt_i, const float *x, const LayerConsts &p, int64_t B, int64_t T,
+                            int64_t M, hipStream_t s)
+{
+    const int64_t blocks_per_batch = (M + BLOCK - 1) / BLOCK;
+    if (blocks_per_batch > 0x7fffffffLL / B) return hipErrorInvalidValue;
+    const dim3 grid(static_cast<unsigned>(blocks_per_batch * B)), block(BLOCK);
+    float *const none = nullptr;
+    double *const no_sum = nullptr;
+    if (whole_lines(M, {x, ckpt_v, ckpt_i}))
+        hipLaunchKernelGGL((layer_lif_forward<SYN, 1, 0, false, true, false>), grid, block, 0, s, none, none, none, ckpt_v,
+                           ckpt_i, none, none, no_sum, x, p, blocks_per_batch, T, M);
+    else
+        hipLaunchKernelGGL((layer_lif_forward<SYN, 1, 0, false, false, false>), grid, block, 0, s, none, none, none,
+                           ckpt_v, ckpt_i, none, none, no_sum, x, p, blocks_per_batch, T, M);
+    return static_cast<int>(hipGetLastError());
+}
+
 // step offsets inside a block of CKPT steps are 32-bit byte offsets
 inline bool too_wide(int64_t neurons) { return neurons >= (int64_t{1} << 25); }
+
+}  // namespace
+
+// ---------------------------------------------------------------------------------------------
+// Checkpoint memory of exodus_layer_lif_backward_from_input, the one entry point that must not
+// allocate.  Every GPU the library runs on holds its own copy of this array, at its own address,
+// until the process ends.  In host code the array's name is only a handle for hipGetSymbolAddress:
+// kernels get the device address looked up below, never the name.
+// ---------------------------------------------------------------------------------------------
+constexpr int64_t SCRATCH_FLOATS = int64_t{1} << 24;           // 64 MiB
+static __device__ __align__(256) float scratch[SCRATCH_FLOATS];
+
+namespace {
+
+constexpr int MAX_DEVICES = 64;
+std::mutex scratch_lock;
+float *scratch_of_device[MAX_DEVICES] = {};
+
+// device address of `scratch` on the current device (looked up once per device)
+int scratch_address(float **out)
+{
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return static_cast<int>(e);
+    if (dev < 0 || dev >= MAX_DEVICES) return hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> hold(scratch_lock);
+    if (!scratch_of_device[dev]) {
+        void *ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return static_cast<int>(e);
+        if (!ptr) return hipErrorInvalidSymbol;
+        scratch_of_device[dev] = static_cast<float *>(ptr);
+    }
+    *out = scratch_of_device[dev];
+    return hipSuccess;
+}
 
 }  // namespace
 
@@ -1033,6 +1092,76 @@ EXODUS_API int exodus_layer_lif_backward(float *grad_input, float *alpha_mem_gra
         default: return hipErrorInvalidValue;
     }
 #undef EXODUS_BWD
+}
+
+EXODUS_API int64_t exodus_layer_scratch_floats(void) { return SCRATCH_FLOATS; }
+
+EXODUS_API int exodus_layer_lif_backward_from_input(
+    float *grad_input, float *alpha_mem_grad, float *alpha_syn_grad, float *vmem_init_grad, float *isyn_init_grad,
+    const float *grad_spikes, const float *grad_v_last, const float *grad_i_last, const float *input,
+    const float *vmem_post_initial, const float *isyn_initial, const float *alpha_mem, const float *alpha_syn,
+    const float *membr_subtract, const float *theta, const float *theta_low, int apply_theta_low, int max_num_spikes,
+    int decay_early, int norm_input, int surrogate_kind, float surr_p0, float surr_p1, const float *surr,
+    const float *grad_v_rec, const float *grad_i_rec, int64_t batch, int64_t t, int64_t neurons, void *stream)
+{
+    if (bad3(batch, t, neurons)) return hipErrorInvalidValue;
+    if (batch == 0 || t == 0 || neurons == 0) return hipSuccess;
+    if (too_wide(neurons)) return hipErrorInvalidValue;
+    const bool syn = alpha_syn != nullptr;
+    if (!grad_input || !grad_spikes || !input || !vmem_post_initial || !alpha_mem || !membr_subtract || !theta ||
+        (apply_theta_low && !theta_low) || (syn && !isyn_initial) ||
+        (surrogate_kind == EXODUS_SURR_TENSOR && !surr) || surrogate_kind < EXODUS_SURR_TENSOR ||
+        surrogate_kind > EXODUS_SURR_HEAVISIDE)
+        return hipErrorInvalidValue;
+    if (syn ? ((grad_v_rec != nullptr) != (grad_i_rec != nullptr)) : grad_i_rec != nullptr) return hipErrorInvalidValue;
+    // checkpoints of one batch element; the batch is walked in slices of as many elements as fit
+    const int64_t n_ck = (t + CKPT - 1) / CKPT;
+    if (n_ck > SCRATCH_FLOATS / neurons) return EXODUS_ERROR_SCRATCH_TOO_SMALL;
+    const int64_t per_element = ((n_ck * neurons + 63) / 64) * 64;          // each tensor starts on a 256-byte boundary
+    const int64_t fit = SCRATCH_FLOATS / (per_element * (syn ? 2 : 1));
+    if (fit < 1) return EXODUS_ERROR_SCRATCH_TOO_SMALL;
+    float *base = nullptr;
+    if (const int rc = scratch_address(&base)) return rc;
+    LayerConsts p;
+    p.v_init = vmem_post_initial;
+    p.i_init = isyn_initial;
+    p.alpha_mem = alpha_mem;
+    p.alpha_syn = alpha_syn;
+    p.c = membr_subtract;
+    p.theta = theta;
+    p.theta_low = theta_low;
+    p.apply_low = apply_theta_low ? 1 : 0;
+    p.decay_early = decay_early ? 1 : 0;
+    p.norm_input = norm_input ? 1 : 0;
+    p.cap = static_cast<unsigned>(max_num_spikes);
+    p.rec_pre = 0;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    auto at = [](auto *q, int64_t offset) { return q ? q + offset : q; };   // absent tensors stay absent
+    for (int64_t b0 = 0; b0 < batch; b0 += fit) {
+        const int64_t nb = batch - b0 < fit ? batch - b0 : fit;
+        const int64_t el = b0 * t * neurons, row = b0 * neurons;             // offsets of this slice
+        float *ckpt_v = base, *ckpt_i = syn ? base + fit * per_element : nullptr;
+        // the checkpoints of a slice are laid out (nb, n_ck, neurons) without padding between elements
+        LayerConsts q = p;
+        q.v_init = at(p.v_init, row);
+        q.i_init = at(p.i_init, row);
+        q.alpha_mem = at(p.alpha_mem, row);
+        q.alpha_syn = at(p.alpha_syn, row);
+        q.c = at(p.c, row);
+        q.theta = at(p.theta, row);
+        q.theta_low = at(p.theta_low, row);
+        const int rc = syn ? launch_checkpoints_only<true>(ckpt_v, ckpt_i, input + el, q, nb, t, neurons, s)
+                           : launch_checkpoints_only<false>(ckpt_v, ckpt_i, input + el, q, nb, t, neurons, s);
+        if (rc) return rc;
+        const int rb = exodus_layer_lif_backward(
+            at(grad_input, el), at(alpha_mem_grad, row), at(alpha_syn_grad, row), at(vmem_init_grad, row),
+            at(isyn_init_grad, row), at(grad_spikes, el), at(grad_v_last, row), at(grad_i_last, row), input + el,
+            ckpt_v, ckpt_i, q.v_init, q.i_init, q.alpha_mem, q.alpha_syn, q.c, q.theta, q.theta_low, apply_theta_low,
+            max_num_spikes, decay_early, norm_input, surrogate_kind, surr_p0, surr_p1, at(surr, el), at(grad_v_rec, el),
+            at(grad_i_rec, el), nb, t, neurons, stream);
+        if (rb) return rb;
+    }
+    return hipSuccess;
 }
 
 EXODUS_API int exodus_layer_leaky_forward(float *out, float *v_last, double *out_sum, const float *input,

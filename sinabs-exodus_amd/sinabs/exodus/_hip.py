@@ -21,7 +21,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("EXODUS_HIP_LIBRARY") or os.path.join(_HERE, "libexodus_hip.so")
 
 SURR_TENSOR, SURR_SINGLE_EXP, SURR_PERIODIC_EXP, SURR_HEAVISIDE = 0, 1, 2, 3
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 _p = ctypes.c_void_p
 _i64 = ctypes.c_int64
@@ -46,6 +46,8 @@ _SIGNATURES = {
     "exodus_layer_checkpoint_interval": ([], _int),
     "exodus_layer_lif_forward": ([_p] * 16 + [_int, _int, _int, _int, _int, _i64, _i64, _i64, _p], _int),
     "exodus_layer_lif_backward": ([_p] * 18 + [_int, _int, _int, _int, _int, _f, _f, _p, _p, _p, _i64, _i64, _i64, _p], _int),
+    "exodus_layer_scratch_floats": ([], _i64),
+    "exodus_layer_lif_backward_from_input": ([_p] * 16 + [_int, _int, _int, _int, _int, _f, _f, _p, _p, _p, _i64, _i64, _i64, _p], _int),
     "exodus_layer_leaky_forward": ([_p] * 6 + [_int, _int, _i64, _i64, _i64, _p], _int),
     "exodus_layer_leaky_backward": ([_p] * 9 + [_int, _int, _i64, _i64, _i64, _p], _int),
 }
@@ -472,6 +474,11 @@ def layerLifForward(input, vmemPostInitial, isynInitial, alphaMem, alphaSyn, mem
     return res
 
 
+def scratchFloats() -> int:
+    """Floats of checkpoint memory the library holds per GPU for ``layerLifBackward(..., ckptV=None)``."""
+    return int(lib.exodus_layer_scratch_floats())
+
+
 def layerLifBackward(gradSpikes, gradVLast, gradILast, input, ckptV, ckptI, vmemPostInitial, isynInitial, alphaMem,
                      alphaSyn, membrSubtract, theta, thetaLow, applyThetaLow: bool, maxNumSpikes: int,
                      decayEarly: bool, normInput: bool, surrogateKind: int, surrP0: float, surrP1: float,
@@ -483,7 +490,9 @@ def layerLifBackward(gradSpikes, gradVLast, gradILast, input, ckptV, ckptI, vmem
     gradient that is not wanted is neither computed nor allocated and comes back as None.
     ``surrogateKind == SURR_TENSOR`` takes the spike function's derivative from ``surr`` (batch, time, neurons).
     ``gradVRec`` / ``gradIRec`` (batch, time, neurons) are gradients on the forward's state records; one that is
-    missing while the other is given counts as zero."""
+    missing while the other is given counts as zero.
+    ``ckptV is None`` calls ``exodus_layer_lif_backward_from_input``: the library rebuilds the checkpoints in its
+    own fixed device array (``scratchFloats()``) and allocates nothing; concurrent calls on one GPU must not overlap."""
     _btm(input, "input")
     b, t, m = input.shape
     n = b * m
@@ -491,9 +500,11 @@ def layerLifBackward(gradSpikes, gradVLast, gradILast, input, ckptV, ckptI, vmem
     if _btm(gradSpikes, "gradSpikes", input).shape != input.shape:
         raise RuntimeError("gradSpikes must have the shape of input")
     n_ck = (t + checkpointInterval() - 1) // checkpointInterval()
-    for nm, x in (("ckptV", ckptV),) + ((("ckptI", ckptI),) if syn else ()):
-        if _btm(x, nm, input).shape != (b, n_ck, m):
-            raise RuntimeError(f"{nm} must have shape ({b}, {n_ck}, {m})")
+    from_input = ckptV is None
+    if not from_input:
+        for nm, x in (("ckptV", ckptV),) + ((("ckptI", ckptI),) if syn else ()):
+            if _btm(x, nm, input).shape != (b, n_ck, m):
+                raise RuntimeError(f"{nm} must have shape ({b}, {n_ck}, {m})")
     rows = [("vmemPostInitial", vmemPostInitial), ("alphaMem", alphaMem), ("membrSubtract", membrSubtract),
             ("theta", theta)]
     if syn:
@@ -547,8 +558,11 @@ def layerLifBackward(gradSpikes, gradVLast, gradILast, input, ckptV, ckptI, vmem
             int(bool(decayEarly)), int(bool(normInput)), int(surrogateKind), float(surrP0), float(surrP1), _ptr(surr),
             _ptr(gradVRec), _ptr(gradIRec), b, t, m, _stream(input))
     with torch.cuda.device(input.device):
-        _check(lib.exodus_layer_lif_backward(*head, _ptr(ckptV), _ptr(ckptI) if syn else None, *tail),
-               "exodus_layer_lif_backward")
+        if from_input:
+            _check(lib.exodus_layer_lif_backward_from_input(*head, *tail), "exodus_layer_lif_backward_from_input")
+        else:
+            _check(lib.exodus_layer_lif_backward(*head, _ptr(ckptV), _ptr(ckptI) if syn else None, *tail),
+                   "exodus_layer_lif_backward")
     return gradInput, am_g, as_g, v0_g, i0_g
 
 

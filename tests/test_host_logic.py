@@ -40,7 +40,7 @@ def test_library_exports_every_declared_symbol():
     extra = [l.split()[-1] for l in exported.splitlines() if " T " in l and not l.split()[-1].startswith("exodus_")]
     assert not extra, f"unexpected exported symbols: {extra}"
     lib.exodus_hip_abi_version.restype = ctypes.c_int
-    assert lib.exodus_hip_abi_version() == 4
+    assert lib.exodus_hip_abi_version() == 5
 
 
 def test_layer_entry_points_reject_too_wide_layers_before_touching_the_device():
@@ -54,6 +54,35 @@ def test_layer_entry_points_reject_too_wide_layers_before_touching_the_device():
     rc = _hip.lib.exodus_layer_leaky_forward(*([null] * 6), 1, 1, 1, 4, wide, null)
     assert rc == 1
     assert _hip.lib.exodus_layer_lif_forward(*([null] * 16), 0, -1, 1, 1, 0, 0, 4, 8, null) == 0   # empty batch
+
+
+def test_backward_without_allocation_rejects_what_its_scratch_cannot_hold():
+    """The size check of exodus_layer_lif_backward_from_input comes before anything touches a device:
+    one batch element whose checkpoints exceed the fixed scratch array is refused with the library's
+    own status, and the message says what to use instead."""
+    from sinabs.exodus import _hip
+    cap = _hip.scratchFloats()
+    assert cap == 1 << 24
+    ck = _hip.checkpointInterval()
+    fake = ctypes.c_void_p(4096)                       # never dereferenced: the call returns before any launch
+    def call(t, neurons, syn):
+        ptrs = [fake] * 16
+        if not syn:
+            ptrs[10] = None                            # isyn_initial
+            ptrs[12] = None                            # alpha_syn
+        return _hip.lib.exodus_layer_lif_backward_from_input(*ptrs, 0, -1, 1, 1, _hip.SURR_SINGLE_EXP, 0.5, 1.0,
+                                                             None, None, None, 3, t, neurons, None)
+    assert call(ck * 1000, 1 << 20, False) == -2       # 1000 checkpoints of 2^20 neurons
+    assert call(ck * 16, 1 << 20, True) == -2          # fits once, but not for potential and current
+    assert call(ck * 16 + 1, 1 << 20, False) == -2     # one step more needs one checkpoint more
+    msg = _hip.lib.exodus_hip_error_string(-2).decode()
+    assert "scratch" in msg and "exodus_layer_lif_backward" in msg
+    with pytest.raises(_hip.ExodusHipError, match="scratch"):
+        _hip._check(-2, "exodus_layer_lif_backward_from_input")
+    assert _hip.lib.exodus_layer_lif_backward_from_input(*([fake] * 16), 0, -1, 1, 1, 9, 0.5, 1.0, None, None, None,
+                                                         1, 8, 8, None) == 1     # unknown surrogate kind
+    assert _hip.lib.exodus_layer_lif_backward_from_input(*([None] * 16), 0, -1, 1, 1, 1, 0.5, 1.0, None, None, None,
+                                                         0, 8, 8, None) == 0     # empty batch
 
 
 def test_loader_signatures_cover_the_header():
