@@ -25,9 +25,11 @@
  *                               v_init == 0, see the note at the function)
  *   oracle_spike_forward        notebook cells 2/4/6 on cumsum(input); bit-equality with
  *                               oracle_lif_forward on a dyadic grid where all arithmetic is exact
- *   oracle_spike_backward       equality with oracle_lif_backward at alpha == 1; quadratic sum ==
- *                               reverse recurrence in fp64.  For alpha != 1 and for clipped steps
- *                               nothing else holds it: parity unpinned there
+ *   oracle_spike_backward       equality with oracle_lif_backward at alpha == 1; for every alpha and
+ *                               with clipped steps: torch autograd through an independent step loop of
+ *                               the model whose exact gradient the reference's sum is (a spike reaches the
+ *                               next step undecayed, a clipped step's lift counts as a constant); its
+ *                               distance to the exact gradient of oracle_spike_forward is measured there
  */
 #include <math.h>
 #include <stdint.h>
@@ -229,9 +231,12 @@ EXPORT void oracle_lif_backward_alpha(float *grad_alpha, const float *grad_out,
  *                          (all arithmetic exact) it equals oracle_lif_forward applied to the
  *                          input whose leaky integral is the given potential
  *   oracle_spike_backward  alpha = 1, nothing clipped: its leaky adjoint equals the notebook's
- *                          cell 4/6 gradients and oracle_lif_backward; for alpha != 1 or clipped
- *                          steps only the agreement of this O(T^2) sum with an O(T) recurrence in
- *                          float64 is checked -- parity unpinned there
+ *                          cell 4/6 gradients and oracle_lif_backward.  Any alpha, clipped steps: the
+ *                          sum has factors (alpha - c y_k) where the forward pass above would give
+ *                          alpha (1 - c y_k); it is the exact gradient of a forward pass in which a
+ *                          spike reaches the next step undecayed and the lift of a clipped step is a
+ *                          constant, and equals torch autograd through a step loop of that model.  It
+ *                          is restated as the reference has it, not corrected.
  * ------------------------------------------------------------------------- */
 
 /* For each step in turn: a potential at or above theta emits min(trunc(u/theta), cap) spikes and

@@ -385,3 +385,85 @@ def test_spike_backward_quadratic_sum_equals_reverse_recurrence(alpha):
         want[:, i] = y[:, i] * go[:, i] - y[:, i] * c * m
         m = go[:, i] * y[:, i] + (alpha - c * y[:, i]) * m
     np.testing.assert_allclose(got.numpy(), want.numpy(), rtol=1e-4, atol=1e-5)
+
+
+class _Surrogate(torch.autograd.Function):
+    """spike count (value taken from `counts`) whose derivative with respect to the potential is `surr`"""
+
+    @staticmethod
+    def forward(ctx, u, counts, surr):
+        ctx.save_for_backward(surr)
+        return counts.clone()
+
+    @staticmethod
+    def backward(ctx, g):
+        (surr,) = ctx.saved_tensors
+        return g * surr, None, None
+
+
+def _spike_function_autograd(v, alpha, c, theta, lo, use_lo, surr, as_backward_formula=False):
+    """The experimental spike generation as a float64 torch step loop, differentiated by autograd, with
+    ds/du := surr.  Returns (leaf v, spikes).
+
+    as_backward_formula=False: what oracle_spike_forward computes (reference
+    cuda/experimental_kernels.h:33-63): every spike lowers the following steps by alpha^j c count,
+    j = 1, 2, ..., and a step below the lower bound raises them by alpha^j (lo - u).
+    as_backward_formula=True: the model whose exact gradient the reference's backward formula is
+    (cuda/experimental_kernels.h:118-140): the first following step loses c count undecayed (alpha^(j-1)),
+    and the amount a clipped step adds to later steps is treated as a constant."""
+    n, t = v.shape
+    v = v.double().clone().requires_grad_(True)
+    adj = torch.zeros(n, dtype=torch.float64)          # what earlier steps add to this one
+    spikes = []
+    for i in range(t):
+        u = v[:, i] + adj
+        counts = torch.where(u >= theta, torch.div(u, theta, rounding_mode="trunc"), torch.zeros_like(u)).detach()
+        below = (u < lo) & (u < theta) if use_lo else torch.zeros_like(u, dtype=torch.bool)
+        y = surr[:, i].double()
+        s = _Surrogate.apply(u, counts, torch.where(below, torch.zeros_like(y), y) if as_backward_formula else y)
+        spikes.append(s)
+        d = -c * s
+        if use_lo:
+            lift = lo - u
+            d = torch.where(below, lift.detach() if as_backward_formula else lift, d)
+        adj = alpha * adj + d if as_backward_formula else alpha * (adj + d)
+    return v, torch.stack(spikes, 1)
+
+
+@pytest.mark.parametrize("use_lo", [False, True])
+@pytest.mark.parametrize("alpha", [1.0, 0.9, 0.6])
+def test_spike_backward_is_the_exact_gradient_of_a_stated_model(alpha, use_lo):
+    """Pins oracle_spike_backward for alpha != 1 and for clipped steps against autograd through an
+    independent step loop.  The reference's sum (cuda/experimental_kernels.h:118-140) has the factors
+    (alpha - c y_k) where its own forward pass (:33-63, first affected step already decayed) would give
+    alpha (1 - c y_k): term by term it is the exact gradient of a forward pass in which a spike reaches the
+    next step undecayed and a clipped step's contribution to later steps counts as a constant.  That is
+    checked here; the distance to the exact gradient of the actual forward pass is printed (zero at
+    alpha = 1 without clipped steps)."""
+    g = torch.Generator().manual_seed(31)
+    n, t, c, theta, lo = 48, 40, 0.6, 1.0, -0.3
+    x = torch.randn(n, t, generator=g) * 0.6 + 0.25
+    v = ref.leaky_forward(x.contiguous(), torch.zeros(n), alpha * torch.ones(n))
+    surr = (torch.rand(n, t, generator=g) * 1.2).contiguous()          # the backward takes them as given
+    go = torch.randn(n, t, generator=g).contiguous()
+    # the actual forward pass: same spike trains as the oracle, so the same function
+    leaf, s = _spike_function_autograd(v, alpha, c, theta, lo, use_lo, surr)
+    u = v.clone()
+    s_oracle = ref.spike_forward(u, alpha, c, theta, lo, use_lo, -1)
+    assert s.sum() > 50 and torch.equal(s.detach().float(), s_oracle)
+    (s * go.double()).sum().backward()
+    exact = leaf.grad
+    nc = (u > lo).float().contiguous() if use_lo else torch.ones(n, t)   # what reference spike.py:88-92 hands over
+    assert not use_lo or 0 < (nc == 0).sum() < nc.numel() // 2
+    got = ref.spike_backward(surr, go, nc, alpha, c).double()
+    # the model of the backward formula, run on potentials that clip exactly where `nc` says
+    leaf2, s2 = _spike_function_autograd(u.double() if use_lo else v, alpha, c, theta, lo, False, surr * nc, True)
+    (s2 * go.double()).sum().backward()
+    np.testing.assert_allclose(got.numpy(), leaf2.grad.numpy(), rtol=1e-4, atol=1e-5)
+    dev = (got - exact).abs().max().item()
+    print(f"alpha={alpha} lower bound={use_lo}: largest |reference formula - exact gradient of the forward pass| = "
+          f"{dev:.3g} (largest gradient {exact.abs().max().item():.3g})")
+    if alpha == 1.0 and not use_lo:
+        np.testing.assert_allclose(got.numpy(), exact.numpy(), rtol=1e-4, atol=1e-5)
+    else:
+        assert dev > 1e-3                                               # not a rounding matter
