@@ -54,6 +54,10 @@ MEASURED_TRAFFIC = {
     ("c2", "exodus_layer_lif_forward"): (10.30e9, "profiles/layer_lif_c2_kernel_stats_pmc.md"),
     ("c3", "exodus_layer_leaky_backward"): (3.15e9, "profiles/layer_leaky_c3_kernel_stats_pmc.md"),
     ("c3", "exodus_layer_leaky_forward"): (2.10e9, "profiles/layer_leaky_c3_kernel_stats_pmc.md"),
+    ("c2", "exodus_lif_forward"): (15.76e9, "profiles/rows_lif_c2_kernel_stats_pmc.md"),
+    ("c2", "exodus_lif_backward_fused"): (16.16e9, "profiles/rows_lif_c2_kernel_stats_pmc.md"),
+    ("c3", "exodus_leaky_forward"): (2.12e9, "profiles/rows_leaky_c3_kernel_stats_pmc.md"),
+    ("c3", "exodus_leaky_backward_fused"): (3.20e9, "profiles/rows_leaky_c3_kernel_stats_pmc.md"),
 }
 
 # what the default run reports next to its headline workload: (workload, path)
@@ -452,6 +456,32 @@ def roofline(key, wl, fwd_ms, bwd_ms, bf, bb, traffic_known=True):
     }
 
 
+def measure_reallocations(args, torch, hip, act, dev):
+    """The chosen workload measured again and again on freshly allocated tensors."""
+    import random
+    rnd = random.Random(5)
+    junk = []
+    build = build_layer_workload if args.path == "layer" else build_workload
+    for k in range(args.reallocations):
+        torch.cuda.empty_cache()
+        wl = build(args.workload, torch, hip, act, dev)
+        m = measure(wl, args.steps, args.warmup, torch)
+        bf, bb = wl.get("bytes", WORKLOADS[args.workload]["bytes"])
+        n_t = wl["N"] * wl["T"]
+        print(json.dumps({"round": k, "other_allocations_held_GiB": round(sum(j.numel() for j in junk) / 2 ** 30, 2),
+                          "fwd_ms": m["fwd_ms"], "bwd_ms": m["bwd_ms"],
+                          "fwd_GBs": n_t * bf / m["fwd_ms"] / 1e6, "bwd_GBs": n_t * bb / m["bwd_ms"] / 1e6,
+                          "fwd_bwd_combined_frac": n_t * (bf + bb) / ((m["fwd_ms"] + m["bwd_ms"]) * 1e-3) / 1e9 / HBM_PEAK_GBS}),
+              flush=True)
+        del wl
+        torch.cuda.empty_cache()
+        # change what the driver has to give out next: hold one more block of another size, or drop one
+        if k % 2 == 0 or not junk:
+            junk.append(torch.empty(int(rnd.uniform(0.3, 9.0) * 2 ** 30), dtype=torch.uint8, device=dev))
+        elif rnd.random() < 0.5:
+            junk.pop(rnd.randrange(len(junk)))
+
+
 def without_cycle_option(argv):
     """The command line without ``--after-hbm-cycle [N]`` (for the child process that measures)."""
     rest, skip = [], False
@@ -495,6 +525,12 @@ def main():
                          "layer API (Conv2d -> IAFSqueeze -> AvgPool -> Conv2d -> IAFSqueeze -> Flatten -> Linear -> "
                          "IAFSqueeze, batch 64 x 300 steps, cross-entropy on spike counts): layer-layout kernels, the "
                          "transposing (rows, time) Functions, and the convolution / pooling / linear layers alone")
+    ap.add_argument("--reallocations", type=int, default=0, metavar="N",
+                    help="instead of the benchmark, build and measure the chosen workload N times in this process, "
+                         "releasing its tensors to the driver and allocating other memory of varying size in between, "
+                         "and print one JSON line per round: the same kernels on the same shapes run at different rates "
+                         "depending on which physical memory their tensors were given (a process that has allocated "
+                         "nothing before, as the default run, gets one fixed placement)")
     ap.add_argument("--after-hbm-cycle", type=int, nargs="?", const=2, default=0, metavar="N",
                     help="first let N (default 2) child processes in turn allocate nearly all device memory and exit, "
                          "then run the chosen measurement in another child process (this process starts no GPU work "
@@ -535,6 +571,10 @@ def main():
         wl = build_workload(args.workload, torch, hip, act, dev)
     fwd, bwd, N, T = wl["fwd"], wl["bwd"], wl["N"], wl["T"]
 
+    if args.reallocations:
+        del wl, fwd, bwd
+        measure_reallocations(args, torch, hip, act, dev)
+        return
     if args.ceilings:
         print(json.dumps(measure_ceilings(args, torch, hip, dev)))
         return
@@ -581,9 +621,22 @@ def main():
         "roofline": roof,
     }
     if args.others and not args.shape:
+        # The same kernels on the same shapes after the tensors were released to the driver and allocated
+        # again (three times): which physical memory an allocation lands on moves the rate of these kernels
+        # by several percent, and a process that has allocated nothing before -- the measurement above --
+        # is handed the placement that has measured slowest.  Reported next to it, not instead of it.
+        del wl, fwd, bwd
+        again = []
+        for _ in range(3):
+            torch.cuda.empty_cache()
+            wl2 = (build_layer_workload if args.path == "layer" else build_workload)(args.workload, torch, hip, act, dev)
+            m2 = measure(wl2, max(3, args.steps // 2), max(2, args.warmup // 2), torch)
+            again.append(roofline(args.workload, wl2, m2["fwd_ms"], m2["bwd_ms"], bf, bb)["frac"])
+            del wl2
+        roof["frac_by_placement"] = {"first_allocation_of_the_process": roof["frac"],
+                                     "after_release_and_reallocation": again}
         # the other configurations and the (rows, time) kernels behind the autograd Functions, a few
         # steps each: same measurement, reported beside the headline workload
-        del wl, fwd, bwd
         result["others"] = []
         for key, path in OTHERS:
             if (key, path) == (args.workload, args.path):
