@@ -11,6 +11,7 @@ the launch stream) and a CPU baseline (the sinabs-style per-time-step torch loop
 timed on this machine's host cores on a bounded sample of the same workload).
 """
 import argparse
+import contextlib
 import json
 import math
 import os
@@ -64,25 +65,48 @@ MEASURED_TRAFFIC = {
 OTHERS = [("c2", "layer"), ("c3", "layer"), ("c5", "rows"), ("c2", "rows"), ("c3", "rows")]
 
 
-def build_layer_workload(key, torch, hip, act, dev):
+class Placement:
+    """Where a workload's tensors are allocated.  With ``regions`` (sinabs.exodus.hbm.HbmRegions) the inputs
+    (x, grad_output) go into the range made of the first kind of HBM, outputs into the second and -- where one
+    range cannot hold them, and for the checkpoints -- the third, so that no kernel writes into the region it
+    reads most from; without, everything comes from torch's ordinary allocator."""
+
+    def __init__(self, torch, dev, regions=None):
+        self.torch, self.dev, self.regions = torch, dev, regions
+
+    def empty(self, shape, k):
+        if self.regions is None:
+            return self.torch.empty(tuple(shape), device=self.dev)
+        return self.regions.empty(shape, region=k)
+
+    def describe(self):
+        if self.regions is None:
+            return {"placement": "ordinary allocator"}
+        return {"placement": "hbm regions (sinabs.exodus.hbm): inputs in one region of HBM, outputs in another, "
+                             "checkpoints in the third",
+                "placement_verified_by_timed_copies": self.regions.verified,
+                "placement_measured": {k: ([round(x) for x in v] if isinstance(v, list) else round(v))
+                                       for k, v in self.regions.report.items()}}
+
+
+def build_layer_workload(key, torch, hip, act, dev, place=None):
     """The same workloads on the layer's own (batch, time, neurons) layout: one kernel per direction,
     forward keeps checkpoints only, backward re-reads the input and rebuilds v_mem / i_syn.
     Algorithmic bytes per neuron-timestep: forward 8 (x in, spikes out), backward 12 (grad_spikes
     and x in, grad_x out)."""
     w = WORKLOADS[key]
+    place = place or Placement(torch, dev)
     B, T, M = w["batch"], w["steps"], w["neurons"]
     N = B * M
     g = torch.Generator(device=dev).manual_seed(list(WORKLOADS).index(key))
-    if key == "c1":
-        x = torch.rand(B, T, M, generator=g, device=dev) * 0.5
-    else:
-        x = torch.randn(B, T, M, generator=g, device=dev) * w["std"] + w["mean"]
-    go = torch.ones(B, T, M, device=dev)
+    x = place.empty((B, T, M), 0)
+    x.uniform_(0.0, 0.5, generator=g) if key == "c1" else x.normal_(w["mean"], w["std"], generator=g)
+    go = place.empty((B, T, M), 0).fill_(1.0)
     rows = lambda v: torch.as_tensor(v, dtype=torch.float32, device=dev).expand(B, M).flatten().contiguous()
     zeros = torch.zeros(N, device=dev); ones = torch.ones(N, device=dev)
     surr = act.SingleExponential()
     kind, p0, p1 = hip.SURR_SINGLE_EXP, surr.grad_width, surr.grad_scale
-    spikes = torch.empty_like(x); gi = torch.empty_like(x)
+    spikes = place.empty(x.shape, 1); gi = place.empty(x.shape, 1)
     if key == "c5":
         cfg = dict(a_mem=rows(math.exp(-1 / 20.0)), a_syn=rows(math.exp(-1 / 5.0)), lo=rows(-1.0), cap=2, norm=True)
     elif key == "c2":
@@ -124,16 +148,15 @@ def build_layer_workload(key, torch, hip, act, dev):
                 bwd_name="exodus_layer_lif_backward", bytes=(8, 12))
 
 
-def build_workload(key, torch, hip, act, dev):
+def build_workload(key, torch, hip, act, dev, place=None):
     w = WORKLOADS[key]
+    place = place or Placement(torch, dev)
     B, T, M = w["batch"], w["steps"], w["neurons"]
     N = B * M
     g = torch.Generator(device=dev).manual_seed(list(WORKLOADS).index(key))
-    if key == "c1":
-        x = torch.rand(N, T, generator=g, device=dev) * 0.5
-    else:
-        x = torch.randn(N, T, generator=g, device=dev) * w["std"] + w["mean"]
-    go = torch.ones(N, T, device=dev)
+    x = place.empty((N, T), 0)
+    x.uniform_(0.0, 0.5, generator=g) if key == "c1" else x.normal_(w["mean"], w["std"], generator=g)
+    go = place.empty((N, T), 0).fill_(1.0)
     rows = lambda v: torch.as_tensor(v, dtype=torch.float32, device=dev).expand(B, M).flatten().contiguous()
     zeros = torch.zeros(N, device=dev)
     ones = torch.ones(N, device=dev)
@@ -143,7 +166,10 @@ def build_workload(key, torch, hip, act, dev):
 
     if key == "c5":
         a_mem = rows(math.exp(-1 / 20.0)); a_syn = rows(math.exp(-1 / 5.0)); lo = rows(-1.0)
-        s = torch.empty_like(x); v = torch.empty_like(x); i = torch.empty_like(x); gi = torch.empty_like(x)
+        # the backward kernel reads one tensor from each region and writes into the third; with its three inputs
+        # in one region it measured 15 % slower
+        s = place.empty(x.shape, 1); v = place.empty(x.shape, 1)
+        i = place.empty(x.shape, 2); gi = place.empty(x.shape, 2)
 
         def fwd():
             hip.synLifForward(x, zeros, zeros, a_mem, a_syn, ones, ones, lo, True, 2, True, True, out=(s, v, i))
@@ -160,8 +186,10 @@ def build_workload(key, torch, hip, act, dev):
         cap = 1 if key == "c2" else -1
         xin = x
         if key == "c2":
-            xin = ((1.0 - a_mem).unsqueeze(1) * x).contiguous()   # norm_input scaling, done once outside the step
-        s = torch.empty_like(x); v = torch.empty_like(x); gi = torch.empty_like(x)
+            xin = place.empty(x.shape, 0)
+            torch.mul((1.0 - a_mem).unsqueeze(1), x, out=xin)     # norm_input scaling, done once outside the step
+        s = place.empty(x.shape, 1); v = place.empty(x.shape, 1)
+        gi = place.empty(x.shape, 2)
 
         def fwd():
             hip.lifForward(s, v, xin, zeros, a_mem, ones, ones, None, False, cap)
@@ -174,12 +202,12 @@ def build_workload(key, torch, hip, act, dev):
     elif key == "c3":
         tau = 5.0 + 45.0 * torch.rand(M, generator=g, device=dev)
         a_mem = rows(torch.exp(-1.0 / tau))
-        out = None
-        gi = torch.empty_like(x)
+        out = place.empty(x.shape, 1)
+        gi = place.empty(x.shape, 2)
         holder = {}
 
         def fwd():
-            holder["out"] = hip.leakyForward(x, zeros, a_mem)
+            holder["out"] = hip.leakyForward(x, zeros, a_mem, output=out)
 
         def bwd():
             r = hip.leakyBackwardFused(go, a_mem, output=holder["out"], vmemInitial=zeros, needAlphaGrad=True,
@@ -456,6 +484,54 @@ def roofline(key, wl, fwd_ms, bwd_ms, bf, bb, traffic_known=True):
     }
 
 
+def measure_region_map(args, torch, dev):
+    """Rates of a flat copy between every two of the buffers that fill device memory, in allocation order."""
+    probes = Probes(torch)
+    gib = args.region_map
+    nel = int(gib * 2 ** 30) // 4
+    free, total = torch.cuda.mem_get_info()
+    n = int((free / 2 ** 30 - 6) // gib)
+    bufs = [torch.empty(nel, device=dev) for _ in range(n)]
+    bufs[0].normal_()
+
+    def rate(dst, src, reps=3):
+        probes.stream(dst, src)
+        ev = [[torch.cuda.Event(enable_timing=True) for _ in range(2)] for _ in range(reps)]
+        for a, b in ev:
+            a.record(); probes.stream(dst, src); b.record()
+        torch.cuda.synchronize()
+        return nel * 8 / sorted(a.elapsed_time(b) for a, b in ev)[reps // 2] / 1e6
+
+    mat = [[rate(bufs[j], bufs[i]) if i != j else 0.0 for j in range(n)] for i in range(n)]
+    flat = sorted(v for row in mat for v in row if v)
+    # the rates fall into two groups; split them at the widest gap between neighbours of the sorted list
+    # (looked for between the 10th and the 90th percentile)
+    lo, hi = len(flat) // 10, len(flat) * 9 // 10
+    cut = max(range(lo, hi), key=lambda k: flat[k + 1] - flat[k])
+    threshold = (flat[cut] + flat[cut + 1]) / 2
+    for i, row in enumerate(mat):
+        print(f"src {i:3d} ({i * gib:5.0f} GiB): " + "".join("-" if i == j else ("#" if v < threshold else ".")
+                                                             for j, v in enumerate(row)), flush=True)
+    slow_with_first = [j for j in range(1, n) if mat[0][j] < threshold]
+    # buffers are grouped by which of them copy slowly into each other
+    groups, seen = [], set()
+    for i in range(n):
+        if i not in seen:
+            grp = [i] + [j for j in range(n) if j != i and mat[i][j] < threshold and j not in seen]
+            seen.update(grp)
+            groups.append(grp)
+    inside = [mat[i][j] for g in groups for i in g for j in g if i != j]
+    across = [mat[i][j] for a in groups for b in groups if a is not b for i in a for j in b]
+    med = lambda r: sorted(r)[len(r) // 2] if r else None
+    print(json.dumps({
+        "buffers": n, "GiB_each": gib, "device_GiB": total / 2 ** 30, "threshold_GBs": threshold,
+        "groups_of_buffers_that_copy_slowly_into_each_other (allocation order, GiB from the first)":
+            [[min(g) * gib, (max(g) + 1) * gib, len(g)] for g in groups],
+        "copy_inside_one_group_GBs": {"min": min(inside), "median": med(inside), "max": max(inside)},
+        "copy_across_groups_GBs": {"min": min(across), "median": med(across), "max": max(across)} if across else None,
+        "pairs_on_the_wrong_side_of_the_threshold": sum(v >= threshold for v in inside) + sum(v < threshold for v in across)}))
+
+
 def measure_reallocations(args, torch, hip, act, dev):
     """The chosen workload measured again and again on freshly allocated tensors."""
     import random
@@ -525,6 +601,17 @@ def main():
                          "layer API (Conv2d -> IAFSqueeze -> AvgPool -> Conv2d -> IAFSqueeze -> Flatten -> Linear -> "
                          "IAFSqueeze, batch 64 x 300 steps, cross-entropy on spike counts): layer-layout kernels, the "
                          "transposing (rows, time) Functions, and the convolution / pooling / linear layers alone")
+    ap.add_argument("--placement", default="regions", choices=["regions", "plain"],
+                    help="regions (default): allocate through sinabs.exodus.hbm -- three ranges of device memory, each made "
+                         "of one of the three regions of this GPU's HBM; inputs in the first, what the kernels write in the others.  A kernel that "
+                         "reads one third and writes another moves 8-12 %% more bytes per second than one that does both "
+                         "inside one third, which is what a process gets from the ordinary allocator.  plain: the ordinary "
+                         "allocator.  The default run reports both (roofline.frac_by_placement); the plain figure is "
+                         "measured first, in a child process, before this process touches the GPU")
+    ap.add_argument("--region-map", type=float, nargs="?", const=4.0, default=0.0, metavar="GIB",
+                    help="instead of the benchmark, fill device memory with buffers of GIB (default 4) GiB in the order "
+                         "the driver hands them out, copy every buffer into every other with a flat copy kernel and print "
+                         "the matrix of rates as text plus one JSON line with the region boundaries found")
     ap.add_argument("--reallocations", type=int, default=0, metavar="N",
                     help="instead of the benchmark, build and measure the chosen workload N times in this process, "
                          "releasing its tensors to the driver and allocating other memory of varying size in between, "
@@ -557,6 +644,23 @@ def main():
         env = dict(os.environ, EXODUS_BENCH_AFTER_HBM_CYCLE=str(args.after_hbm_cycle))
         sys.exit(subprocess.run([sys.executable, os.path.abspath(__file__)] + rest, env=env).returncode)
 
+    plain_first, plain_note = None, None
+    special = args.region_map or args.reallocations or args.ceilings or args.conv_snn or args.shape or args.copy_probe
+    if args.placement == "regions" and args.others and not special:
+        # the same measurement with the ordinary allocator, in a process of its own and before this one touches
+        # the GPU, so that it sees what a program that allocates without further thought is handed
+        import subprocess
+        child = subprocess.run([sys.executable, os.path.abspath(__file__), "--placement", "plain", "--no-others",
+                                "--no-cpu-baseline", "--workload", args.workload, "--path", args.path,
+                                "--steps", str(args.steps), "--warmup", str(args.warmup)],
+                               capture_output=True, text=True)
+        try:
+            r = json.loads(child.stdout.strip().splitlines()[-1])["roofline"]
+            plain_first = {"frac": r["frac"], "fwd_bwd_combined_frac": r["fwd_bwd_combined_frac"],
+                           "kernel_ms": r["kernel_ms"], "other_kernel_ms": r["other_kernel"]["kernel_ms"]}
+        except (IndexError, KeyError, ValueError):
+            plain_first = {"error": (child.stderr or child.stdout)[-400:]}
+
     import torch
     assert torch.cuda.is_available(), "bench.py needs the GPU"
     from sinabs.exodus import _hip as hip
@@ -564,17 +668,23 @@ def main():
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    if args.path == "layer":
-        wl = build_layer_workload(args.workload, torch, hip, act, dev)
-    else:
-        args.path = "rows"
-        wl = build_workload(args.workload, torch, hip, act, dev)
-    fwd, bwd, N, T = wl["fwd"], wl["bwd"], wl["N"], wl["T"]
-
+    if args.region_map:
+        measure_region_map(args, torch, dev)
+        return
     if args.reallocations:
-        del wl, fwd, bwd
         measure_reallocations(args, torch, hip, act, dev)
         return
+    place = Placement(torch, dev)
+    if args.placement == "regions" and not (args.ceilings or args.conv_snn):
+        from sinabs.exodus import hbm
+        try:
+            place = Placement(torch, dev, hbm.enable(gib_per_region=32.0, device=dev))
+        except RuntimeError as err:                     # device memory in use by something else: measure without
+            plain_note = f"regions unavailable ({err}); ordinary allocator used"
+            print("[bench] " + plain_note, file=sys.stderr, flush=True)
+    build = build_layer_workload if args.path == "layer" else build_workload
+    wl = build(args.workload, torch, hip, act, dev, place)
+    fwd, bwd, N, T = wl["fwd"], wl["bwd"], wl["N"], wl["T"]
     if args.ceilings:
         print(json.dumps(measure_ceilings(args, torch, hip, dev)))
         return
@@ -616,33 +726,24 @@ def main():
         "data": "synthetic",
         "config": {"workload": WORKLOADS[args.workload]["name"], "path": args.path, "rows": N, "time_steps": T,
                    "algorithmic_bytes_per_neuron_timestep": bf + bb,
+                   **place.describe(),
                    **({"after_hbm_cycles": int(os.environ["EXODUS_BENCH_AFTER_HBM_CYCLE"])}
                       if os.environ.get("EXODUS_BENCH_AFTER_HBM_CYCLE") else {})},
         "roofline": roof,
     }
+    if plain_first is not None:
+        roof["frac_by_placement"] = {
+            "regions (this run's figures)": {"frac": roof["frac"], "fwd_bwd_combined_frac": roof["fwd_bwd_combined_frac"]},
+            "ordinary allocator, first allocations of a process (measured before this one touched the GPU)": plain_first}
     if args.others and not args.shape:
-        # The same kernels on the same shapes after the tensors were released to the driver and allocated
-        # again (three times): which physical memory an allocation lands on moves the rate of these kernels
-        # by several percent, and a process that has allocated nothing before -- the measurement above --
-        # is handed the placement that has measured slowest.  Reported next to it, not instead of it.
-        del wl, fwd, bwd
-        again = []
-        for _ in range(3):
-            torch.cuda.empty_cache()
-            wl2 = (build_layer_workload if args.path == "layer" else build_workload)(args.workload, torch, hip, act, dev)
-            m2 = measure(wl2, max(3, args.steps // 2), max(2, args.warmup // 2), torch)
-            again.append(roofline(args.workload, wl2, m2["fwd_ms"], m2["bwd_ms"], bf, bb)["frac"])
-            del wl2
-        roof["frac_by_placement"] = {"first_allocation_of_the_process": roof["frac"],
-                                     "after_release_and_reallocation": again}
         # the other configurations and the (rows, time) kernels behind the autograd Functions, a few
-        # steps each: same measurement, reported beside the headline workload
+        # steps each: same measurement and placement, reported beside the headline workload
+        del wl, fwd, bwd
         result["others"] = []
         for key, path in OTHERS:
             if (key, path) == (args.workload, args.path):
                 continue
-            torch.cuda.empty_cache()
-            other = (build_layer_workload if path == "layer" else build_workload)(key, torch, hip, act, dev)
+            other = (build_layer_workload if path == "layer" else build_workload)(key, torch, hip, act, dev, place)
             mo = measure(other, max(3, args.steps // 2), max(2, args.warmup // 2), torch)
             obf, obb = other.get("bytes", WORKLOADS[key]["bytes"])
             result["others"].append({
@@ -652,6 +753,8 @@ def main():
                 "algorithmic_bytes_per_neuron_timestep": obf + obb,
                 "roofline": roofline(key, other, mo["fwd_ms"], mo["bwd_ms"], obf, obb)})
             del other
+    if plain_note:
+        result["config"]["placement_note"] = plain_note
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(args.workload, torch)
     print(json.dumps(result))

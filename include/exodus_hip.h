@@ -29,13 +29,14 @@ extern "C" {
 #endif
 
 /* ABI version of this header; bumped on any signature change. */
-#define EXODUS_HIP_ABI_VERSION 5
+#define EXODUS_HIP_ABI_VERSION 6
 
 int exodus_hip_abi_version(void);
 const char *exodus_hip_error_string(int status);
 
 /* Status values of this library's own (negative, so that they cannot collide with a hipError_t). */
 #define EXODUS_ERROR_SCRATCH_TOO_SMALL (-2)
+#define EXODUS_ERROR_REGIONS_NOT_FOUND (-3)
 
 /* ---------------------------------------------------------------------------------------------
  * One-to-one counterparts of the reference bindings
@@ -281,6 +282,45 @@ int exodus_spike_forward(float *out_spikes, float *vmem, float alpha, float memb
 int exodus_spike_backward(float *input_grad, const float *surr, const float *output_grad,
                           const float *not_clipped, float alpha, float membr_subtract, int64_t n,
                           int64_t t, void *stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Device memory sorted by HBM region (no counterpart in the reference, whose extension leaves the
+ * placement of its tensors to torch's allocator, reference cuda/bindings.cu:98,144,183)
+ * ------------------------------------------------------------------------------------------- */
+
+/* The HBM of an MI355X behaves as three regions: a kernel that reads one and writes another moves
+ * 8-12 % more bytes per second than one that reads and writes inside one region.
+ * exodus_hbm_regions_create takes nearly all free device memory in chunks of chunk_bytes (a multiple
+ * of the allocation granularity and of 16 KiB; 4 GiB is a good value: copies of less tell the regions apart less clearly), finds by timed copies which
+ * chunks lie in one region, maps ceil(bytes_per_region / chunk_bytes) chunks of each region behind
+ * each other into an address range of its own and returns the rest to the driver.  report->base[k] /
+ * bytes[k] are the three ranges; the caller hands out memory from them as it likes (the Python host
+ * side is sinabs/exodus/hbm.py) and must stop using them before exodus_hbm_regions_destroy.
+ * Returns EXODUS_ERROR_REGIONS_NOT_FOUND when the copies do not show three kinds of chunks with a
+ * clear gap (the report's fields up to kinds_found are then filled), hipErrorOutOfMemory when too
+ * little memory is free to find or fill three regions, hipErrorInvalidValue for bad arguments or a
+ * device that already has its ranges.  Takes a second or two; synchronises the device. */
+#define EXODUS_HBM_REGIONS 3
+#define EXODUS_HBM_PROBES 15
+typedef struct exodus_hbm_report {
+    void *base[EXODUS_HBM_REGIONS];
+    uint64_t bytes[EXODUS_HBM_REGIONS];
+    uint64_t chunk_bytes;
+    int32_t chunks_examined;                         /* physical chunks taken for sorting */
+    int32_t kinds_found;                             /* groups among the probe chunks; 3 on success */
+    int32_t chunks_ambiguous;                        /* chunks that matched no region clearly (not used) */
+    int32_t chunks_of_region[EXODUS_HBM_REGIONS];    /* chunks sorted into each region before enough were found */
+    float threshold_GBs;                             /* copy rate that separated "same region" from "other" */
+    float probe_same_kind_GBs, probe_other_kind_GBs; /* mean copy rate between probe chunks of one / of two regions */
+    float copy_inside_GBs[EXODUS_HBM_REGIONS];       /* finished ranges: first half of range k into its second half */
+    float copy_across_GBs[6];                        /* range j into range k: (0,1) (0,2) (1,0) (1,2) (2,0) (2,1) */
+    int32_t probe_chunk[EXODUS_HBM_PROBES];          /* the probe chunks (position in the order of creation), */
+    int32_t probe_kind[EXODUS_HBM_PROBES];           /* the group each was put in, and the copy rate between every */
+    float probe_pair_GBs[EXODUS_HBM_PROBES][EXODUS_HBM_PROBES];   /* two of them (mean of both directions) */
+} exodus_hbm_report;
+int exodus_hbm_regions_create(int device, uint64_t bytes_per_region, uint64_t chunk_bytes,
+                              exodus_hbm_report *report);
+int exodus_hbm_regions_destroy(int device);
 
 #ifdef __cplusplus
 }

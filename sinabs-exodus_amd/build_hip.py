@@ -12,7 +12,7 @@ import sys
 import tempfile
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-SRCS = [os.path.join(HERE, "csrc", f) for f in ("exodus_hip.hip", "exodus_layer.hip")]
+SRCS = [os.path.join(HERE, "csrc", f) for f in ("exodus_hip.hip", "exodus_layer.hip", "exodus_hbm.hip")]
 SRC = SRCS[0]
 INCLUDE = os.path.join(os.path.dirname(HERE), "include")
 OUT = os.path.join(HERE, "sinabs", "exodus", "libexodus_hip.so")

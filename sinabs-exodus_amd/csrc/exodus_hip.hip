@@ -809,6 +809,10 @@ EXODUS_API const char *exodus_hip_error_string(int status)
         return "one batch element needs more checkpoint memory than the library's fixed scratch array holds "
                "(see exodus_layer_scratch_floats); use exodus_layer_lif_forward / exodus_layer_lif_backward with "
                "caller-allocated checkpoints";
+    if (status == EXODUS_ERROR_REGIONS_NOT_FOUND)
+        return "timed copies between chunks of device memory did not show three kinds of chunks with a clear gap "
+               "between them: this device's memory has no regions to sort tensors by, or something else was "
+               "using it during the measurement";
     return hipGetErrorString(static_cast<hipError_t>(status));
 }
 

@@ -16,12 +16,14 @@ from typing import Optional
 
 import torch  # must be imported before the library so both share one HIP runtime
 
+from . import hbm
+
 _HERE = os.path.dirname(os.path.abspath(__file__))
 # EXODUS_HIP_LIBRARY may point at another build of the same ABI (e.g. one compiled with other flags)
 LIB_PATH = os.environ.get("EXODUS_HIP_LIBRARY") or os.path.join(_HERE, "libexodus_hip.so")
 
 SURR_TENSOR, SURR_SINGLE_EXP, SURR_PERIODIC_EXP, SURR_HEAVISIDE = 0, 1, 2, 3
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 _p = ctypes.c_void_p
 _i64 = ctypes.c_int64
@@ -50,6 +52,8 @@ _SIGNATURES = {
     "exodus_layer_lif_backward_from_input": ([_p] * 16 + [_int, _int, _int, _int, _int, _f, _f, _p, _p, _p, _i64, _i64, _i64, _p], _int),
     "exodus_layer_leaky_forward": ([_p] * 6 + [_int, _int, _i64, _i64, _i64, _p], _int),
     "exodus_layer_leaky_backward": ([_p] * 9 + [_int, _int, _i64, _i64, _i64, _p], _int),
+    "exodus_hbm_regions_create": ([_int, ctypes.c_uint64, ctypes.c_uint64, _p], _int),
+    "exodus_hbm_regions_destroy": ([_int], _int),
 }
 
 
@@ -182,15 +186,15 @@ def lifBackwardAlpha(surr, outputGrad, vmemPost, vmemPostInitial, notClipped, al
     return alphaGrad
 
 
-def leakyForward(input, vmemInitial, alpha) -> torch.Tensor:
-    """reference cuda/bindings.cu:163-193."""
+def leakyForward(input, vmemInitial, alpha, *, output=None) -> torch.Tensor:
+    """reference cuda/bindings.cu:163-193.  ``output`` (not in the reference) is a preallocated result."""
     _dev(input, "input")
     if input.ndim != 2:
         raise RuntimeError("input must be 2-D (rows, time)")
     n, t = input.shape
     _rows(_dev(vmemInitial, "vmemInitial", input), "vmemInitial", n)
     _rows(_dev(alpha, "alpha", input), "alpha", n)
-    out = torch.empty_like(input)
+    out = torch.empty_like(input) if output is None else _mat(_dev(output, "output", input), "output", n, t)
     with torch.cuda.device(input.device):
         _check(lib.exodus_leaky_forward(_ptr(out), _ptr(input), _ptr(vmemInitial), _ptr(alpha), n, t,
                                         _stream(input)), "exodus_leaky_forward")
@@ -445,11 +449,13 @@ def layerLifForward(input, vmemPostInitial, isynInitial, alphaMem, alphaSyn, mem
         _rows(_dev(thetaLow, "thetaLow", input), "thetaLow", n)
     else:
         thetaLow = None
-    spikes = torch.empty_like(input) if outSpikes is None else outSpikes
+    # big outputs go where hbm.enable() wants them (another region of HBM than what the kernel reads)
+    spikes = hbm.empty_like(input) if outSpikes is None else outSpikes
     if spikes.shape != input.shape:
         raise RuntimeError("outSpikes must have the shape of input")
     _dev(spikes, "outSpikes", input)
-    new = lambda *shape: torch.empty(shape, dtype=torch.float32, device=input.device)
+    new = lambda *shape: (hbm.empty(shape, input, away_from=[input, spikes]) if len(shape) == 3
+                          else torch.empty(shape, dtype=torch.float32, device=input.device))
     n_ck = (t + checkpointInterval() - 1) // checkpointInterval()
     state_shape = (n,) if stateShape is None else tuple(stateShape)
     if math.prod(state_shape) != n:
@@ -519,7 +525,7 @@ def layerLifBackward(gradSpikes, gradVLast, gradILast, input, ckptV, ckptI, vmem
     else:
         thetaLow = None
     if gradInput is None:
-        gradInput = torch.empty_like(input)
+        gradInput = hbm.empty_like(input, away_from=[input, gradSpikes])
     elif _btm(gradInput, "gradInput", input).shape != input.shape:
         raise RuntimeError("gradInput must have the shape of input")
     if surrogateKind == SURR_TENSOR:
@@ -578,7 +584,7 @@ def layerLeakyForward(input, vmemInitial, alpha, decayEarly: bool, normInput: bo
     state_shape = (n,) if stateShape is None else tuple(stateShape)
     if math.prod(state_shape) != n:
         raise RuntimeError(f"stateShape {state_shape} does not hold {n} neurons")
-    out = torch.empty_like(input)
+    out = hbm.empty_like(input)
     v_last = torch.empty(state_shape, dtype=torch.float32, device=input.device)
     out_sum = torch.zeros((), dtype=torch.float64, device=input.device) if wantSum else None
     if t == 0:
@@ -606,7 +612,7 @@ def layerLeakyBackward(gradOut, gradVLast, out, input, vmemInitial, alpha, decay
         _rows(_dev(vmemInitial, "vmemInitial", gradOut), "vmemInitial", n)
     if need_x and _btm(input, "input", gradOut).shape != gradOut.shape:
         raise RuntimeError("input must have the shape of gradOut")
-    grad_input = torch.empty_like(gradOut)
+    grad_input = hbm.empty_like(gradOut, away_from=[gradOut, out if needAlphaGrad else None, input if need_x else None])
     alpha_grad = torch.zeros(n, dtype=torch.float32, device=gradOut.device) if needAlphaGrad else None
     v_init_grad = torch.zeros(n, dtype=torch.float32, device=gradOut.device)
     if t == 0 and gradVLast is not None:
