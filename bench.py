@@ -71,18 +71,19 @@ class Placement:
     range cannot hold them, and for the checkpoints -- the third, so that no kernel writes into the region it
     reads most from; without, everything comes from torch's ordinary allocator."""
 
-    def __init__(self, torch, dev, regions=None):
-        self.torch, self.dev, self.regions = torch, dev, regions
+    def __init__(self, torch, dev, regions=None, one_region=False):
+        self.torch, self.dev, self.regions, self.one_region = torch, dev, regions, one_region
 
     def empty(self, shape, k):
         if self.regions is None:
             return self.torch.empty(tuple(shape), device=self.dev)
-        return self.regions.empty(shape, region=k)
+        return self.regions.empty(shape, region=0 if self.one_region else k)
 
     def describe(self):
         if self.regions is None:
             return {"placement": "ordinary allocator"}
-        return {"placement": "hbm regions (sinabs.exodus.hbm): inputs in one region of HBM, outputs in another, "
+        return {"placement": "all big tensors in ONE region of HBM (the control experiment)" if self.one_region else
+                             "hbm regions (sinabs.exodus.hbm): inputs in one region of HBM, outputs in another, "
                              "checkpoints in the third",
                 "placement_verified_by_timed_copies": self.regions.verified,
                 "placement_measured": {k: ([round(x) for x in v] if isinstance(v, list) else round(v))
@@ -601,12 +602,13 @@ def main():
                          "layer API (Conv2d -> IAFSqueeze -> AvgPool -> Conv2d -> IAFSqueeze -> Flatten -> Linear -> "
                          "IAFSqueeze, batch 64 x 300 steps, cross-entropy on spike counts): layer-layout kernels, the "
                          "transposing (rows, time) Functions, and the convolution / pooling / linear layers alone")
-    ap.add_argument("--placement", default="regions", choices=["regions", "plain"],
+    ap.add_argument("--placement", default="regions", choices=["regions", "one-region", "plain"],
                     help="regions (default): allocate through sinabs.exodus.hbm -- three ranges of device memory, each made "
                          "of one of the three regions of this GPU's HBM; inputs in the first, what the kernels write in the others.  A kernel that "
                          "reads one third and writes another moves 8-12 %% more bytes per second than one that does both "
-                         "inside one third, which is what a process gets from the ordinary allocator.  plain: the ordinary "
-                         "allocator.  The default run reports both (roofline.frac_by_placement); the plain figure is "
+                         "inside one third, which is what a process gets from the ordinary allocator on a machine that has run "
+                         "little.  one-region: the control -- the same sorted memory, every big tensor in the first range.  "
+                         "plain: the ordinary allocator.  The default run reports both (roofline.frac_by_placement); the plain figure is "
                          "measured first, in a child process, before this process touches the GPU")
     ap.add_argument("--region-map", type=float, nargs="?", const=4.0, default=0.0, metavar="GIB",
                     help="instead of the benchmark, fill device memory with buffers of GIB (default 4) GiB in the order "
@@ -675,10 +677,14 @@ def main():
         measure_reallocations(args, torch, hip, act, dev)
         return
     place = Placement(torch, dev)
-    if args.placement == "regions" and not (args.ceilings or args.conv_snn):
+    if args.placement != "plain" and not (args.ceilings or args.conv_snn):
         from sinabs.exodus import hbm
         try:
-            place = Placement(torch, dev, hbm.enable(gib_per_region=32.0, device=dev))
+            if args.placement == "one-region":
+                # the wrappers' own choices (checkpoints) stay off: they would move tensors out of the region
+                place = Placement(torch, dev, hbm.HbmRegions(gib_per_region=40.0, device=dev), one_region=True)
+            else:
+                place = Placement(torch, dev, hbm.enable(gib_per_region=32.0, device=dev))
         except RuntimeError as err:                     # device memory in use by something else: measure without
             plain_note = f"regions unavailable ({err}); ordinary allocator used"
             print("[bench] " + plain_note, file=sys.stderr, flush=True)

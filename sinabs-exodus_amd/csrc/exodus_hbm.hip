@@ -188,25 +188,51 @@ int create(int device, uint64_t bytes_per_region, uint64_t chunk_bytes, exodus_h
             all.push_back(pair[a][b]);
         }
     const float threshold = two_group_threshold(all);
-    // two probes are of one kind if they agree about most of the others (one noisy pair does not join kinds)
+    // Groups of probes: every probe starts as a group of its own, and the two groups with the slowest mean copy
+    // rate between them are joined until three are left (single pairs scatter by a few percent around the two
+    // typical rates; means over all pairs of two groups do not).  Whether the three are real is checked below.
     int kind[PROBES];
-    int kinds = 0;
-    int leader[PROBES];
-    for (int a = 0; a < PROBES; ++a) {
-        kind[a] = -1;
-        for (int k = 0; k < kinds && kind[a] < 0; ++k) {
-            const int b = leader[k];
-            int agree = 0, seen = 0;
-            for (int c = 0; c < PROBES; ++c)
-                if (c != a && c != b) { ++seen; agree += (pair[a][c] < threshold) == (pair[b][c] < threshold); }
-            if (agree * 10 >= seen * 7) kind[a] = k;
-        }
-        if (kind[a] < 0) {
-            if (kinds == PROBES) break;
-            leader[kinds] = a;
-            kind[a] = kinds++;
-        }
+    for (int a = 0; a < PROBES; ++a) kind[a] = a;
+    for (int groups = PROBES; groups > REGIONS; --groups) {
+        int best_a = -1, best_b = -1;
+        float best = 1e30f;
+        for (int ga = 0; ga < PROBES; ++ga)
+            for (int gb = 0; gb < ga; ++gb) {
+                double sum = 0;
+                int cnt = 0;
+                for (int a = 0; a < PROBES; ++a)
+                    for (int b = 0; b < PROBES; ++b)
+                        if (kind[a] == ga && kind[b] == gb) { sum += pair[a][b]; ++cnt; }
+                if (cnt && sum / cnt < best) { best = static_cast<float>(sum / cnt); best_a = ga; best_b = gb; }
+            }
+        for (int a = 0; a < PROBES; ++a)
+            if (kind[a] == best_a) kind[a] = best_b;
     }
+    // number the groups by their first probe: on a machine that has run little, region 0 is where the first
+    // ordinary allocations of a process lie
+    {
+        int label[PROBES], next = 0;
+        for (int a = 0; a < PROBES; ++a) label[a] = -1;
+        for (int a = 0; a < PROBES; ++a) {
+            if (label[kind[a]] < 0) label[kind[a]] = next++;
+        }
+        for (int a = 0; a < PROBES; ++a) kind[a] = label[kind[a]];
+    }
+    // real groups: between every two of them copies are clearly faster than inside either
+    int kinds = REGIONS;
+    for (int ga = 0; ga < REGIONS; ++ga)
+        for (int gb = 0; gb < ga; ++gb) {
+            double in_sum = 0, out_sum = 0;
+            int in_n = 0, out_n = 0;
+            for (int a = 0; a < PROBES; ++a)
+                for (int b = 0; b < a; ++b) {
+                    const bool a_in = kind[a] == ga || kind[a] == gb, b_in = kind[b] == ga || kind[b] == gb;
+                    if (!a_in || !b_in) continue;
+                    if (kind[a] == kind[b]) { in_sum += pair[a][b]; ++in_n; } else { out_sum += pair[a][b]; ++out_n; }
+                }
+            // (a group of one probe has no pair inside; the other group's pairs stand for both)
+            if (in_n == 0 || out_n == 0 || out_sum / out_n < 1.025 * (in_sum / in_n)) kinds = REGIONS - 1;
+        }
     for (int a = 0; a < PROBES; ++a) {
         rep->probe_chunk[a] = static_cast<int32_t>(probe[a]);
         rep->probe_kind[a] = kind[a];
@@ -230,12 +256,14 @@ int create(int device, uint64_t bytes_per_region, uint64_t chunk_bytes, exodus_h
     rep->probe_other_kind_GBs = fast_sum / fast_n;
     if (rep->probe_other_kind_GBs < 1.025f * rep->probe_same_kind_GBs) return EXODUS_ERROR_REGIONS_NOT_FOUND;
 
-    // 2. every chunk against two probes of each kind (where a kind has two): the kind it copies to slowest
-    int refs[REGIONS][2];
+    // 2. every chunk against up to three probes of each kind: the kind it copies to slowest
+    constexpr int REFS = 3;
+    int refs[REGIONS][REFS];
     for (int k = 0; k < REGIONS; ++k) {
-        refs[k][0] = refs[k][1] = -1;
-        for (int a = 0; a < PROBES; ++a)
-            if (kind[a] == k) { if (refs[k][0] < 0) refs[k][0] = a; else if (refs[k][1] < 0) refs[k][1] = a; }
+        int cnt = 0;
+        for (int r = 0; r < REFS; ++r) refs[k][r] = -1;
+        for (int a = 0; a < PROBES && cnt < REFS; ++a)
+            if (kind[a] == k) refs[k][cnt++] = a;
     }
     std::vector<int> kind_of(n, -1);
     for (int a = 0; a < PROBES; ++a) kind_of[probe[a]] = kind[a];
@@ -249,7 +277,7 @@ int create(int device, uint64_t bytes_per_region, uint64_t chunk_bytes, exodus_h
         for (int k = 0; k < REGIONS; ++k) {
             float sum = 0.f;
             int cnt = 0;
-            for (int r = 0; r < 2; ++r)
+            for (int r = 0; r < REFS; ++r)
                 if (refs[k][r] >= 0) {
                     float v = 0.f;
                     HBM_TRY(s.rate(s.at(probe[refs[k][r]]), s.at(i), chunk, 2, &v));
