@@ -71,8 +71,9 @@ class Placement:
     range cannot hold them, and for the checkpoints -- the third, so that no kernel writes into the region it
     reads most from; without, everything comes from torch's ordinary allocator."""
 
-    def __init__(self, torch, dev, regions=None, one_region=False):
+    def __init__(self, torch, dev, regions=None, one_region=False, assign=(0, 0, 1, 1)):
         self.torch, self.dev, self.regions, self.one_region = torch, dev, regions, one_region
+        self.assign = assign        # layer workloads: region of input, grad_output, spikes, grad_input
 
     def empty(self, shape, k):
         if self.regions is None:
@@ -84,7 +85,9 @@ class Placement:
             return {"placement": "ordinary allocator"}
         return {"placement": "all big tensors in ONE region of HBM (the control experiment)" if self.one_region else
                              "hbm regions (sinabs.exodus.hbm): inputs in one region of HBM, outputs in another, "
-                             "checkpoints in the third",
+                             "checkpoints in the third" if self.assign == (0, 0, 1, 1) else
+                             "hbm regions, layer tensors (input, grad_output, spikes, grad_input) in regions "
+                             f"{self.assign}",
                 "placement_verified_by_timed_copies": self.regions.verified,
                 "placement_measured": {k: ([round(x) for x in v] if isinstance(v, list) else round(v))
                                        for k, v in self.regions.report.items()}}
@@ -100,14 +103,15 @@ def build_layer_workload(key, torch, hip, act, dev, place=None):
     B, T, M = w["batch"], w["steps"], w["neurons"]
     N = B * M
     g = torch.Generator(device=dev).manual_seed(list(WORKLOADS).index(key))
-    x = place.empty((B, T, M), 0)
+    rx, rgo, rs, rgi = place.assign
+    x = place.empty((B, T, M), rx)
     x.uniform_(0.0, 0.5, generator=g) if key == "c1" else x.normal_(w["mean"], w["std"], generator=g)
-    go = place.empty((B, T, M), 0).fill_(1.0)
+    go = place.empty((B, T, M), rgo).fill_(1.0)
     rows = lambda v: torch.as_tensor(v, dtype=torch.float32, device=dev).expand(B, M).flatten().contiguous()
     zeros = torch.zeros(N, device=dev); ones = torch.ones(N, device=dev)
     surr = act.SingleExponential()
     kind, p0, p1 = hip.SURR_SINGLE_EXP, surr.grad_width, surr.grad_scale
-    spikes = place.empty(x.shape, 1); gi = place.empty(x.shape, 1)
+    spikes = place.empty(x.shape, rs); gi = place.empty(x.shape, rgi)
     if key == "c5":
         cfg = dict(a_mem=rows(math.exp(-1 / 20.0)), a_syn=rows(math.exp(-1 / 5.0)), lo=rows(-1.0), cap=2, norm=True)
     elif key == "c2":
@@ -610,6 +614,10 @@ def main():
                          "little.  one-region: the control -- the same sorted memory, every big tensor in the first range.  "
                          "plain: the ordinary allocator.  The default run reports both (roofline.frac_by_placement); the plain figure is "
                          "measured first, in a child process, before this process touches the GPU")
+    ap.add_argument("--assign", default="0,0,1,1", metavar="X,GO,S,GI",
+                    help="with --placement regions and --path layer: the region (0, 1, 2) that the input, the incoming "
+                         "gradient, the spikes and the input gradient are allocated in (default 0,0,1,1: each kernel reads one "
+                         "region and writes another; the checkpoints go where the wrappers put them)")
     ap.add_argument("--region-map", type=float, nargs="?", const=4.0, default=0.0, metavar="GIB",
                     help="instead of the benchmark, fill device memory with buffers of GIB (default 4) GiB in the order "
                          "the driver hands them out, copy every buffer into every other with a flat copy kernel and print "
@@ -647,7 +655,8 @@ def main():
         sys.exit(subprocess.run([sys.executable, os.path.abspath(__file__)] + rest, env=env).returncode)
 
     plain_first, plain_note = None, None
-    special = args.region_map or args.reallocations or args.ceilings or args.conv_snn or args.shape or args.copy_probe
+    special = (args.region_map or args.reallocations or args.ceilings or args.conv_snn or args.shape or args.copy_probe
+               or args.assign != "0,0,1,1")
     if args.placement == "regions" and args.others and not special:
         # the same measurement with the ordinary allocator, in a process of its own and before this one touches
         # the GPU, so that it sees what a program that allocates without further thought is handed
@@ -684,7 +693,9 @@ def main():
                 # the wrappers' own choices (checkpoints) stay off: they would move tensors out of the region
                 place = Placement(torch, dev, hbm.HbmRegions(gib_per_region=40.0, device=dev), one_region=True)
             else:
-                place = Placement(torch, dev, hbm.enable(gib_per_region=32.0, device=dev))
+                assign = tuple(int(v) for v in args.assign.split(","))
+                assert len(assign) == 4 and all(0 <= v <= 2 for v in assign), "--assign takes four regions out of 0, 1, 2"
+                place = Placement(torch, dev, hbm.enable(gib_per_region=32.0, device=dev), assign=assign)
         except RuntimeError as err:                     # device memory in use by something else: measure without
             plain_note = f"regions unavailable ({err}); ordinary allocator used"
             print("[bench] " + plain_note, file=sys.stderr, flush=True)
