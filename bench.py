@@ -66,28 +66,39 @@ OTHERS = [("c2", "layer"), ("c3", "layer"), ("c5", "rows"), ("c2", "rows"), ("c3
 
 
 class Placement:
-    """Where a workload's tensors are allocated.  With ``regions`` (sinabs.exodus.hbm.HbmRegions) the inputs
-    (x, grad_output) go into the range made of the first kind of HBM, outputs into the second and -- where one
-    range cannot hold them, and for the checkpoints -- the third, so that no kernel writes into the region it
-    reads most from; without, everything comes from torch's ordinary allocator."""
+    """Where a workload's tensors are allocated (``mode``; ``regions`` = sinabs.exodus.hbm.HbmRegions):
+    striped      inputs (x, grad_output) in the range made of the first region of HBM, everything the kernels write
+                 in the striped range, whose 64 MiB pages alternate between the three regions
+    all-striped  every big tensor in the striped range
+    regions      every tensor in one region's range: inputs in the first, outputs in the second and -- where one
+                 range cannot hold them, and for the checkpoints -- the third
+    one-region   the control: every big tensor in the first region's range
+    plain        torch's ordinary allocator"""
 
-    def __init__(self, torch, dev, regions=None, one_region=False, assign=(0, 0, 1, 1)):
-        self.torch, self.dev, self.regions, self.one_region = torch, dev, regions, one_region
-        self.assign = assign        # layer workloads: region of input, grad_output, spikes, grad_input
+    def __init__(self, torch, dev, regions=None, mode="plain", assign=(0, 0, 1, 1)):
+        self.torch, self.dev, self.regions, self.mode = torch, dev, regions, mode
+        self.assign = assign        # mode "regions", layer workloads: region of input, grad_output, spikes, grad_input
 
     def empty(self, shape, k):
         if self.regions is None:
             return self.torch.empty(tuple(shape), device=self.dev)
-        return self.regions.empty(shape, region=0 if self.one_region else k)
+        if self.mode == "striped":
+            return self.regions.empty(shape, region=0 if k == 0 else 3)
+        if self.mode == "all-striped":
+            return self.regions.empty(shape, region=3)
+        return self.regions.empty(shape, region=0 if self.mode == "one-region" else k)
 
     def describe(self):
         if self.regions is None:
             return {"placement": "ordinary allocator"}
-        return {"placement": "all big tensors in ONE region of HBM (the control experiment)" if self.one_region else
-                             "hbm regions (sinabs.exodus.hbm): inputs in one region of HBM, outputs in another, "
-                             "checkpoints in the third" if self.assign == (0, 0, 1, 1) else
-                             "hbm regions, layer tensors (input, grad_output, spikes, grad_input) in regions "
-                             f"{self.assign}",
+        text = {"striped": "hbm regions (sinabs.exodus.hbm): inputs in one region of HBM, everything the kernels write in "
+                           "memory whose 64 MiB pages alternate between the three regions",
+                "all-striped": "every big tensor in memory whose 64 MiB pages alternate between the three regions of HBM",
+                "one-region": "all big tensors in ONE region of HBM (the control experiment)",
+                "regions": "hbm regions, one region per tensor: inputs in the first, outputs in the second, checkpoints in "
+                           "the third" if self.assign == (0, 0, 1, 1) else
+                           f"hbm regions, layer tensors (input, grad_output, spikes, grad_input) in regions {self.assign}"}
+        return {"placement": text[self.mode],
                 "placement_verified_by_timed_copies": self.regions.verified,
                 "placement_measured": {k: ([round(x) for x in v] if isinstance(v, list) else round(v))
                                        for k, v in self.regions.report.items()}}
@@ -103,7 +114,7 @@ def build_layer_workload(key, torch, hip, act, dev, place=None):
     B, T, M = w["batch"], w["steps"], w["neurons"]
     N = B * M
     g = torch.Generator(device=dev).manual_seed(list(WORKLOADS).index(key))
-    rx, rgo, rs, rgi = place.assign
+    rx, rgo, rs, rgi = place.assign if place.mode == "regions" else (0, 0, 1, 1)
     x = place.empty((B, T, M), rx)
     x.uniform_(0.0, 0.5, generator=g) if key == "c1" else x.normal_(w["mean"], w["std"], generator=g)
     go = place.empty((B, T, M), rgo).fill_(1.0)
@@ -606,14 +617,17 @@ def main():
                          "layer API (Conv2d -> IAFSqueeze -> AvgPool -> Conv2d -> IAFSqueeze -> Flatten -> Linear -> "
                          "IAFSqueeze, batch 64 x 300 steps, cross-entropy on spike counts): layer-layout kernels, the "
                          "transposing (rows, time) Functions, and the convolution / pooling / linear layers alone")
-    ap.add_argument("--placement", default="regions", choices=["regions", "one-region", "plain"],
-                    help="regions (default): allocate through sinabs.exodus.hbm -- three ranges of device memory, each made "
-                         "of one of the three regions of this GPU's HBM; inputs in the first, what the kernels write in the others.  A kernel that "
-                         "reads one third and writes another moves 8-12 %% more bytes per second than one that does both "
-                         "inside one third, which is what a process gets from the ordinary allocator on a machine that has run "
-                         "little.  one-region: the control -- the same sorted memory, every big tensor in the first range.  "
-                         "plain: the ordinary allocator.  The default run reports both (roofline.frac_by_placement); the plain figure is "
-                         "measured first, in a child process, before this process touches the GPU")
+    ap.add_argument("--placement", default="striped", choices=["striped", "all-striped", "regions", "one-region", "plain"],
+                    help="striped (default): allocate through sinabs.exodus.hbm, which sorts device memory by the three "
+                         "regions of this GPU's HBM -- inputs in the first region's range, everything the kernels write in the "
+                         "striped range, whose 64 MiB pages alternate between the regions (a kernel's writes are held back by "
+                         "the region they go to; spread over all three they are not).  all-striped: every big tensor in the "
+                         "striped range -- what a program gets that allocates everything there without further thought.  "
+                         "regions: one region per tensor (inputs in the first, outputs in the others; see --assign).  "
+                         "one-region: the control -- the same sorted memory, every big tensor in the first region.  "
+                         "plain: the ordinary allocator.  The default run reports striped, all-striped and plain "
+                         "(roofline.frac_by_placement); the plain figure is measured first, in a child process, before this "
+                         "process touches the GPU")
     ap.add_argument("--assign", default="0,0,1,1", metavar="X,GO,S,GI",
                     help="with --placement regions and --path layer: the region (0, 1, 2) that the input, the incoming "
                          "gradient, the spikes and the input gradient are allocated in (default 0,0,1,1: each kernel reads one "
@@ -657,20 +671,27 @@ def main():
     plain_first, plain_note = None, None
     special = (args.region_map or args.reallocations or args.ceilings or args.conv_snn or args.shape or args.copy_probe
                or args.assign != "0,0,1,1")
-    if args.placement == "regions" and args.others and not special:
+    if args.placement == "striped" and args.others and not special:
         # the same measurement with the ordinary allocator, in a process of its own and before this one touches
-        # the GPU, so that it sees what a program that allocates without further thought is handed
+        # the GPU, so that it sees what a program that allocates without further thought is handed; then with
+        # every tensor in the striped range
         import subprocess
-        child = subprocess.run([sys.executable, os.path.abspath(__file__), "--placement", "plain", "--no-others",
-                                "--no-cpu-baseline", "--workload", args.workload, "--path", args.path,
-                                "--steps", str(args.steps), "--warmup", str(args.warmup)],
-                               capture_output=True, text=True)
-        try:
-            r = json.loads(child.stdout.strip().splitlines()[-1])["roofline"]
-            plain_first = {"frac": r["frac"], "fwd_bwd_combined_frac": r["fwd_bwd_combined_frac"],
-                           "kernel_ms": r["kernel_ms"], "other_kernel_ms": r["other_kernel"]["kernel_ms"]}
-        except (IndexError, KeyError, ValueError):
-            plain_first = {"error": (child.stderr or child.stdout)[-400:]}
+
+        def child_run(placement):
+            child = subprocess.run([sys.executable, os.path.abspath(__file__), "--placement", placement, "--no-others",
+                                    "--no-cpu-baseline", "--workload", args.workload, "--path", args.path,
+                                    "--steps", str(args.steps), "--warmup", str(args.warmup)],
+                                   capture_output=True, text=True)
+            try:
+                r = json.loads(child.stdout.strip().splitlines()[-1])["roofline"]
+                return {"frac": r["frac"], "fwd_bwd_combined_frac": r["fwd_bwd_combined_frac"],
+                        "kernel_ms": r["kernel_ms"], "other_kernel_ms": r["other_kernel"]["kernel_ms"]}
+            except (IndexError, KeyError, ValueError):
+                return {"error": (child.stderr or child.stdout)[-400:]}
+
+        plain_first = child_run("plain")
+        # (the all-striped figure is measured last, after this process has given its memory back: a process that
+        # has allocated device memory in pages leaves it to the next one as a mixture of the regions)
 
     import torch
     assert torch.cuda.is_available(), "bench.py needs the GPU"
@@ -691,11 +712,29 @@ def main():
         try:
             if args.placement == "one-region":
                 # the wrappers' own choices (checkpoints) stay off: they would move tensors out of the region
-                place = Placement(torch, dev, hbm.HbmRegions(gib_per_region=40.0, device=dev), one_region=True)
-            else:
+                place = Placement(torch, dev, hbm.HbmRegions(gib_per_region=40.0, gib_striped=0.0, device=dev),
+                                  mode="one-region")
+            elif args.placement == "regions":
                 assign = tuple(int(v) for v in args.assign.split(","))
                 assert len(assign) == 4 and all(0 <= v <= 2 for v in assign), "--assign takes four regions out of 0, 1, 2"
-                place = Placement(torch, dev, hbm.enable(gib_per_region=32.0, device=dev), assign=assign)
+                place = Placement(torch, dev, hbm.enable(gib_per_region=32.0, gib_striped=0.0, device=dev),
+                                  mode="regions", assign=assign)
+            elif args.placement == "all-striped":
+                place = Placement(torch, dev, hbm.enable(gib_per_region=0.0, gib_striped=72.0, device=dev),
+                                  mode="all-striped")
+            else:
+                try:
+                    place = Placement(torch, dev, hbm.enable(gib_per_region=24.0, gib_striped=48.0, device=dev),
+                                      mode="striped")
+                except RuntimeError as err:
+                    if "did not show three kinds" not in str(err):
+                        raise
+                    # memory that earlier processes left as a mixture of the regions: no region to put the inputs
+                    # in; everything goes into the striped range, made of that memory as it is
+                    plain_note = "no regions found in device memory (earlier processes left it mixed): all-striped used"
+                    print("[bench] " + plain_note, file=sys.stderr, flush=True)
+                    place = Placement(torch, dev, hbm.enable(gib_per_region=0.0, gib_striped=72.0, device=dev),
+                                      mode="all-striped")
         except RuntimeError as err:                     # device memory in use by something else: measure without
             plain_note = f"regions unavailable ({err}); ordinary allocator used"
             print("[bench] " + plain_note, file=sys.stderr, flush=True)
@@ -750,7 +789,8 @@ def main():
     }
     if plain_first is not None:
         roof["frac_by_placement"] = {
-            "regions (this run's figures)": {"frac": roof["frac"], "fwd_bwd_combined_frac": roof["fwd_bwd_combined_frac"]},
+            "striped: inputs in one region, outputs striped over the three (this run's figures)":
+                {"frac": roof["frac"], "fwd_bwd_combined_frac": roof["fwd_bwd_combined_frac"]},
             "ordinary allocator, first allocations of a process (measured before this one touched the GPU)": plain_first}
     if args.others and not args.shape:
         # the other configurations and the (rows, time) kernels behind the autograd Functions, a few
@@ -774,6 +814,17 @@ def main():
         result["config"]["placement_note"] = plain_note
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(args.workload, torch)
+    if plain_first is not None:
+        # every tensor in the striped range, in a process of its own, once this one has given its memory back
+        wl = fwd = bwd = place = None
+        if args.placement != "plain":
+            hbm.disable()
+        import gc
+        gc.collect()
+        torch.cuda.empty_cache()
+        torch.cuda.synchronize()
+        roof["frac_by_placement"]["all-striped: every tensor striped over the three regions "
+                                  "(measured last, in a process of its own)"] = child_run("all-striped")
     print(json.dumps(result))
 
 

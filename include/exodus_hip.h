@@ -29,7 +29,7 @@ extern "C" {
 #endif
 
 /* ABI version of this header; bumped on any signature change. */
-#define EXODUS_HIP_ABI_VERSION 6
+#define EXODUS_HIP_ABI_VERSION 7
 
 int exodus_hip_abi_version(void);
 const char *exodus_hip_error_string(int status);
@@ -288,24 +288,33 @@ int exodus_spike_backward(float *input_grad, const float *surr, const float *out
  * placement of its tensors to torch's allocator, reference cuda/bindings.cu:98,144,183)
  * ------------------------------------------------------------------------------------------- */
 
-/* The HBM of an MI355X behaves as three regions: a kernel that reads one and writes another moves
- * 8-12 % more bytes per second than one that reads and writes inside one region.
- * exodus_hbm_regions_create takes nearly all free device memory in chunks of chunk_bytes (a multiple
- * of the allocation granularity and of 16 KiB; 4 GiB is a good value: copies of less tell the regions apart less clearly), finds by timed copies which
- * chunks lie in one region, maps ceil(bytes_per_region / chunk_bytes) chunks of each region behind
- * each other into an address range of its own and returns the rest to the driver.  report->base[k] /
- * bytes[k] are the three ranges; the caller hands out memory from them as it likes (the Python host
- * side is sinabs/exodus/hbm.py) and must stop using them before exodus_hbm_regions_destroy.
- * Returns EXODUS_ERROR_REGIONS_NOT_FOUND when the copies do not show three kinds of chunks with a
- * clear gap (the report's fields up to kinds_found are then filled), hipErrorOutOfMemory when too
- * little memory is free to find or fill three regions, hipErrorInvalidValue for bad arguments or a
- * device that already has its ranges.  Takes a second or two; synchronises the device. */
+/* The HBM of an MI355X behaves as three regions.  A kernel's writes are held back by the region they go to: the
+ * layer kernels write at 5.6 TB/s into one region and at 6.0-6.3 TB/s into memory whose 64 MiB pages alternate
+ * between the regions; a kernel that reads one region and writes another moves 8-12 % more than one that does both
+ * inside one region.
+ * exodus_hbm_regions_create takes nearly all free device memory in chunks of chunk_bytes (a multiple of
+ * EXODUS_HBM_PAGE_BYTES; 4 GiB is a good value: copies of less tell the regions apart less clearly), finds by timed
+ * copies which chunks lie in one region, and builds four address ranges: ranges 0-2 hold
+ * ceil(bytes_per_region / chunk_bytes) chunks of one region each; range 3 (the striped one) holds bytes_striped,
+ * rounded up to a multiple of three chunks, in pages of EXODUS_HBM_PAGE_BYTES that come from chunks of regions 0, 1,
+ * 2, 0, 1, 2, ... in turn.  Either size may be 0 (that range is then absent, base NULL).  The rest goes back to the
+ * driver.  report->base[k] / bytes[k] are the ranges; the caller hands out memory from them as it likes (the Python
+ * host side is sinabs/exodus/hbm.py) and must stop using them before exodus_hbm_regions_destroy.
+ * When the copies do not show three kinds of chunks with a clear gap (memory that earlier processes allocated and
+ * freed in small pieces comes back as a mixture of the regions below the size of a chunk): with bytes_per_region > 0
+ * the call returns EXODUS_ERROR_REGIONS_NOT_FOUND (the report's fields up to kinds_found are then filled); with only
+ * a striped range asked for it succeeds with kinds_found < 3, the pages taking turns between chunks spread evenly
+ * over the memory instead.  hipErrorOutOfMemory when too little memory is free to find or fill the ranges,
+ * hipErrorInvalidValue for bad arguments or a device that already has its ranges.  Takes a second or two;
+ * synchronises the device. */
 #define EXODUS_HBM_REGIONS 3
+#define EXODUS_HBM_ARENAS 4                          /* one range per region, and the striped one */
+#define EXODUS_HBM_PAGE_BYTES (64ull << 20)          /* stripe width; 32-128 MiB measured alike, 8 and 512 MiB worse */
 #define EXODUS_HBM_PROBES 15
 typedef struct exodus_hbm_report {
-    void *base[EXODUS_HBM_REGIONS];
-    uint64_t bytes[EXODUS_HBM_REGIONS];
-    uint64_t chunk_bytes;
+    void *base[EXODUS_HBM_ARENAS];
+    uint64_t bytes[EXODUS_HBM_ARENAS];
+    uint64_t chunk_bytes, page_bytes;
     int32_t chunks_examined;                         /* physical chunks taken for sorting */
     int32_t kinds_found;                             /* groups among the probe chunks; 3 on success */
     int32_t chunks_ambiguous;                        /* chunks that matched no region clearly (not used) */
@@ -314,11 +323,12 @@ typedef struct exodus_hbm_report {
     float probe_same_kind_GBs, probe_other_kind_GBs; /* mean copy rate between probe chunks of one / of two regions */
     float copy_inside_GBs[EXODUS_HBM_REGIONS];       /* finished ranges: first half of range k into its second half */
     float copy_across_GBs[6];                        /* range j into range k: (0,1) (0,2) (1,0) (1,2) (2,0) (2,1) */
+    float copy_striped_GBs;                          /* first half of the striped range into its second half */
     int32_t probe_chunk[EXODUS_HBM_PROBES];          /* the probe chunks (position in the order of creation), */
     int32_t probe_kind[EXODUS_HBM_PROBES];           /* the group each was put in, and the copy rate between every */
     float probe_pair_GBs[EXODUS_HBM_PROBES][EXODUS_HBM_PROBES];   /* two of them (mean of both directions) */
 } exodus_hbm_report;
-int exodus_hbm_regions_create(int device, uint64_t bytes_per_region, uint64_t chunk_bytes,
+int exodus_hbm_regions_create(int device, uint64_t bytes_per_region, uint64_t bytes_striped, uint64_t chunk_bytes,
                               exodus_hbm_report *report);
 int exodus_hbm_regions_destroy(int device);
 

@@ -21,6 +21,25 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));    // one 16-byte chunk
 #define EXODUS_TT_3 32    // three or more LDS slots
 #endif
 
+// The same for the driver that addresses a wave's rows as one span of memory, by LDS tiles per wave.
+#ifndef EXODUS_TT_S1
+#define EXODUS_TT_S1 32
+#endif
+#ifndef EXODUS_TT_S2
+#define EXODUS_TT_S2 32
+#endif
+#ifndef EXODUS_TT_S3
+#define EXODUS_TT_S3 32
+#endif
+// most waves per SIMD the span driver's register budget is set for, and how many 4-step chunks of a
+// tile its recurrence loop is unrolled by
+#ifndef EXODUS_WPE_MAX
+#define EXODUS_WPE_MAX 4
+#endif
+#ifndef EXODUS_SPAN_UNROLL_Q
+#define EXODUS_SPAN_UNROLL_Q 2
+#endif
+
 // Unroll factor of the per-tile chunk loop (each chunk = 4 time steps).  Full unrolling lets the
 // compiler hoist every LDS read of the tile, which costs registers and therefore resident waves.
 #ifndef EXODUS_UNROLL_Q

@@ -10,7 +10,19 @@
 // chunks of one kind behind each other into three address ranges ("arenas").  What is left over goes
 // back to the driver.  The host side (sinabs/exodus/hbm.py) hands out tensors from the arenas.
 //
-//   exodus_hbm_regions_create(device, bytes_per_region, chunk_bytes, &report)
+// What costs most is writing: a kernel whose output lies in one region is held back by that region
+// alone (the time-strided layer kernels write at 5.6 TB/s into one region; the (rows, time) kernels,
+// which write single 128-byte lines, at 4.4-4.9), while the same kernel writing into memory whose pages
+// alternate between the regions reaches 6.0-6.3 and 5.6-5.8 TB/s.  A fourth arena is therefore made of
+// 64 MiB pages taken from the three regions in turn ("striped"): any tensor of a few hundred MiB in it
+// spreads over all of them.  Stripes of 32 to 128 MiB measured alike; 8 MiB and 512 MiB measured worse.
+// A mapping cannot start inside an allocation, so the pages have to be allocations of their own, and
+// pages allocated one after the other are neighbours in physical memory only on a machine whose memory
+// has never been handed out in pages before.  The pages of a known region are therefore made from a
+// sorted chunk: with all other free memory held, the chunk is released and 64 pages are allocated at
+// once, which can only come from the hole it left.
+//
+//   exodus_hbm_regions_create(device, bytes_per_region, bytes_striped, chunk_bytes, &report)
 //   exodus_hbm_regions_destroy(device)
 //
 // Both calls synchronise the device.  One set of arenas per device; creating a second one fails with
@@ -30,6 +42,9 @@
 namespace {
 
 constexpr int REGIONS = EXODUS_HBM_REGIONS;
+constexpr int ARENAS = EXODUS_HBM_ARENAS;   // one per region and the striped one
+constexpr int STRIPED = REGIONS;
+constexpr size_t PAGE = EXODUS_HBM_PAGE_BYTES;
 constexpr int MAX_DEVICES = 64;
 constexpr int PROBES = EXODUS_HBM_PROBES;   // chunks whose pairwise copy rates are measured to find the kinds
 constexpr int COPY_PER_THREAD = 4;
@@ -49,10 +64,38 @@ __global__ void __launch_bounds__(256) region_copy(f32x4 *__restrict__ dst, cons
 
 struct Arenas {
     bool live = false;
-    size_t chunk = 0;
-    void *base[REGIONS] = {nullptr, nullptr, nullptr};
-    size_t reserved[REGIONS] = {0, 0, 0};
-    std::vector<hipMemGenericAllocationHandle_t> handles[REGIONS];
+    void *base[ARENAS] = {nullptr, nullptr, nullptr, nullptr};
+    size_t reserved[ARENAS] = {0, 0, 0, 0};
+    size_t unit[ARENAS] = {0, 0, 0, 0};     // bytes per allocation: a chunk in the regions' arenas, a page in the striped one
+    std::vector<hipMemGenericAllocationHandle_t> handles[ARENAS];   // allocation j is mapped at base + j * unit
+
+    // unmaps and releases everything; returns the first error
+    hipError_t release()
+    {
+        hipError_t status = hipSuccess;
+        for (int k = 0; k < ARENAS; ++k) {
+            for (size_t j = 0; j < handles[k].size(); ++j) {
+                const hipError_t u = hipMemUnmap(static_cast<char *>(base[k]) + j * unit[k], unit[k]);
+                const hipError_t r = hipMemRelease(handles[k][j]);
+                if (status == hipSuccess) status = u != hipSuccess ? u : r;
+            }
+            if (base[k]) {
+                const hipError_t f = hipMemAddressFree(base[k], reserved[k]);
+                if (status == hipSuccess) status = f;
+            }
+        }
+        *this = Arenas{};
+        return status;
+    }
+};
+
+// allocations that belong to nobody yet: released when the scope ends, unless moved on
+struct Loose {
+    std::vector<hipMemGenericAllocationHandle_t> handles;
+    ~Loose()
+    {
+        for (hipMemGenericAllocationHandle_t h : handles) (void)hipMemRelease(h);
+    }
 };
 
 std::mutex table_mutex;
@@ -129,7 +172,7 @@ float two_group_threshold(const std::vector<float> &v)
     return 0.5f * (lo + hi);
 }
 
-int create(int device, uint64_t bytes_per_region, uint64_t chunk_bytes, exodus_hbm_report *rep)
+int create(int device, uint64_t bytes_per_region, uint64_t bytes_striped, uint64_t chunk_bytes, exodus_hbm_report *rep)
 {
     HBM_TRY(hipSetDevice(device));
     HBM_TRY(hipDeviceSynchronize());
@@ -139,9 +182,13 @@ int create(int device, uint64_t bytes_per_region, uint64_t chunk_bytes, exodus_h
     prop.location.id = device;
     size_t gran = 0;
     HBM_TRY(hipMemGetAllocationGranularity(&gran, &prop, hipMemAllocationGranularityRecommended));
-    if (gran == 0 || chunk_bytes % gran != 0 || chunk_bytes % (16 * 256 * COPY_PER_THREAD) != 0) return hipErrorInvalidValue;
+    if (gran == 0 || PAGE % gran != 0 || chunk_bytes % PAGE != 0 || chunk_bytes % (16 * 256 * COPY_PER_THREAD) != 0)
+        return hipErrorInvalidValue;
     const size_t chunk = chunk_bytes;
-    const size_t need = (bytes_per_region + chunk - 1) / chunk;          // chunks per arena
+    const size_t ppc = chunk / PAGE;                                    // pages per chunk
+    const size_t need_pure = (bytes_per_region + chunk - 1) / chunk;    // chunks of each region for its own arena
+    const size_t need_striped = (bytes_striped + REGIONS * chunk - 1) / (REGIONS * chunk);   // ... for the striped one
+    const size_t need = need_pure + need_striped;                       // chunks wanted of each region
     size_t free_b = 0, total_b = 0;
     HBM_TRY(hipMemGetInfo(&free_b, &total_b));
     const size_t margin = size_t(6) << 30;                              // left to everybody else while sorting
@@ -242,7 +289,10 @@ int create(int device, uint64_t bytes_per_region, uint64_t chunk_bytes, exodus_h
     rep->chunks_examined = static_cast<int32_t>(n);
     rep->threshold_GBs = threshold;
     rep->kinds_found = kinds;
-    if (kinds != REGIONS) return EXODUS_ERROR_REGIONS_NOT_FOUND;
+    // Without three kinds there are no regions to sort by: then the memory the driver hands out is already a
+    // mixture at a scale below the chunks (after processes that allocated and freed it in small pieces), which
+    // is what the striped range wants to be; ranges of one region cannot be made.
+    bool sorted = kinds == REGIONS;
     // the gap between the two groups of rates has to be a real one
     float slow_max = 0.f, fast_min = 1e30f, slow_sum = 0.f, fast_sum = 0.f;
     int slow_n = 0, fast_n = 0;
@@ -251,10 +301,14 @@ int create(int device, uint64_t bytes_per_region, uint64_t chunk_bytes, exodus_h
             if (kind[a] == kind[b]) { slow_max = std::max(slow_max, pair[a][b]); slow_sum += pair[a][b]; ++slow_n; }
             else { fast_min = std::min(fast_min, pair[a][b]); fast_sum += pair[a][b]; ++fast_n; }
         }
-    if (slow_n == 0 || fast_n == 0) return EXODUS_ERROR_REGIONS_NOT_FOUND;
-    rep->probe_same_kind_GBs = slow_sum / slow_n;
-    rep->probe_other_kind_GBs = fast_sum / fast_n;
-    if (rep->probe_other_kind_GBs < 1.025f * rep->probe_same_kind_GBs) return EXODUS_ERROR_REGIONS_NOT_FOUND;
+    if (slow_n == 0 || fast_n == 0) sorted = false;
+    else {
+        rep->probe_same_kind_GBs = slow_sum / slow_n;
+        rep->probe_other_kind_GBs = fast_sum / fast_n;
+        if (rep->probe_other_kind_GBs < 1.025f * rep->probe_same_kind_GBs) sorted = false;
+    }
+    if (!sorted) rep->kinds_found = std::min(rep->kinds_found, REGIONS - 1);
+    if (!sorted && need_pure) return EXODUS_ERROR_REGIONS_NOT_FOUND;
 
     // 2. every chunk against up to three probes of each kind: the kind it copies to slowest
     constexpr int REFS = 3;
@@ -270,7 +324,7 @@ int create(int device, uint64_t bytes_per_region, uint64_t chunk_bytes, exodus_h
     int ambiguous = 0;
     size_t have[REGIONS] = {0, 0, 0};
     for (int a = 0; a < PROBES; ++a) ++have[kind[a]];
-    for (size_t i = 0; i < n; ++i) {
+    for (size_t i = 0; i < n && sorted; ++i) {
         if (kind_of[i] >= 0) continue;
         if (have[0] >= need && have[1] >= need && have[2] >= need) break;   // enough of every kind
         float mean[REGIONS];
@@ -294,22 +348,28 @@ int create(int device, uint64_t bytes_per_region, uint64_t chunk_bytes, exodus_h
     }
     rep->chunks_ambiguous = ambiguous;
     for (int k = 0; k < REGIONS; ++k) rep->chunks_of_region[k] = static_cast<int32_t>(have[k]);
-    if (have[0] < need || have[1] < need || have[2] < need) return hipErrorOutOfMemory;
+    if (sorted && (have[0] < need || have[1] < need || have[2] < need)) return hipErrorOutOfMemory;
 
-    // 3. the arenas: the first `need` chunks of each kind, behind each other in a range of their own.
+    // 3. the arenas.  Of the chunks of each kind, in the order of creation, the first need_pure go behind each other
+    // into the kind's own range and the next need_striped are turned into pages for the striped range.
     // Kinds are numbered by the position of their first chunk, so that a process that comes first on a
     // machine finds region 0 where its ordinary allocations lie.
     Arenas built;
-    built.chunk = chunk;
     HBM_TRY(hipDeviceSynchronize());
     int status = hipSuccess;
-    for (int k = 0; k < REGIONS && status == hipSuccess; ++k) {
+    std::vector<size_t> to_pages[REGIONS];                              // chunks that become pages, by kind
+    for (int k = 0; k < REGIONS && status == hipSuccess && sorted; ++k) {
         void *base = nullptr;
-        if ((status = hipMemAddressReserve(&base, need * chunk, 0, nullptr, 0)) != hipSuccess) break;
-        built.base[k] = base;
-        built.reserved[k] = need * chunk;
-        for (size_t i = 0; i < n && built.handles[k].size() < need && status == hipSuccess; ++i) {
+        if (need_pure) {
+            if ((status = hipMemAddressReserve(&base, need_pure * chunk, 0, nullptr, 0)) != hipSuccess) break;
+            built.base[k] = base;
+            built.reserved[k] = need_pure * chunk;
+            built.unit[k] = chunk;
+        }
+        size_t taken = 0;
+        for (size_t i = 0; i < n && taken < need && status == hipSuccess; ++i) {
             if (kind_of[i] != k) continue;
+            if (taken++ >= need_pure) { to_pages[k].push_back(i); continue; }
             if ((status = hipMemUnmap(s.at(i), chunk)) != hipSuccess) break;
             s.mapped[i] = 0;
             char *dst = static_cast<char *>(base) + built.handles[k].size() * chunk;
@@ -319,33 +379,86 @@ int create(int device, uint64_t bytes_per_region, uint64_t chunk_bytes, exodus_h
             status = hipMemSetAccess(dst, chunk, &acc, 1);
         }
     }
-    auto undo = [&built]() {
-        for (int k = 0; k < REGIONS; ++k) {
-            for (size_t j = 0; j < built.handles[k].size(); ++j) {
-                (void)hipMemUnmap(static_cast<char *>(built.base[k]) + j * built.chunk, built.chunk);
-                (void)hipMemRelease(built.handles[k][j]);
-            }
-            if (built.base[k]) (void)hipMemAddressFree(built.base[k], built.reserved[k]);
+    if (status == hipSuccess && need_striped) {
+        // Pages of a known region: hold what is still free (all but half a GiB), then release one sorted chunk at
+        // a time and allocate its size in pages at once -- they can only come from the hole the chunk left (a few
+        // may come from the half GiB, which the striping does not notice).
+        Loose held;
+        size_t free_now = 0, total_now = 0;
+        status = hipMemGetInfo(&free_now, &total_now);
+        const size_t spare = size_t(512) << 20;
+        while (status == hipSuccess && free_now > spare + PAGE) {
+            hipMemGenericAllocationHandle_t h;
+            const hipError_t e = hipMemCreate(&h, PAGE, &prop, 0);
+            if (e == hipErrorOutOfMemory) { (void)hipGetLastError(); break; }
+            if ((status = e) != hipSuccess) break;
+            held.handles.push_back(h);
+            free_now -= PAGE;
         }
-    };
-    if (status != hipSuccess) { undo(); return status; }
+        // the chunks whose pages take turns in the range: one of each kind after the other -- or, with no kinds,
+        // chunks spread evenly over the order of creation
+        const size_t lanes = REGIONS * need_striped;
+        std::vector<size_t> turn;
+        for (size_t c = 0; c < lanes; ++c)
+            turn.push_back(sorted ? to_pages[c % REGIONS][c / REGIONS] : (n * (2 * c + 1)) / (2 * lanes));
+        std::vector<Loose> pages(lanes);
+        for (size_t c = 0; c < lanes && status == hipSuccess; ++c) {
+            const size_t i = turn[c];
+            if ((status = hipMemUnmap(s.at(i), chunk)) != hipSuccess) break;
+            s.mapped[i] = 0;
+            if ((status = hipMemRelease(s.handle[i])) != hipSuccess) break;
+            s.owned[i] = 0;
+            for (size_t j = 0; j < ppc && status == hipSuccess; ++j) {
+                hipMemGenericAllocationHandle_t h;
+                if ((status = hipMemCreate(&h, PAGE, &prop, 0)) == hipSuccess) pages[c].handles.push_back(h);
+            }
+        }
+        const size_t total = lanes * ppc;                               // pages of the striped range
+        void *base = nullptr;
+        if (status == hipSuccess && (status = hipMemAddressReserve(&base, total * PAGE, 0, nullptr, 0)) == hipSuccess) {
+            built.base[STRIPED] = base;
+            built.reserved[STRIPED] = total * PAGE;
+            built.unit[STRIPED] = PAGE;
+            // page q of the range is page q / lanes of chunk q mod lanes; the arena owns a page once it is mapped
+            for (size_t q = 0; q < total && status == hipSuccess; ++q) {
+                const hipMemGenericAllocationHandle_t h = pages[q % lanes].handles[q / lanes];
+                if ((status = hipMemMap(static_cast<char *>(base) + q * PAGE, PAGE, 0, h, 0)) != hipSuccess) break;
+                built.handles[STRIPED].push_back(h);
+            }
+            // the pages that were mapped are the first ones of each chunk's list, in turn
+            for (size_t c = 0; c < lanes; ++c) {
+                const size_t mapped_c = (built.handles[STRIPED].size() + lanes - 1 - c) / lanes;
+                pages[c].handles.erase(pages[c].handles.begin(), pages[c].handles.begin() + mapped_c);
+            }
+            if (status == hipSuccess) status = hipMemSetAccess(base, total * PAGE, &acc, 1);
+        }
+    }                                                                   // what was held goes back here
+    if (status != hipSuccess) { (void)built.release(); return status; }
 
-    // 4. the proof: copies inside each arena (first half to second half) and between the arenas
-    const size_t half = (need / 2) * chunk;                  // 0 when a range is one chunk
-    for (int k = 0; k < REGIONS && status == hipSuccess; ++k) {
+    // 4. the proof: copies inside each arena (first half to second half) and between the regions' arenas
+    const size_t half = (need_pure / 2) * chunk;             // 0 when a range is one chunk or absent
+    for (int k = 0; k < ARENAS; ++k) {
         rep->base[k] = built.base[k];
-        rep->bytes[k] = need * chunk;
+        rep->bytes[k] = built.reserved[k];
+    }
+    rep->page_bytes = PAGE;
+    for (int k = 0; k < REGIONS && status == hipSuccess; ++k) {
         rep->copy_inside_GBs[k] = 0.f;
         if (half)
-            status = s.rate(static_cast<char *>(built.base[k]) + (need - need / 2) * chunk, built.base[k], half, 3,
+            status = s.rate(static_cast<char *>(built.base[k]) + (need_pure - need_pure / 2) * chunk, built.base[k], half, 3,
                             &rep->copy_inside_GBs[k]);
     }
     int slot = 0;
-    const size_t across = need * chunk;
-    for (int j = 0; j < REGIONS && status == hipSuccess; ++j)
+    const size_t across = need_pure * chunk;
+    for (int j = 0; j < REGIONS && status == hipSuccess && across; ++j)
         for (int k = 0; k < REGIONS && status == hipSuccess; ++k)
             if (j != k) status = s.rate(built.base[k], built.base[j], across, 3, &rep->copy_across_GBs[slot++]);
-    if (status != hipSuccess) { (void)hipDeviceSynchronize(); undo(); return status; }
+    rep->copy_striped_GBs = 0.f;
+    if (status == hipSuccess && need_striped) {
+        const size_t h = built.reserved[STRIPED] / (2 * chunk) * chunk;
+        if (h) status = s.rate(static_cast<char *>(built.base[STRIPED]) + h, built.base[STRIPED], h, 3, &rep->copy_striped_GBs);
+    }
+    if (status != hipSuccess) { (void)hipDeviceSynchronize(); (void)built.release(); return status; }
     built.live = true;
     table[device] = std::move(built);
     return hipSuccess;          // ~Sorting returns the unused chunks
@@ -355,17 +468,17 @@ int create(int device, uint64_t bytes_per_region, uint64_t chunk_bytes, exodus_h
 
 extern "C" {
 
-EXODUS_API int exodus_hbm_regions_create(int device, uint64_t bytes_per_region, uint64_t chunk_bytes,
-                                         exodus_hbm_report *report)
+EXODUS_API int exodus_hbm_regions_create(int device, uint64_t bytes_per_region, uint64_t bytes_striped,
+                                         uint64_t chunk_bytes, exodus_hbm_report *report)
 {
-    if (device < 0 || device >= MAX_DEVICES || !report || bytes_per_region == 0 || chunk_bytes == 0)
+    if (device < 0 || device >= MAX_DEVICES || !report || (bytes_per_region == 0 && bytes_striped == 0) || chunk_bytes == 0)
         return hipErrorInvalidValue;
     std::lock_guard<std::mutex> guard(table_mutex);
     if (table[device].live) return hipErrorInvalidValue;
     int before = 0;
     if (hipGetDevice(&before) != hipSuccess) return hipErrorInvalidDevice;
     *report = exodus_hbm_report{};
-    const int status = create(device, bytes_per_region, chunk_bytes, report);
+    const int status = create(device, bytes_per_region, bytes_striped, chunk_bytes, report);
     (void)hipSetDevice(before);
     return status;
 }
@@ -380,18 +493,8 @@ EXODUS_API int exodus_hbm_regions_destroy(int device)
     if (hipGetDevice(&before) != hipSuccess) return hipErrorInvalidDevice;
     int status = hipSetDevice(device);
     if (status == hipSuccess) status = hipDeviceSynchronize();
-    for (int k = 0; k < REGIONS; ++k) {
-        for (size_t j = 0; j < a.handles[k].size(); ++j) {
-            const hipError_t u = hipMemUnmap(static_cast<char *>(a.base[k]) + j * a.chunk, a.chunk);
-            const hipError_t r = hipMemRelease(a.handles[k][j]);
-            if (status == hipSuccess) status = u != hipSuccess ? u : r;
-        }
-        if (a.base[k]) {
-            const hipError_t f = hipMemAddressFree(a.base[k], a.reserved[k]);
-            if (status == hipSuccess) status = f;
-        }
-    }
-    a = Arenas{};
+    const hipError_t released = a.release();
+    if (status == hipSuccess) status = released;
     (void)hipSetDevice(before);
     return status;
 }

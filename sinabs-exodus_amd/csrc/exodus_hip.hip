@@ -251,6 +251,189 @@ __global__ void __launch_bounds__(WAVE) scan_kernel(const Op op, const int64_t n
 }
 
 // ---------------------------------------------------------------------------------------------
+// The same driver for the common case (row length a multiple of 4, 16-byte aligned tensors), with raw
+// buffer instructions.  A wave's 64 rows are one contiguous span of memory, at most 2^30 bytes long, so
+// every access is  span base (resource descriptor in SGPRs) + 32-bit lane offset:
+//   * no 64-bit address arithmetic and no per-access bounds code: one offset register per wave-wide
+//     load (shared by all tensors) plus the tile's offset; the driver above spends 170-370 registers
+//     on addresses, hoisted tile reads and prefetch data and keeps 1-3 waves per SIMD resident, this
+//     one 4-6, which is what hides the chains of dependent instructions of the recurrences;
+//   * the descriptor's size ends the span at the last valid row, so rows past the end of the tensor
+//     read zeros and drop their stores in hardware;
+//   * a row's first and last tiles share their memory lines with the neighbouring rows: there a lane
+//     whose 16 bytes lie outside its row gets an offset beyond the span (reads zero, stores nothing).
+// UQ = chunks of 4 steps the recurrence loop is unrolled by (caps how many tile reads are hoisted).
+// ---------------------------------------------------------------------------------------------
+typedef __amdgpu_buffer_rsrc_t Rsrc;
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+constexpr unsigned OUTSIDE = 0x80000000u;                     // an offset beyond any span
+
+__device__ __forceinline__ Rsrc span_rsrc(const float *base, unsigned bytes)
+{
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(base), 0, static_cast<int>(bytes), 0x00020000);
+}
+template <bool STREAM> __device__ __forceinline__ f32x4 span_load(Rsrc r, unsigned off)
+{
+    return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, (STREAM && EXODUS_NT_LOAD) ? 2 : 0));
+}
+__device__ __forceinline__ void span_store(f32x4 v, Rsrc r, unsigned off)
+{
+    // the whole offset travels in the vector register and a short wait that reads the data follows: a 16-byte
+    // buffer store with a scalar offset, directly followed by a write to its data registers, has stored wrong
+    // values on gfx950
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), r, off, 0, EXODUS_NT_STORE ? 2 : 0);
+    asm volatile("s_nop 1" : : "v"(v));
+}
+
+template <class Op, int TT, int UQ, int WPE>
+__global__ void __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(WPE, WPE)))
+scan_span_kernel(const Op op, const int64_t n_rows, const int n_steps, const int n_tiles, const int base_shift)
+{
+    using G = Geom<TT>;
+    constexpr int NIN = Op::NIN, NOUT = Op::NOUT;
+    constexpr int NSLOT = NIN > NOUT ? NIN : NOUT;
+    constexpr int TILE = WAVE * TT;
+    constexpr int NDER = Op::NDER, NROWP = Op::NROWP;
+    extern __shared__ f32x4 lds_raw[];
+    float *lds = reinterpret_cast<float *>(lds_raw);
+    float *rowp = lds + NSLOT * TILE;
+
+    const int lane = threadIdx.x;
+    const int64_t row0 = static_cast<int64_t>(blockIdx.x) * WAVE;
+    const int n_loc = n_rows - row0 < WAVE ? static_cast<int>(n_rows - row0) : WAVE;   // rows of this wave
+    const bool row_ok = lane < n_loc;
+
+    typename Op::State st;
+    op.init(st, row_ok ? row0 + lane : n_rows - 1, row_ok);
+    if constexpr (NDER > 0) {
+        float consts[NROWP > 0 ? NROWP : 1];
+        op.stash(st, consts);
+#pragma unroll
+        for (int k = 0; k < NROWP; ++k) rowp[lane * NROWP + k] = consts[k];
+    }
+
+    // the span: from the tile boundary at or below the first row's first step to the last row's end
+    const int64_t e0 = row0 * n_steps;
+    const int d = static_cast<int>((base_shift + e0) & (TT - 1));
+    const unsigned span_bytes = 4u * static_cast<unsigned>(d + n_loc * n_steps);
+    Rsrc rin[NIN > 0 ? NIN : 1], rout[NOUT > 0 ? NOUT : 1], rder;
+#pragma unroll
+    for (int j = 0; j < NIN; ++j) rin[j] = span_rsrc(op.in[j] + (e0 - d), span_bytes);
+#pragma unroll
+    for (int j = 0; j < NOUT; ++j) rout[j] = span_rsrc(op.out[j] + (e0 - d), span_bytes);
+    if constexpr (NDER > 0) rder = span_rsrc(op.der + (e0 - d), span_bytes);
+
+    const int l_chunk = lane % G::CPR;
+    const int l_row = lane / G::CPR;
+    // float position of a row's first step inside the span, and its distance from the tile boundary below
+    auto start_of = [&](int r) { return d + r * n_steps; };
+    const int my_shift = start_of(lane) & (TT - 1);
+    unsigned voff[G::NLD];                                    // byte offset of this lane's 16 bytes in tile 0
+#pragma unroll
+    for (int i = 0; i < G::NLD; ++i)
+        voff[i] = 4u * static_cast<unsigned>(start_of(l_row + i * G::RPI) & ~(TT - 1)) + 16u * l_chunk;
+    // first and last tiles: the offset, or OUTSIDE where the 16 bytes are not part of the row
+    auto edge_off = [&](int tile, int i) {
+        const int r = l_row + i * G::RPI;
+        const int t = tile * TT - (start_of(r) & (TT - 1)) + 4 * l_chunk;
+        return (r < n_loc && t >= 0 && t + 3 < n_steps) ? voff[i] + static_cast<unsigned>(tile) * (TT * 4u) : OUTSIDE;
+    };
+    auto interior = [&](int tile) { return tile >= 1 && (tile + 1) * TT <= n_steps; };
+
+    f32x4 pre[NIN > 0 ? NIN : 1][G::NLD];
+    auto fetch = [&](int tile) {
+        if (interior(tile)) {
+            const unsigned toff = static_cast<unsigned>(tile) * (TT * 4u);
+#pragma unroll
+            for (int i = 0; i < G::NLD; ++i)
+#pragma unroll
+                for (int j = 0; j < NIN; ++j) pre[j][i] = span_load<true>(rin[j], voff[i] + toff);
+        } else {
+            // lines shared with the neighbouring rows, which ask for them many tiles away in time: cacheable
+#pragma unroll
+            for (int i = 0; i < G::NLD; ++i) {
+                const unsigned off = edge_off(tile, i);
+#pragma unroll
+                for (int j = 0; j < NIN; ++j) pre[j][i] = span_load<false>(rin[j], off);
+            }
+        }
+    };
+
+    auto compute = [&](int t_first, auto guard) {
+        constexpr bool GUARD = decltype(guard)::value;
+        EXODUS_UNROLL(UQ)
+        for (int qq = 0; qq < G::CPR; ++qq) {
+            const int q = Op::REVERSE ? G::CPR - 1 - qq : qq;
+            f32x4 xin[NIN > 0 ? NIN : 1];
+            f32x4 yout[NOUT > 0 ? NOUT : 1];
+#pragma unroll
+            for (int j = 0; j < NIN; ++j)
+                xin[j] = *reinterpret_cast<const f32x4 *>(lds + j * TILE + G::off(lane, q));
+#pragma unroll
+            for (int j = 0; j < NOUT; ++j) yout[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ee = 0; ee < 4; ++ee) {
+                const int e = Op::REVERSE ? 3 - ee : ee;
+                const int t = t_first + 4 * q + e;
+                if (!GUARD || static_cast<unsigned>(t) < static_cast<unsigned>(n_steps)) {
+                    float x[NIN > 0 ? NIN : 1];
+                    float y[NOUT > 0 ? NOUT : 1];
+#pragma unroll
+                    for (int j = 0; j < NIN; ++j) x[j] = get(xin[j], e);
+                    op.step(st, x, y);
+#pragma unroll
+                    for (int j = 0; j < NOUT; ++j) put(yout[j], e, y[j]);
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < NOUT; ++j)
+                *reinterpret_cast<f32x4 *>(lds + j * TILE + G::off(lane, q)) = yout[j];
+        }
+    };
+
+    fetch(Op::REVERSE ? n_tiles - 1 : 0);
+
+    for (int it = 0; it < n_tiles; ++it) {
+        const int tile = Op::REVERSE ? n_tiles - 1 - it : it;
+#pragma unroll
+        for (int j = 0; j < NIN; ++j)
+#pragma unroll
+            for (int i = 0; i < G::NLD; ++i)
+                *reinterpret_cast<f32x4 *>(lds + j * TILE + G::off(l_row + i * G::RPI, l_chunk)) = pre[j][i];
+
+        if (it + 1 < n_tiles) fetch(Op::REVERSE ? tile - 1 : tile + 1);
+
+        wave_sync();
+        const bool inner = interior(tile);
+        if (inner)
+            compute(tile * TT - my_shift, std::false_type{});
+        else
+            compute(tile * TT - my_shift, std::true_type{});
+        op.end_tile(st);
+
+        if (NOUT > 0) {
+            wave_sync();
+#pragma unroll
+            for (int i = 0; i < G::NLD; ++i) {
+                const unsigned off = inner ? voff[i] + static_cast<unsigned>(tile) * (TT * 4u) : edge_off(tile, i);
+#pragma unroll
+                for (int j = 0; j < NOUT; ++j) {
+                    const f32x4 v = *reinterpret_cast<const f32x4 *>(lds + j * TILE + G::off(l_row + i * G::RPI, l_chunk));
+                    span_store(v, rout[j], off);
+                    if constexpr (NDER > 0) {
+                        if (j == Op::DER_SRC)
+                            span_store(op.derive(rowp + (l_row + i * G::RPI) * NROWP, v), rder, off);
+                    }
+                }
+            }
+        }
+        wave_sync();
+    }
+
+    if (row_ok) op.finish(st, row0 + lane);
+}
+
+// ---------------------------------------------------------------------------------------------
 // Ops
 // ---------------------------------------------------------------------------------------------
 struct LeakyFwdOp {
@@ -672,17 +855,27 @@ struct SpikeBwdOp {
 // host side
 // ---------------------------------------------------------------------------------------------
 
+// Tile length, unrolling and register budget of the span driver by the number of tiles an op keeps in LDS.
+// A wave's LDS footprint is slots * 64 rows * TT steps * 4 bytes of the CU's 160 KB; the register budget is
+// set to the number of waves per SIMD that this footprint allows (at most EXODUS_WPE_MAX).
+template <class Op>
+struct SpanPlan {
+    static constexpr int NSLOT = Op::NIN > Op::NOUT ? Op::NIN : Op::NOUT;
+    static constexpr int TT = NSLOT >= 3 ? EXODUS_TT_S3 : (NSLOT == 2 ? EXODUS_TT_S2 : EXODUS_TT_S1);
+    static constexpr int LDS_BYTES = (NSLOT * WAVE * TT + WAVE * Op::NROWP) * 4;
+    static constexpr int PER_CU = (160 * 1024) / LDS_BYTES;
+    static constexpr int WPE_LDS = (PER_CU + 3) / 4;
+    static constexpr int WPE = WPE_LDS < 1 ? 1 : (WPE_LDS > EXODUS_WPE_MAX ? EXODUS_WPE_MAX : WPE_LDS);
+    static constexpr int UQ = EXODUS_SPAN_UNROLL_Q;
+};
+
 template <class Op, int TT>
-int launch(const Op &op, int64_t n, int64_t t, void *stream)
+int launch_rows(const Op &op, int64_t n, int64_t t, bool vec, void *stream)
 {
     constexpr int NSLOT = Op::NIN > Op::NOUT ? Op::NIN : Op::NOUT;
     const size_t lds_bytes = (static_cast<size_t>(NSLOT) * WAVE * TT + WAVE * Op::NROWP) * sizeof(float);
     const int64_t n_blocks = (n + WAVE - 1) / WAVE;
     if (n_blocks > 0x7fffffffLL) return hipErrorInvalidValue;
-    bool vec = (t % 4) == 0;
-    for (int j = 0; j < Op::NIN; ++j) vec = vec && aligned16(op.in[j]);
-    for (int j = 0; j < Op::NOUT; ++j) vec = vec && aligned16(op.out[j]);
-    if constexpr (Op::NDER > 0) vec = vec && aligned16(op.der);   // the derived output leaves through the same stores
     // Tiles are aligned to the first tensor's address (allocators hand out >= 256-byte aligned
     // blocks, so in practice every tensor shares this alignment).  Row shifts are
     // (base_shift + r*t) mod TT, i.e. base_shift plus multiples of g = gcd(t, TT); the largest one
@@ -695,11 +888,28 @@ int launch(const Op &op, int64_t n, int64_t t, void *stream)
     const int64_t n_tiles = (t - 1 + max_shift) / TT + 1;
     const dim3 grid(static_cast<unsigned>(n_blocks)), block(WAVE);
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (vec)
-        hipLaunchKernelGGL((scan_kernel<Op, TT, true>), grid, block, lds_bytes, s, op, n, t, n_tiles, base_shift);
-    else
-        hipLaunchKernelGGL((scan_kernel<Op, TT, false>), grid, block, lds_bytes, s, op, n, t, n_tiles, base_shift);
+    if constexpr (TT == SpanPlan<Op>::TT) {
+        // 64 rows of at most 2^22 steps: a wave's span stays below 2^30 bytes
+        if (vec && t <= (1 << 22)) {
+            hipLaunchKernelGGL((scan_span_kernel<Op, TT, SpanPlan<Op>::UQ, SpanPlan<Op>::WPE>), grid, block, lds_bytes,
+                               s, op, n, static_cast<int>(t), static_cast<int>(n_tiles), base_shift);
+            return static_cast<int>(hipGetLastError());
+        }
+    }
+    hipLaunchKernelGGL((scan_kernel<Op, TT, false>), grid, block, lds_bytes, s, op, n, t, n_tiles, base_shift);
     return static_cast<int>(hipGetLastError());
+}
+
+// `TT_GENERIC` is the tile length of the driver for rows of any length and alignment
+template <class Op, int TT_GENERIC>
+int launch(const Op &op, int64_t n, int64_t t, void *stream)
+{
+    bool vec = (t % 4) == 0;
+    for (int j = 0; j < Op::NIN; ++j) vec = vec && aligned16(op.in[j]);
+    for (int j = 0; j < Op::NOUT; ++j) vec = vec && aligned16(op.out[j]);
+    if constexpr (Op::NDER > 0) vec = vec && aligned16(op.der);   // the derived output leaves through the same stores
+    if (vec && t <= (1 << 22)) return launch_rows<Op, SpanPlan<Op>::TT>(op, n, t, true, stream);
+    return launch_rows<Op, TT_GENERIC>(op, n, t, false, stream);
 }
 
 inline bool bad_dims(int64_t n, int64_t t) { return n < 0 || t < 0 || (t > 0 && n > INT64_MAX / t); }

@@ -23,7 +23,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("EXODUS_HIP_LIBRARY") or os.path.join(_HERE, "libexodus_hip.so")
 
 SURR_TENSOR, SURR_SINGLE_EXP, SURR_PERIODIC_EXP, SURR_HEAVISIDE = 0, 1, 2, 3
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 _p = ctypes.c_void_p
 _i64 = ctypes.c_int64
@@ -52,7 +52,7 @@ _SIGNATURES = {
     "exodus_layer_lif_backward_from_input": ([_p] * 16 + [_int, _int, _int, _int, _int, _f, _f, _p, _p, _p, _i64, _i64, _i64, _p], _int),
     "exodus_layer_leaky_forward": ([_p] * 6 + [_int, _int, _i64, _i64, _i64, _p], _int),
     "exodus_layer_leaky_backward": ([_p] * 9 + [_int, _int, _i64, _i64, _i64, _p], _int),
-    "exodus_hbm_regions_create": ([_int, ctypes.c_uint64, ctypes.c_uint64, _p], _int),
+    "exodus_hbm_regions_create": ([_int, ctypes.c_uint64, ctypes.c_uint64, ctypes.c_uint64, _p], _int),
     "exodus_hbm_regions_destroy": ([_int], _int),
 }
 

@@ -1,22 +1,25 @@
 """Where tensors live in HBM: region-aware allocation for MI355X.
 
-The 288 GiB of HBM3E of an MI355X behave as three regions of 96 GiB.  A kernel that streams from one
-region into another moves its data 8-12 % faster than one that reads and writes inside one region:
-a flat copy between 4 GiB buffers runs at 5.7-6.1 TB/s inside a region and at 6.3-6.5 TB/s across, and the
-time-strided layer kernels go from 5.2-5.4 TB/s to 5.6-5.9 TB/s.  Reads alone and writes alone do not care
-where they go; it is the mix of both in one region that costs.
+The 288 GiB of HBM3E of an MI355X behave as three regions of 96 GiB, and what a kernel *writes* is held back by
+the region it goes to.  Into a tensor that lies in one region the time-strided layer kernels write at 5.5-5.7 TB/s
+and the (rows, time) kernels (single 128-byte lines) at 4.4-4.9 TB/s; into a tensor whose memory alternates between
+the regions every 64 MiB the same kernels reach 6.0-6.3 and 5.6-5.8 TB/s.  Where the data they *read* lies matters
+less: inputs in one region and outputs striped over the others is the best case, everything striped is 3-4 % behind
+it, outputs in a single region 9-25 % (reads alone and writes alone in flat copies do not care).
 
 A process cannot ask the driver for memory of a region, and the order in which the driver hands memory out
 follows the regions only on a machine that has run nothing yet.  So the library sorts: it takes the free
-device memory in chunks of 4 GiB, measures with timed copies which chunks disturb each other, maps chunks of
-one kind behind each other into three address ranges and gives the rest back
-(``exodus_hbm_regions_create``, csrc/exodus_hbm.hip).  ``HbmRegions`` hands out tensors from these ranges.
+device memory in pages of 64 MiB, judges every 4 GiB of consecutively created pages with timed copies (which chunks
+disturb each other), and maps pages into four address ranges: one per region, and a *striped* one whose consecutive
+pages come from regions 0, 1, 2, 0, 1, 2, ... (``exodus_hbm_regions_create``, csrc/exodus_hbm.hip).  The rest goes
+back to the driver.  ``HbmRegions`` hands out tensors from these ranges.
 
-``empty(shape, region=k)`` allocates in range k; ``empty_like(x, away_from=[...])`` in a range that none of
-the given tensors lies in.  Tensors of the ranges are recognised by their addresses; for a tensor from
-elsewhere (the ordinary allocator) the range it copies to slowest is looked up once per storage with three
-short timed copies.  After ``enable()`` the layer-layout wrappers (``_hip.layerLifForward`` and friends)
-allocate their outputs this way; without it nothing changes.  The reference has no counterpart (its CUDA
+``empty(shape)`` allocates in the striped range, ``empty(shape, region=k)`` in the range of region k (0, 1, 2).
+After ``enable()`` the layer-layout wrappers (``_hip.layerLifForward`` and friends) allocate their outputs through
+``empty_like`` / ``empty`` of this module -- striped when there is a striped range; with region ranges only, in a
+range that none of the tensors the kernel reads lies in (tensors of the ranges are recognised by their addresses;
+for a tensor from the ordinary allocator the range it copies to slowest is looked up once per storage with three
+short timed copies).  Without ``enable()`` nothing changes.  The reference has no counterpart (its CUDA
 extension allocates outputs with ``torch.empty_like``, reference cuda/bindings.cu:98,144,183).
 
 Memory of a released tensor is handed out again at once, without regard to streams: a tensor from here is for
@@ -35,6 +38,8 @@ GIB = 2 ** 30
 CHUNK = 4 * GIB                 # physical memory is sorted in pieces of this size: shorter copies tell less
 ALIGN = 2 * 2 ** 20             # every tensor of a range starts on a 2 MiB boundary
 PROBES = 15                     # EXODUS_HBM_PROBES of include/exodus_hip.h
+ARENAS = 4                      # EXODUS_HBM_ARENAS: one range per region and the striped one
+STRIPED = 3                     # index of the striped range
 SMALLEST_PLACED = 2 ** 20       # smaller requests are left to the ordinary allocator
 PROBE_BYTES = GIB               # the slice of a foreign tensor that is timed against the ranges
 SMALLEST_PROBE = 256 * 2 ** 20  # foreign tensors below this are not classified (too short to time, too small to matter)
@@ -42,12 +47,14 @@ SMALLEST_PROBE = 256 * 2 ** 20  # foreign tensors below this are not classified 
 
 class _Report(ctypes.Structure):
     """exodus_hbm_report of include/exodus_hip.h"""
-    _fields_ = [("base", ctypes.c_void_p * 3), ("bytes", ctypes.c_uint64 * 3), ("chunk_bytes", ctypes.c_uint64),
+    _fields_ = [("base", ctypes.c_void_p * ARENAS), ("bytes", ctypes.c_uint64 * ARENAS),
+                ("chunk_bytes", ctypes.c_uint64), ("page_bytes", ctypes.c_uint64),
                 ("chunks_examined", ctypes.c_int32), ("kinds_found", ctypes.c_int32),
                 ("chunks_ambiguous", ctypes.c_int32), ("chunks_of_region", ctypes.c_int32 * 3),
                 ("threshold_GBs", ctypes.c_float), ("probe_same_kind_GBs", ctypes.c_float),
                 ("probe_other_kind_GBs", ctypes.c_float), ("copy_inside_GBs", ctypes.c_float * 3),
-                ("copy_across_GBs", ctypes.c_float * 6), ("probe_chunk", ctypes.c_int32 * PROBES),
+                ("copy_across_GBs", ctypes.c_float * 6), ("copy_striped_GBs", ctypes.c_float),
+                ("probe_chunk", ctypes.c_int32 * PROBES),
                 ("probe_kind", ctypes.c_int32 * PROBES), ("probe_pair_GBs", (ctypes.c_float * PROBES) * PROBES)]
 
 
@@ -81,40 +88,47 @@ def _copy_rate(dst: torch.Tensor, src: torch.Tensor, reps: int = 5) -> float:
 
 
 class HbmRegions:
-    """Three ranges of device memory, each made of physical memory of one region of HBM.
+    """Address ranges of device memory sorted by region of HBM: one per region (``gib_per_region`` each, may be 0)
+    and a striped one (``gib_striped``, may be 0) whose 64 MiB pages alternate between the regions.
 
-    ``gib_per_region`` is what each range holds for good (until ``close()``); a request that a range cannot
+    The sizes are what the ranges hold for good (until ``close()``); a request that a range cannot
     serve is passed to the ordinary allocator, which is harmless but loses the placement.  Creating the ranges
     takes nearly all free device memory for a second or two and gives back what it does not keep, so do it
     early, before the program's big allocations.  ``report`` holds what the sorting measured, ``verified``
-    whether copies between the finished ranges beat copies inside them.
-    Raises RuntimeError when the device's memory shows no three regions or too little of it is free.
+    whether copies between regions beat copies inside them on the finished ranges (on the probe chunks when there
+    are no region ranges).
+    Raises RuntimeError when too little memory is free, or when ranges of single regions are asked for and the
+    device's memory shows no three regions (a striped range alone is then still made, ``sorted`` False).
     """
 
-    def __init__(self, gib_per_region: float = 24.0, device: Optional[torch.device] = None):
+    def __init__(self, gib_per_region: float = 0.0, gib_striped: float = 48.0,
+                 device: Optional[torch.device] = None):
         from . import _hip
         self.device = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
         if self.device.type != "cuda":
             raise RuntimeError("HbmRegions needs a HIP device")
         if self.device.index is None:
             self.device = torch.device("cuda", torch.cuda.current_device())
-        if not 1 <= gib_per_region <= 80:
-            raise ValueError("gib_per_region must be between 1 and 80 (rounded up to whole chunks of 4 GiB): a range "
-                             "has to fit inside one region")
+        if gib_per_region < 0 or gib_striped < 0 or (gib_per_region == 0 and gib_striped == 0):
+            raise ValueError("gib_per_region and gib_striped must not be negative, and one of them positive")
+        if gib_per_region + gib_striped / 3 > 80:
+            raise ValueError("gib_per_region + gib_striped / 3 must not exceed 80 (rounded up to whole chunks of "
+                             "4 GiB): that much is taken from each region, and a region has 96 GiB")
         self._lib = _hip.lib
         rep = _Report()
         with torch.cuda.device(self.device):
             torch.zeros(1, device=self.device)             # the device's context exists
             torch.cuda.empty_cache()                       # what torch has cached cannot be sorted
             torch.cuda.synchronize()
-            rc = self._lib.exodus_hbm_regions_create(self.device.index, int(gib_per_region * GIB), CHUNK,
-                                                     ctypes.byref(rep))
+            rc = self._lib.exodus_hbm_regions_create(self.device.index, int(gib_per_region * GIB),
+                                                     int(gib_striped * GIB), CHUNK, ctypes.byref(rep))
         self.report: Dict[str, object] = {
             "chunks_examined": rep.chunks_examined, "kinds_found": rep.kinds_found,
             "chunks_ambiguous": rep.chunks_ambiguous, "chunks_of_region": list(rep.chunks_of_region),
             "threshold_GBs": rep.threshold_GBs, "probe_chunks_same_region_GBs": rep.probe_same_kind_GBs,
             "probe_chunks_other_region_GBs": rep.probe_other_kind_GBs,
-            "inside_one_range_GBs": list(rep.copy_inside_GBs), "across_ranges_GBs": list(rep.copy_across_GBs)}
+            "inside_one_range_GBs": list(rep.copy_inside_GBs), "across_ranges_GBs": list(rep.copy_across_GBs),
+            "inside_striped_range_GBs": rep.copy_striped_GBs}
         # the probe chunks: position, group, and the copy rate between every two (what the groups were read from)
         self.probes = {"chunk": list(rep.probe_chunk), "kind": list(rep.probe_kind),
                        "pair_GBs": [[rep.probe_pair_GBs[a][b] for b in range(PROBES)] for a in range(PROBES)]}
@@ -123,20 +137,24 @@ class HbmRegions:
             raise RuntimeError(f"exodus_hbm_regions_create: {text.decode() if isinstance(text, bytes) else text} "
                                f"(status {rc}; measured: {self.report}; "
                                f"probe chunks {self.probes['chunk']} in groups {self.probes['kind']})")
-        self.bases: List[int] = [int(rep.base[k]) for k in range(3)]
-        self.sizes: List[int] = [int(rep.bytes[k]) for k in range(3)]
+        self.bases: List[int] = [int(rep.base[k] or 0) for k in range(ARENAS)]
+        self.sizes: List[int] = [int(rep.bytes[k]) for k in range(ARENAS)]
+        self.page_bytes = int(rep.page_bytes)
+        # False: the copies showed no three regions (memory that came back from earlier processes as a mixture of
+        # them); the striped range is then made of chunks spread over the memory, as they are
+        self.sorted = rep.kinds_found == 3
         self._free: List[List[List[int]]] = [[[0, n]] for n in self.sizes]   # per range: [offset, bytes], by offset
         self._lock = threading.Lock()
         self._live, self._closing, self._closed = 0, False, False
         self._foreign: Dict[int, int] = {}
         self._anchors: Optional[List[torch.Tensor]] = None
         inside = [r for r in rep.copy_inside_GBs if r > 0] or [rep.probe_same_kind_GBs]
-        across = list(rep.copy_across_GBs)
+        across = [r for r in rep.copy_across_GBs if r > 0] or [rep.probe_other_kind_GBs]
         # single pairs of chunks scatter by a few percent around 6.0 (same region) and 6.35 TB/s (two regions);
         # the copies over whole ranges average over many pairs
-        self.verified = bool(sum(across) / len(across) > 1.025 * sum(inside) / len(inside))
-        if not self.verified:
-            warnings.warn(f"HbmRegions: copies between the finished ranges are not clearly faster than copies "
+        self.verified = bool(self.sorted and sum(across) / len(across) > 1.025 * sum(inside) / len(inside))
+        if self.sorted and not self.verified:
+            warnings.warn(f"HbmRegions: copies between the regions are not clearly faster than copies "
                           f"inside them ({self.report}); allocation works, the gain may not be there")
 
     # ------------------------------------------------------------------ the ranges' free lists
@@ -182,21 +200,22 @@ class HbmRegions:
 
     # ------------------------------------------------------------------ queries
     def pool_of(self, t: torch.Tensor) -> Optional[int]:
-        """Index of the range whose memory holds ``t``, or None."""
+        """Index of the range whose memory holds ``t`` (0, 1, 2: a region's; 3: the striped one), or None."""
         p = t.data_ptr()
-        for k in range(3):
-            if self.bases[k] <= p < self.bases[k] + self.sizes[k]:
+        for k in range(ARENAS):
+            if self.sizes[k] and self.bases[k] <= p < self.bases[k] + self.sizes[k]:
                 return k
         return None
 
     def region_of(self, t: torch.Tensor) -> Optional[int]:
-        """The range (0, 1, 2) made of the same kind of memory as ``t``: by address for tensors of the ranges,
-        by three timed copies (once per storage) for others; None for tensors too small to tell or to matter."""
+        """The region (0, 1, 2) that holds ``t``: by address for tensors of the regions' ranges, by three timed
+        copies (once per storage) for others; None for tensors of the striped range, tensors too small to tell or
+        to matter, and when there are no region ranges to time against."""
         k = self.pool_of(t)
         if k is not None:
-            return k
+            return k if k < STRIPED else None
         nbytes = t.numel() * t.element_size()
-        if nbytes < SMALLEST_PROBE or not t.is_contiguous() or t.device != self.device:
+        if nbytes < SMALLEST_PROBE or not t.is_contiguous() or t.device != self.device or not self.sizes[0]:
             return None
         key = t.untyped_storage().data_ptr()
         if key not in self._foreign:
@@ -204,7 +223,7 @@ class HbmRegions:
                 return None                                # timing needs to wait for the device
             with torch.cuda.device(self.device), torch.no_grad():
                 if self._anchors is None:
-                    n = min(PROBE_BYTES, min(self.sizes) // 4)
+                    n = min(PROBE_BYTES, min(self.sizes[:3]) // 4)
                     self._anchors = [self.empty((n,), torch.uint8, region=j) for j in range(3)]
                 n = min(self._anchors[0].numel(), nbytes)
                 src = t.detach().reshape(-1).view(torch.uint8)[:n]
@@ -226,16 +245,17 @@ class HbmRegions:
     # ------------------------------------------------------------------ allocation
     def empty(self, shape: Sequence[int], dtype=torch.float32, region: Optional[int] = None,
               away_from: Iterable[Optional[torch.Tensor]] = ()) -> torch.Tensor:
-        """An uninitialised tensor in range ``region``, or in the range that holds none (or the least) of
-        ``away_from``; from the ordinary allocator if it is tiny or the range is full."""
+        """An uninitialised tensor in range ``region`` (0, 1, 2: that region; ``STRIPED``); without ``region`` in
+        the striped range, or -- when there is none -- in the region that holds none (or the least) of
+        ``away_from``.  From the ordinary allocator if it is tiny or the range is full or absent."""
         shape = tuple(int(s) for s in shape)
         count = 1
         for s in shape:
             count *= s
         nbytes = count * torch.empty((), dtype=dtype).element_size()
         if nbytes >= SMALLEST_PLACED:
-            k = self._pick(away_from) if region is None else int(region)
-            offset = self._take(k, nbytes)
+            k = int(region) if region is not None else (STRIPED if self.sizes[STRIPED] else self._pick(away_from))
+            offset = self._take(k, nbytes) if self.sizes[k] else None
             if offset is not None:
                 block = _Block(self, k, offset, nbytes, -(-nbytes // ALIGN) * ALIGN)
                 return torch.as_tensor(block, device=self.device).view(dtype).view(shape)
@@ -258,12 +278,13 @@ class HbmRegions:
 _active: Optional[HbmRegions] = None
 
 
-def enable(gib_per_region: float = 24.0, device: Optional[torch.device] = None) -> HbmRegions:
+def enable(gib_per_region: float = 0.0, gib_striped: float = 48.0,
+           device: Optional[torch.device] = None) -> HbmRegions:
     """Create the ranges and make the layer-layout kernels' wrappers allocate their outputs through them."""
     global _active
     if _active is not None:
         disable()
-    _active = HbmRegions(gib_per_region, device)
+    _active = HbmRegions(gib_per_region, gib_striped, device)
     return _active
 
 
@@ -280,8 +301,8 @@ def active() -> Optional[HbmRegions]:
 
 
 def empty_like(like: torch.Tensor, away_from: Optional[Iterable[Optional[torch.Tensor]]] = None) -> torch.Tensor:
-    """``torch.empty_like(like)``, or -- after ``enable()`` -- a tensor of that shape in a region of HBM that
-    none of ``away_from`` (default: ``like`` itself) lies in."""
+    """``torch.empty_like(like)``, or -- after ``enable()`` -- a tensor of that shape in the striped range, or
+    (region ranges only) in a region of HBM that none of ``away_from`` (default: ``like`` itself) lies in."""
     if _active is None or like.device != _active.device:
         return torch.empty_like(like)
     return _active.empty_like(like, away_from)

@@ -40,7 +40,7 @@ def test_library_exports_every_declared_symbol():
     extra = [l.split()[-1] for l in exported.splitlines() if " T " in l and not l.split()[-1].startswith("exodus_")]
     assert not extra, f"unexpected exported symbols: {extra}"
     lib.exodus_hip_abi_version.restype = ctypes.c_int
-    assert lib.exodus_hip_abi_version() == 6
+    assert lib.exodus_hip_abi_version() == 7
 
 
 def test_layer_entry_points_reject_too_wide_layers_before_touching_the_device():
