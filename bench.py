@@ -47,18 +47,18 @@ WORKLOADS = {
 # and the committed summary the figure comes from.  These are measurements of the kernels as they were
 # when the summary was made; a kernel that changes needs its counters taken again.
 MEASURED_TRAFFIC = {
-    ("c5", "exodus_layer_lif_backward"): (25.74e9, "profiles/layer_lif_c5_pmc.md"),
-    ("c5", "exodus_layer_lif_forward"): (17.34e9, "profiles/layer_lif_c5_pmc.md"),
-    ("c5", "exodus_synlif_backward"): (33.79e9, "profiles/rows_synlif_c5_pmc.md"),
-    ("c5", "exodus_synlif_forward"): (33.64e9, "profiles/rows_synlif_c5_pmc.md"),
-    ("c2", "exodus_layer_lif_backward"): (15.37e9, "profiles/layer_lif_c2_kernel_stats_pmc.md"),
-    ("c2", "exodus_layer_lif_forward"): (10.30e9, "profiles/layer_lif_c2_kernel_stats_pmc.md"),
-    ("c3", "exodus_layer_leaky_backward"): (3.15e9, "profiles/layer_leaky_c3_kernel_stats_pmc.md"),
-    ("c3", "exodus_layer_leaky_forward"): (2.10e9, "profiles/layer_leaky_c3_kernel_stats_pmc.md"),
-    ("c2", "exodus_lif_forward"): (15.76e9, "profiles/rows_lif_c2_kernel_stats_pmc.md"),
-    ("c2", "exodus_lif_backward_fused"): (16.16e9, "profiles/rows_lif_c2_kernel_stats_pmc.md"),
-    ("c3", "exodus_leaky_forward"): (2.12e9, "profiles/rows_leaky_c3_kernel_stats_pmc.md"),
-    ("c3", "exodus_leaky_backward_fused"): (3.20e9, "profiles/rows_leaky_c3_kernel_stats_pmc.md"),
+    ("c5", "exodus_layer_lif_backward"): (25.74e9, "profiles/all_workloads_striped_placement_kernel_stats_pmc.md"),
+    ("c5", "exodus_layer_lif_forward"): (17.34e9, "profiles/all_workloads_striped_placement_kernel_stats_pmc.md"),
+    ("c5", "exodus_synlif_backward"): (33.79e9, "profiles/all_workloads_striped_placement_kernel_stats_pmc.md"),
+    ("c5", "exodus_synlif_forward"): (33.64e9, "profiles/all_workloads_striped_placement_kernel_stats_pmc.md"),
+    ("c2", "exodus_layer_lif_backward"): (15.38e9, "profiles/all_workloads_striped_placement_kernel_stats_pmc.md"),
+    ("c2", "exodus_layer_lif_forward"): (10.30e9, "profiles/all_workloads_striped_placement_kernel_stats_pmc.md"),
+    ("c3", "exodus_layer_leaky_backward"): (3.15e9, "profiles/all_workloads_striped_placement_kernel_stats_pmc.md"),
+    ("c3", "exodus_layer_leaky_forward"): (2.10e9, "profiles/all_workloads_striped_placement_kernel_stats_pmc.md"),
+    ("c2", "exodus_lif_forward"): (15.75e9, "profiles/all_workloads_striped_placement_kernel_stats_pmc.md"),
+    ("c2", "exodus_lif_backward_fused"): (16.06e9, "profiles/all_workloads_striped_placement_kernel_stats_pmc.md"),
+    ("c3", "exodus_leaky_forward"): (2.12e9, "profiles/all_workloads_striped_placement_kernel_stats_pmc.md"),
+    ("c3", "exodus_leaky_backward_fused"): (3.20e9, "profiles/all_workloads_striped_placement_kernel_stats_pmc.md"),
 }
 
 # what the default run reports next to its headline workload: (workload, path)
