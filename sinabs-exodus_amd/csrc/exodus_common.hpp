@@ -39,6 +39,10 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));    // one 16-byte chunk
 #ifndef EXODUS_SPAN_UNROLL_Q
 #define EXODUS_SPAN_UNROLL_Q 2
 #endif
+// 64-byte sectors shared by two rows of a wave are written in one piece (0: each row writes its part)
+#ifndef EXODUS_WHOLE_SECTORS
+#define EXODUS_WHOLE_SECTORS 1
+#endif
 
 // Unroll factor of the per-tile chunk loop (each chunk = 4 time steps).  Full unrolling lets the
 // compiler hoist every LDS read of the tile, which costs registers and therefore resident waves.

@@ -287,7 +287,8 @@ __device__ __forceinline__ void span_store(f32x4 v, Rsrc r, unsigned off)
 
 template <class Op, int TT, int UQ, int WPE>
 __global__ void __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(WPE, WPE)))
-scan_span_kernel(const Op op, const int64_t n_rows, const int n_steps, const int n_tiles, const int base_shift)
+scan_span_kernel(const Op op, const int64_t n_rows, const int n_steps, const int n_tiles, const int base_shift,
+                 const int whole_sectors)
 {
     using G = Geom<TT>;
     constexpr int NIN = Op::NIN, NOUT = Op::NOUT;
@@ -297,6 +298,7 @@ scan_span_kernel(const Op op, const int64_t n_rows, const int n_steps, const int
     extern __shared__ f32x4 lds_raw[];
     float *lds = reinterpret_cast<float *>(lds_raw);
     float *rowp = lds + NSLOT * TILE;
+    float *kept_back = rowp + WAVE * NROWP;                   // [NOUT][64 rows][4 chunks] with whole_sectors
 
     const int lane = threadIdx.x;
     const int64_t row0 = static_cast<int64_t>(blockIdx.x) * WAVE;
@@ -411,11 +413,11 @@ scan_span_kernel(const Op op, const int64_t n_rows, const int n_steps, const int
             compute(tile * TT - my_shift, std::true_type{});
         op.end_tile(st);
 
-        if (NOUT > 0) {
+        if (NOUT > 0 && inner) {
             wave_sync();
 #pragma unroll
             for (int i = 0; i < G::NLD; ++i) {
-                const unsigned off = inner ? voff[i] + static_cast<unsigned>(tile) * (TT * 4u) : edge_off(tile, i);
+                const unsigned off = voff[i] + static_cast<unsigned>(tile) * (TT * 4u);
 #pragma unroll
                 for (int j = 0; j < NOUT; ++j) {
                     const f32x4 v = *reinterpret_cast<const f32x4 *>(lds + j * TILE + G::off(l_row + i * G::RPI, l_chunk));
@@ -423,6 +425,50 @@ scan_span_kernel(const Op op, const int64_t n_rows, const int n_steps, const int
                     if constexpr (NDER > 0) {
                         if (j == Op::DER_SRC)
                             span_store(op.derive(rowp + (l_row + i * G::RPI) * NROWP, v), rder, off);
+                    }
+                }
+            }
+        } else if (NOUT > 0) {
+            // A row's first and last tile.  Where rows do not start on 64-byte boundaries, the sector that holds the
+            // end of one row and the start of the next would be written in two parts, many tiles apart in time (a
+            // partial write costs the memory a read and a write).  With whole_sectors the part that is produced first
+            // -- the next row's first values when time runs forward, the row's last values when it runs backward --
+            // is kept back in LDS and leaves together with the other part, through the lanes that hold that part's
+            // line anyway.  Only the sectors between the rows of two waves stay split.
+            wave_sync();
+#pragma unroll
+            for (int i = 0; i < G::NLD; ++i) {
+                const int r = l_row + i * G::RPI;
+                const int sh = start_of(r) & (TT - 1);
+                const int t = tile * TT - sh + 4 * l_chunk;
+                const bool in_row = r < n_loc && t >= 0 && t + 3 < n_steps;
+                unsigned off = in_row ? voff[i] + static_cast<unsigned>(tile) * (TT * 4u) : OUTSIDE;
+                bool keep = false, kept = false;              // this lane's values stay here / come from what was kept
+                int src = r;                                  // the row whose values this lane stores
+                if (whole_sectors) {
+                    const int sector = tile * (TT / 16) + (l_chunk >> 2);   // of this lane's 16 bytes, from the row's tile 0
+                    const int e = sh + n_steps;                             // where the next row starts, likewise
+                    if (!Op::REVERSE) {
+                        keep = in_row && r >= 1 && (sh & 15) != 0 && sector == (sh >> 4);
+                        kept = !in_row && r + 1 < n_loc && t >= n_steps && (e & 15) != 0 && sector == (e >> 4);
+                        if (kept) src = r + 1;
+                    } else {
+                        keep = in_row && r + 1 < n_loc && (e & 15) != 0 && sector == (e >> 4);
+                        kept = !in_row && r >= 1 && r < n_loc && t < 0 && (sh & 15) != 0 && sector == (sh >> 4);
+                        if (kept) src = r - 1;
+                    }
+                    if (kept) off = voff[i] + static_cast<unsigned>(tile) * (TT * 4u);
+                    if (keep) off = OUTSIDE;
+                }
+#pragma unroll
+                for (int j = 0; j < NOUT; ++j) {
+                    f32x4 v = *reinterpret_cast<const f32x4 *>(lds + j * TILE + G::off(r, l_chunk));
+                    f32x4 *slot = reinterpret_cast<f32x4 *>(kept_back + ((j * WAVE + src) * 4 + (l_chunk & 3)) * 4);
+                    if (keep) *slot = v;
+                    if (kept) v = *slot;
+                    span_store(v, rout[j], off);
+                    if constexpr (NDER > 0) {
+                        if (j == Op::DER_SRC) span_store(op.derive(rowp + src * NROWP, v), rder, off);
                     }
                 }
             }
@@ -891,8 +937,14 @@ int launch_rows(const Op &op, int64_t n, int64_t t, bool vec, void *stream)
     if constexpr (TT == SpanPlan<Op>::TT) {
         // 64 rows of at most 2^22 steps: a wave's span stays below 2^30 bytes
         if (vec && t <= (1 << 22)) {
-            hipLaunchKernelGGL((scan_span_kernel<Op, TT, SpanPlan<Op>::UQ, SpanPlan<Op>::WPE>), grid, block, lds_bytes,
-                               s, op, n, static_cast<int>(t), static_cast<int>(n_tiles), base_shift);
+            // rows that do not all start on 64-byte boundaries: sectors shared by two rows are written whole, which
+            // takes 4 chunks of LDS per row and output (rows of at least a tile, so that a row's two ends lie in
+            // different tiles)
+            const int whole_sectors = EXODUS_WHOLE_SECTORS && Op::NOUT > 0 && t > TT && (t % 16 != 0 || base_shift % 16 != 0);
+            const size_t lds_kept = whole_sectors ? static_cast<size_t>(Op::NOUT) * WAVE * 16 * sizeof(float) : 0;
+            hipLaunchKernelGGL((scan_span_kernel<Op, TT, SpanPlan<Op>::UQ, SpanPlan<Op>::WPE>), grid, block,
+                               lds_bytes + lds_kept, s, op, n, static_cast<int>(t), static_cast<int>(n_tiles), base_shift,
+                               whole_sectors);
             return static_cast<int>(hipGetLastError());
         }
     }

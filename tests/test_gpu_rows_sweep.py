@@ -1,6 +1,7 @@
 """Seeded sweep through the (rows, time) entry points against the C restatement of the reference kernels:
 random row counts and lengths (around the 64-row waves and the 32-step tiles), matrices that start at element
-offsets 0-3 inside a larger buffer (16-byte vector accesses next to unaligned rows), caps, clamp, the three
+offsets 0-3, 4 and 12 inside a larger buffer (16-byte vector accesses next to unaligned rows; rows that share
+64-byte sectors, which the kernels then write in one piece), caps, clamp, the three
 in-kernel surrogates, with and without a gradient on the membrane potential.  Forward outputs bit for bit;
 gradients within rtol 1e-4 / atol 1e-5 (alpha gradients: atol scaled by sqrt(T)) plus 1e-5 of the largest magnitude."""
 import random
@@ -29,8 +30,9 @@ def test_random_rows_against_the_c_oracle():
     worst = 0.0
     for case in range(300):
         n = rnd.choice([1, 2, 3, 63, 64, 65, 100, 127, 128, 129, 200, 256, 300, 513])
-        t = rnd.choice([1, 2, 3, 4, 5, 7, 8, 15, 16, 17, 31, 32, 33, 47, 63, 64, 65, 96, 100, 127, 128, 129, 200, 300, 301, 303])
-        off = rnd.choice([0, 0, 1, 2, 3])
+        t = rnd.choice([1, 2, 3, 4, 5, 7, 8, 15, 16, 17, 31, 32, 33, 36, 44, 47, 63, 64, 65, 68, 96, 100, 127, 128, 129, 132, 200,
+                        260, 300, 301, 303])
+        off = rnd.choice([0, 0, 0, 1, 2, 3, 4, 12])       # 4, 12: 16-byte aligned, but rows start inside 64-byte sectors
         g = gen(9000 + case)
         use_lo = rnd.random() < 0.6
         cap = rnd.choice([-1, 1, 2, 3])
@@ -41,7 +43,7 @@ def test_random_rows_against_the_c_oracle():
         what = f"case {case}: n={n} t={t} offset={off} clamp={use_lo} cap={cap}"
 
         def on_device(z):                                  # a device copy that starts `off` elements into a buffer
-            buf = torch.empty(z.numel() + 8, device="cuda")
+            buf = torch.empty(z.numel() + 16, device="cuda")
             view = buf[off:off + z.numel()].view(z.shape)
             view.copy_(z)
             return view
