@@ -789,7 +789,8 @@ def main():
     }
     if plain_first is not None:
         roof["frac_by_placement"] = {
-            "striped: inputs in one region, outputs striped over the three (this run's figures)":
+            ("striped: inputs in one region, outputs striped over the three (this run's figures)" if place.mode == "striped"
+             else f"{place.mode} (this run's figures; {plain_note})"):
                 {"frac": roof["frac"], "fwd_bwd_combined_frac": roof["fwd_bwd_combined_frac"]},
             "ordinary allocator, first allocations of a process (measured before this one touched the GPU)": plain_first}
     if args.others and not args.shape:

@@ -304,7 +304,9 @@ int exodus_spike_backward(float *input_grad, const float *surr, const float *out
  * freed in small pieces comes back as a mixture of the regions below the size of a chunk): with bytes_per_region > 0
  * the call returns EXODUS_ERROR_REGIONS_NOT_FOUND (the report's fields up to kinds_found are then filled); with only
  * a striped range asked for it succeeds with kinds_found < 3, the pages taking turns between chunks spread evenly
- * over the memory instead.  hipErrorOutOfMemory when too little memory is free to find or fill the ranges,
+ * over the memory instead.  sort = 0 skips the timed copies and builds the striped range that way at once
+ * (kinds_found = 0; bytes_per_region must be 0): cheaper, and enough on a machine whose memory is known to come back
+ * mixed.  hipErrorOutOfMemory when too little memory is free to find or fill the ranges,
  * hipErrorInvalidValue for bad arguments or a device that already has its ranges.  Takes a second or two;
  * synchronises the device. */
 #define EXODUS_HBM_REGIONS 3
@@ -329,7 +331,7 @@ typedef struct exodus_hbm_report {
     float probe_pair_GBs[EXODUS_HBM_PROBES][EXODUS_HBM_PROBES];   /* two of them (mean of both directions) */
 } exodus_hbm_report;
 int exodus_hbm_regions_create(int device, uint64_t bytes_per_region, uint64_t bytes_striped, uint64_t chunk_bytes,
-                              exodus_hbm_report *report);
+                              int sort, exodus_hbm_report *report);
 int exodus_hbm_regions_destroy(int device);
 
 #ifdef __cplusplus

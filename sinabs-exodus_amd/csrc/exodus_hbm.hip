@@ -22,7 +22,7 @@
 // sorted chunk: with all other free memory held, the chunk is released and 64 pages are allocated at
 // once, which can only come from the hole it left.
 //
-//   exodus_hbm_regions_create(device, bytes_per_region, bytes_striped, chunk_bytes, &report)
+//   exodus_hbm_regions_create(device, bytes_per_region, bytes_striped, chunk_bytes, sort, &report)
 //   exodus_hbm_regions_destroy(device)
 //
 // Both calls synchronise the device.  One set of arenas per device; creating a second one fails with
@@ -172,7 +172,8 @@ float two_group_threshold(const std::vector<float> &v)
     return 0.5f * (lo + hi);
 }
 
-int create(int device, uint64_t bytes_per_region, uint64_t bytes_striped, uint64_t chunk_bytes, exodus_hbm_report *rep)
+int create(int device, uint64_t bytes_per_region, uint64_t bytes_striped, uint64_t chunk_bytes, bool sort,
+           exodus_hbm_report *rep)
 {
     HBM_TRY(hipSetDevice(device));
     HBM_TRY(hipDeviceSynchronize());
@@ -226,7 +227,7 @@ int create(int device, uint64_t bytes_per_region, uint64_t bytes_striped, uint64
     for (int p = 0; p < PROBES; ++p) probe[p] = (n * (2 * p + 1)) / (2 * PROBES);
     float pair[PROBES][PROBES] = {};
     std::vector<float> all;
-    for (int a = 0; a < PROBES; ++a)
+    for (int a = 0; a < PROBES && sort; ++a)
         for (int b = 0; b < a; ++b) {
             float ab = 0.f, ba = 0.f;
             HBM_TRY(s.rate(s.at(probe[b]), s.at(probe[a]), chunk, 3, &ab));
@@ -234,6 +235,7 @@ int create(int device, uint64_t bytes_per_region, uint64_t bytes_striped, uint64
             pair[a][b] = pair[b][a] = 0.5f * (ab + ba);
             all.push_back(pair[a][b]);
         }
+    if (!sort) all.assign(1, 0.f);                           // nothing was timed: every probe one group, no kinds
     const float threshold = two_group_threshold(all);
     // Groups of probes: every probe starts as a group of its own, and the two groups with the slowest mean copy
     // rate between them are joined until three are left (single pairs scatter by a few percent around the two
@@ -292,7 +294,7 @@ int create(int device, uint64_t bytes_per_region, uint64_t bytes_striped, uint64
     // Without three kinds there are no regions to sort by: then the memory the driver hands out is already a
     // mixture at a scale below the chunks (after processes that allocated and freed it in small pieces), which
     // is what the striped range wants to be; ranges of one region cannot be made.
-    bool sorted = kinds == REGIONS;
+    bool sorted = sort && kinds == REGIONS;
     // the gap between the two groups of rates has to be a real one
     float slow_max = 0.f, fast_min = 1e30f, slow_sum = 0.f, fast_sum = 0.f;
     int slow_n = 0, fast_n = 0;
@@ -307,7 +309,7 @@ int create(int device, uint64_t bytes_per_region, uint64_t bytes_striped, uint64
         rep->probe_other_kind_GBs = fast_sum / fast_n;
         if (rep->probe_other_kind_GBs < 1.025f * rep->probe_same_kind_GBs) sorted = false;
     }
-    if (!sorted) rep->kinds_found = std::min(rep->kinds_found, REGIONS - 1);
+    if (!sorted) rep->kinds_found = sort ? std::min(rep->kinds_found, REGIONS - 1) : 0;
     if (!sorted && need_pure) return EXODUS_ERROR_REGIONS_NOT_FOUND;
 
     // 2. every chunk against up to three probes of each kind: the kind it copies to slowest
@@ -469,16 +471,17 @@ int create(int device, uint64_t bytes_per_region, uint64_t bytes_striped, uint64
 extern "C" {
 
 EXODUS_API int exodus_hbm_regions_create(int device, uint64_t bytes_per_region, uint64_t bytes_striped,
-                                         uint64_t chunk_bytes, exodus_hbm_report *report)
+                                         uint64_t chunk_bytes, int sort, exodus_hbm_report *report)
 {
     if (device < 0 || device >= MAX_DEVICES || !report || (bytes_per_region == 0 && bytes_striped == 0) || chunk_bytes == 0)
         return hipErrorInvalidValue;
+    if (!sort && bytes_per_region != 0) return hipErrorInvalidValue;    // ranges of one region need the sorting
     std::lock_guard<std::mutex> guard(table_mutex);
     if (table[device].live) return hipErrorInvalidValue;
     int before = 0;
     if (hipGetDevice(&before) != hipSuccess) return hipErrorInvalidDevice;
     *report = exodus_hbm_report{};
-    const int status = create(device, bytes_per_region, bytes_striped, chunk_bytes, report);
+    const int status = create(device, bytes_per_region, bytes_striped, chunk_bytes, sort != 0, report);
     (void)hipSetDevice(before);
     return status;
 }

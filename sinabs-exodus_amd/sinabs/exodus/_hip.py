@@ -52,7 +52,7 @@ _SIGNATURES = {
     "exodus_layer_lif_backward_from_input": ([_p] * 16 + [_int, _int, _int, _int, _int, _f, _f, _p, _p, _p, _i64, _i64, _i64, _p], _int),
     "exodus_layer_leaky_forward": ([_p] * 6 + [_int, _int, _i64, _i64, _i64, _p], _int),
     "exodus_layer_leaky_backward": ([_p] * 9 + [_int, _int, _i64, _i64, _i64, _p], _int),
-    "exodus_hbm_regions_create": ([_int, ctypes.c_uint64, ctypes.c_uint64, ctypes.c_uint64, _p], _int),
+    "exodus_hbm_regions_create": ([_int, ctypes.c_uint64, ctypes.c_uint64, ctypes.c_uint64, _int, _p], _int),
     "exodus_hbm_regions_destroy": ([_int], _int),
 }
 

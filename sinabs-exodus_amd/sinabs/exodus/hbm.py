@@ -94,7 +94,10 @@ class HbmRegions:
     The sizes are what the ranges hold for good (until ``close()``); a request that a range cannot
     serve is passed to the ordinary allocator, which is harmless but loses the placement.  Creating the ranges
     takes nearly all free device memory for a second or two and gives back what it does not keep, so do it
-    early, before the program's big allocations.  ``report`` holds what the sorting measured, ``verified``
+    early, before the program's big allocations.  ``chunk_bytes`` is the amount of memory judged as one piece
+    (4 GiB; smaller pieces copy too quickly to tell the regions apart reliably).  ``report`` holds what the sorting
+    measured; ``sort=False`` skips the timed copies and makes the striped range from chunks spread evenly over the
+    free memory (what is done anyway when the memory shows no regions); ``verified`` says
     whether copies between regions beat copies inside them on the finished ranges (on the probe chunks when there
     are no region ranges).
     Raises RuntimeError when too little memory is free, or when ranges of single regions are asked for and the
@@ -102,7 +105,7 @@ class HbmRegions:
     """
 
     def __init__(self, gib_per_region: float = 0.0, gib_striped: float = 48.0,
-                 device: Optional[torch.device] = None):
+                 device: Optional[torch.device] = None, chunk_bytes: int = CHUNK, sort: bool = True):
         from . import _hip
         self.device = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
         if self.device.type != "cuda":
@@ -111,6 +114,10 @@ class HbmRegions:
             self.device = torch.device("cuda", torch.cuda.current_device())
         if gib_per_region < 0 or gib_striped < 0 or (gib_per_region == 0 and gib_striped == 0):
             raise ValueError("gib_per_region and gib_striped must not be negative, and one of them positive")
+        if not sort and gib_per_region:
+            raise ValueError("ranges of single regions (gib_per_region) need the sorting")
+        if chunk_bytes <= 0 or chunk_bytes % (64 * 2 ** 20):
+            raise ValueError("chunk_bytes must be a multiple of the 64 MiB page")
         if gib_per_region + gib_striped / 3 > 80:
             raise ValueError("gib_per_region + gib_striped / 3 must not exceed 80 (rounded up to whole chunks of "
                              "4 GiB): that much is taken from each region, and a region has 96 GiB")
@@ -121,7 +128,8 @@ class HbmRegions:
             torch.cuda.empty_cache()                       # what torch has cached cannot be sorted
             torch.cuda.synchronize()
             rc = self._lib.exodus_hbm_regions_create(self.device.index, int(gib_per_region * GIB),
-                                                     int(gib_striped * GIB), CHUNK, ctypes.byref(rep))
+                                                     int(gib_striped * GIB), int(chunk_bytes), int(bool(sort)),
+                                                     ctypes.byref(rep))
         self.report: Dict[str, object] = {
             "chunks_examined": rep.chunks_examined, "kinds_found": rep.kinds_found,
             "chunks_ambiguous": rep.chunks_ambiguous, "chunks_of_region": list(rep.chunks_of_region),

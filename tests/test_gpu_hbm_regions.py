@@ -195,6 +195,25 @@ def test_striped_range_alone_is_made_of_whatever_memory_there_is(hbm):
     hbm.disable()
 
 
+def test_striped_range_without_sorting(hbm):
+    """``sort=False``: no timed copies; the striped range is made of chunks spread evenly over the free memory --
+    the same code that runs when the copies show no regions (memory left mixed by earlier processes) -- and holds
+    what is written to it; ranges of single regions cannot be had that way."""
+    regions = hbm.HbmRegions(gib_per_region=0.0, gib_striped=6.0, sort=False)
+    print(f"\nsorted: {regions.sorted}; {regions.report}")
+    assert regions.sorted is False and regions.verified is False and regions.report["kinds_found"] == 0
+    assert regions.sizes[hbm.STRIPED] == 12 * 2 ** 30 and regions.sizes[:3] == [0, 0, 0]   # three chunks of 4 GiB
+    t = regions.empty((2 ** 31,))                              # 8 GiB: pages of all three chunks
+    assert regions.pool_of(t) == hbm.STRIPED
+    pattern = torch.arange(2 ** 31, device=t.device, dtype=torch.int32) % 4099
+    t.copy_(pattern)
+    assert t.view(-1, 2 ** 15)[::37].eq(pattern.view(-1, 2 ** 15)[::37]).all()
+    del t, pattern
+    regions.close()
+    with pytest.raises(ValueError):
+        hbm.HbmRegions(gib_per_region=1.0, gib_striped=0.0, sort=False)
+
+
 def test_too_little_free_memory_is_refused(hbm):
     with pytest.raises(ValueError):
         hbm.HbmRegions(gib_per_region=96.0)
