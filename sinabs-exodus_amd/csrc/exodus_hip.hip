@@ -16,6 +16,10 @@
 // no workgroup barrier exists anywhere; ordering between the phases only needs the in-order
 // execution of one wave's LDS instructions plus a compiler fence.
 //
+// Two drivers implement this scheme: scan_span_kernel for rows whose length is a multiple of 4 in
+// 16-byte aligned tensors (raw buffer instructions on the wave's span of memory, sectors shared by two
+// rows written whole), scan_kernel for everything else (global loads, element-wise at row boundaries).
+//
 // Arithmetic of the forward recurrences is written with explicit round-to-nearest multiplies and
 // adds (no fused multiply-add), in the operation order of the reference device code, so spike
 // trains are reproducible bit for bit against a scalar CPU evaluation.
@@ -49,7 +53,6 @@ template <class T> __device__ __forceinline__ T ld_pick(const T *p, bool keep)
     return keep ? *p : ld_stream(p);
 }
 
-template <bool VEC>
 __device__ __forceinline__ f32x4 load4(const float *__restrict__ base, int64_t row, int64_t n_rows,
                                        int64_t t, int64_t n_steps, bool keep)
 {
@@ -57,9 +60,7 @@ __device__ __forceinline__ f32x4 load4(const float *__restrict__ base, int64_t r
     f32x4 v = f32x4{0.f, 0.f, 0.f, 0.f};
     if (row < n_rows) {
         const float *p = base + row * n_steps + t;
-        if (VEC) {
-            if (t >= 0 && t + 3 < n_steps) v = ld_pick(reinterpret_cast<const f32x4 *>(p), keep);
-        } else if (t >= 0 && t + 3 < n_steps && (reinterpret_cast<uintptr_t>(p) & 15u) == 0) {
+        if (t >= 0 && t + 3 < n_steps && (reinterpret_cast<uintptr_t>(p) & 15u) == 0) {
             // rows of any length: tiles are aligned to memory, so a chunk that lies inside its row is a
             // 16-byte aligned vector; only the chunks that straddle a row boundary go element by element
             v = ld_pick(reinterpret_cast<const f32x4 *>(p), keep);
@@ -73,15 +74,12 @@ __device__ __forceinline__ f32x4 load4(const float *__restrict__ base, int64_t r
     return v;
 }
 
-template <bool VEC>
 __device__ __forceinline__ void store4(float *__restrict__ base, int64_t row, int64_t n_rows, int64_t t,
                                        int64_t n_steps, f32x4 v)
 {
     if (row < n_rows) {
         float *p = base + row * n_steps + t;
-        if (VEC) {
-            if (t >= 0 && t + 3 < n_steps) st_stream(v, reinterpret_cast<f32x4 *>(p));
-        } else if (t >= 0 && t + 3 < n_steps && (reinterpret_cast<uintptr_t>(p) & 15u) == 0) {
+        if (t >= 0 && t + 3 < n_steps && (reinterpret_cast<uintptr_t>(p) & 15u) == 0) {
             st_stream(v, reinterpret_cast<f32x4 *>(p));
         } else {
             if (t + 0 >= 0 && t + 0 < n_steps) st_stream(v.x, p + 0);
@@ -114,7 +112,7 @@ __device__ __forceinline__ void put(f32x4 &v, int e, float x) { v[e] = x; }
 // load and store then moves whole aligned TT*4-byte segments, and only the first and last tile
 // of a row are partial (their out-of-row steps are masked per lane).
 // ---------------------------------------------------------------------------------------------
-template <class Op, int TT, bool VEC>
+template <class Op, int TT>
 __global__ void __launch_bounds__(WAVE) scan_kernel(const Op op, const int64_t n_rows, const int64_t n_steps,
                                                     const int64_t n_tiles, const int base_shift)
 {
@@ -163,7 +161,7 @@ __global__ void __launch_bounds__(WAVE) scan_kernel(const Op op, const int64_t n
             const int64_t t = tile * TT - mv_shift[i] + 4 * l_chunk;
 #pragma unroll
             for (int j = 0; j < NIN; ++j)
-                pre[j][i] = load4<VEC>(op.in[j], row0 + l_row + i * G::RPI, n_rows, t, n_steps, keep);
+                pre[j][i] = load4(op.in[j], row0 + l_row + i * G::RPI, n_rows, t, n_steps, keep);
         }
     };
 
@@ -235,10 +233,10 @@ __global__ void __launch_bounds__(WAVE) scan_kernel(const Op op, const int64_t n
 #pragma unroll
                 for (int j = 0; j < NOUT; ++j) {
                     const f32x4 v = *reinterpret_cast<const f32x4 *>(lds + j * TILE + G::off(l_row + i * G::RPI, l_chunk));
-                    store4<VEC>(op.out[j], row0 + l_row + i * G::RPI, n_rows, t, n_steps, v);
+                    store4(op.out[j], row0 + l_row + i * G::RPI, n_rows, t, n_steps, v);
                     if constexpr (NDER > 0) {
                         if (j == Op::DER_SRC)
-                            store4<VEC>(op.der, row0 + l_row + i * G::RPI, n_rows, t, n_steps,
+                            store4(op.der, row0 + l_row + i * G::RPI, n_rows, t, n_steps,
                                         op.derive(rowp + (l_row + i * G::RPI) * NROWP, v));
                     }
                 }
@@ -948,7 +946,7 @@ int launch_rows(const Op &op, int64_t n, int64_t t, bool vec, void *stream)
             return static_cast<int>(hipGetLastError());
         }
     }
-    hipLaunchKernelGGL((scan_kernel<Op, TT, false>), grid, block, lds_bytes, s, op, n, t, n_tiles, base_shift);
+    hipLaunchKernelGGL((scan_kernel<Op, TT>), grid, block, lds_bytes, s, op, n, t, n_tiles, base_shift);
     return static_cast<int>(hipGetLastError());
 }
 

@@ -158,7 +158,7 @@ def lifBackward(surr, outputGrad, notClipped, alpha, membrSubtract) -> torch.Ten
     _mat(_dev(notClipped, "notClipped", surr), "notClipped", n, t)
     _rows(_dev(alpha, "alpha", surr), "alpha", n)
     _rows(_dev(membrSubtract, "membrSubtract", surr), "membrSubtract", n)
-    inputGrad = torch.empty_like(surr)
+    inputGrad = hbm.empty_like(surr)
     with torch.cuda.device(surr.device):
         _check(lib.exodus_lif_backward(_ptr(inputGrad), _ptr(surr), _ptr(outputGrad), _ptr(notClipped),
                                        _ptr(alpha), _ptr(membrSubtract), n, t, _stream(surr)),
@@ -194,7 +194,7 @@ def leakyForward(input, vmemInitial, alpha, *, output=None) -> torch.Tensor:
     n, t = input.shape
     _rows(_dev(vmemInitial, "vmemInitial", input), "vmemInitial", n)
     _rows(_dev(alpha, "alpha", input), "alpha", n)
-    out = torch.empty_like(input) if output is None else _mat(_dev(output, "output", input), "output", n, t)
+    out = hbm.empty_like(input) if output is None else _mat(_dev(output, "output", input), "output", n, t)
     with torch.cuda.device(input.device):
         _check(lib.exodus_leaky_forward(_ptr(out), _ptr(input), _ptr(vmemInitial), _ptr(alpha), n, t,
                                         _stream(input)), "exodus_leaky_forward")
@@ -208,7 +208,7 @@ def leakyBackward(outputGrad, alpha) -> torch.Tensor:
         raise RuntimeError("outputGrad must be 2-D (rows, time)")
     n, t = outputGrad.shape
     _rows(_dev(alpha, "alpha", outputGrad), "alpha", n)
-    inputGrad = torch.empty_like(outputGrad)
+    inputGrad = hbm.empty_like(outputGrad)
     with torch.cuda.device(outputGrad.device):
         _check(lib.exodus_leaky_backward(_ptr(inputGrad), _ptr(outputGrad), _ptr(alpha), n, t,
                                          _stream(outputGrad)), "exodus_leaky_backward")
@@ -240,7 +240,7 @@ def spikeForward(vmem, alpha: float, membrSubtract: float, theta: float, thetaLo
     if vmem.ndim != 2:
         raise RuntimeError("vmem must be 2-D (rows, time)")
     n, t = vmem.shape
-    spikes = torch.empty_like(vmem)
+    spikes = hbm.empty_like(vmem)
     with torch.cuda.device(vmem.device):
         _check(lib.exodus_spike_forward(_ptr(spikes), _ptr(vmem), float(alpha), float(membrSubtract), float(theta),
                                         float(thetaLow), int(bool(applyThetaLow)), int(maxNumSpikes), n, t,
@@ -256,7 +256,7 @@ def spikeBackward(surr, outputGrad, notClipped, alpha: float, membrSubtract: flo
     n, t = surr.shape
     _mat(_dev(outputGrad, "outputGrad", surr), "outputGrad", n, t)
     _mat(_dev(notClipped, "notClipped", surr), "notClipped", n, t)
-    inputGrad = torch.empty_like(surr)
+    inputGrad = hbm.empty_like(surr)
     with torch.cuda.device(surr.device):
         _check(lib.exodus_spike_backward(_ptr(inputGrad), _ptr(surr), _ptr(outputGrad), _ptr(notClipped),
                                          float(alpha), float(membrSubtract), n, t, _stream(surr)),
@@ -280,7 +280,7 @@ def leakyBackwardFused(outputGrad, alpha, output=None, vmemInitial=None, needAlp
         _mat(_dev(output, "output", outputGrad), "output", n, t)
         _rows(_dev(vmemInitial, "vmemInitial", outputGrad), "vmemInitial", n)
     if inputGrad is None:
-        inputGrad = torch.empty_like(outputGrad)
+        inputGrad = hbm.empty_like(outputGrad)
     else:
         _mat(_dev(inputGrad, "inputGrad", outputGrad), "inputGrad", n, t)
     initGrad = torch.zeros_like(alpha)
@@ -321,7 +321,7 @@ def lifBackwardFused(gradSpikes, gradVmem, vmem, vmemPostInitial, alpha, membrSu
     else:
         surr = None
     if inputGrad is None:
-        inputGrad = torch.empty_like(vmem)
+        inputGrad = hbm.empty_like(vmem)
     else:
         _mat(_dev(inputGrad, "inputGrad", vmem), "inputGrad", n, t)
     initGrad = torch.zeros_like(alpha)
@@ -353,7 +353,7 @@ def synLifForward(input, vmemPostInitial, isynInitial, alphaMem, alphaSyn, membr
     else:
         thetaLow = None
     if out is None:
-        out = (torch.empty_like(input), torch.empty_like(input), torch.empty_like(input))
+        out = (hbm.empty_like(input), hbm.empty_like(input), hbm.empty_like(input))
     spikes, vmem, isyn = out
     for nm, x in (("spikes", spikes), ("vmem", vmem), ("isyn", isyn)):
         _mat(_dev(x, nm, input), nm, n, t)
@@ -390,7 +390,7 @@ def synLifBackward(gradSpikes, gradVmem, gradIsyn, vmem, isyn, vmemPostInitial, 
     else:
         thetaLow = None
     if inputGrad is None:
-        inputGrad = torch.empty_like(vmem)
+        inputGrad = hbm.empty_like(vmem)
     else:
         _mat(_dev(inputGrad, "inputGrad", vmem), "inputGrad", n, t)
     per_row = [torch.zeros_like(alphaMem) for _ in range(4)]

@@ -15,8 +15,8 @@ pages come from regions 0, 1, 2, 0, 1, 2, ... (``exodus_hbm_regions_create``, cs
 back to the driver.  ``HbmRegions`` hands out tensors from these ranges.
 
 ``empty(shape)`` allocates in the striped range, ``empty(shape, region=k)`` in the range of region k (0, 1, 2).
-After ``enable()`` the layer-layout wrappers (``_hip.layerLifForward`` and friends) allocate their outputs through
-``empty_like`` / ``empty`` of this module -- striped when there is a striped range; with region ranges only, in a
+After ``enable()`` the kernels' wrappers (``_hip.layerLifForward`` and friends, the (rows, time) wrappers, the
+``IntegrateAndFire`` Function) allocate their big outputs through ``empty_like`` / ``empty`` of this module -- striped when there is a striped range; with region ranges only, in a
 range that none of the tensors the kernel reads lies in (tensors of the ranges are recognised by their addresses;
 for a tensor from the ordinary allocator the range it copies to slowest is looked up once per storage with three
 short timed copies).  Without ``enable()`` nothing changes.  The reference has no counterpart (its CUDA

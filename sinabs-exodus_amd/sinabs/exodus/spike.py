@@ -20,7 +20,7 @@ from typing import Callable, Optional, Tuple, Union
 
 import torch
 
-from . import _hip
+from . import _hip, hbm
 from ._checks import check_per_row, check_rows_by_time
 from ._validate import check_parameters
 
@@ -88,8 +88,8 @@ class IntegrateAndFire(torch.autograd.Function):
 
         check_parameters([alpha], threshold, min_v_mem)      # alpha in [0, 1], threshold > min_v_mem
 
-        v_mem = torch.empty_like(inp)
-        output_spikes = torch.empty_like(inp)
+        v_mem = hbm.empty_like(inp)                # after hbm.enable(): in memory striped over the regions of HBM
+        output_spikes = hbm.empty_like(inp)
         max_spikes = -1 if max_num_spikes_per_bin is None else int(max_num_spikes_per_bin)
 
         _hip.lifForward(

@@ -74,7 +74,9 @@ def test_striped_range_takes_writes_faster_than_one_region(hbm):
     print(f"leaky forward into one region {into_one:.2f} TB/s, into the striped range {into_striped:.2f} TB/s")
     assert torch.equal(one_region, striped)
     assert into_striped > 1.08 * into_one
-    del one_region, striped
+    own = hip.leakyForward(x, zeros, alpha)                    # the wrapper's own allocation goes there as well
+    assert regions.pool_of(own) == hbm.STRIPED and torch.equal(own, striped)
+    del one_region, striped, own
     # the layer wrappers allocate in the striped range, and the values are what the ordinary allocator gives
     xs = x[:65536 * 4].view(4, 1024, 65536)
     f = hip.layerLifForward(xs, zeros[:4 * 65536], None, alpha[:4 * 65536], None, alpha[:4 * 65536] + 0.1,
