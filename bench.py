@@ -369,12 +369,13 @@ class Probes:
         self._call("exodus_probe_write", self._ptr(dst), dst.numel())
 
 
-def measure_ceilings(args, torch, hip, dev):
-    """GB/s of data-movement-only kernels on tensors of the chosen workload's shape."""
+def measure_ceilings(args, torch, hip, dev, place):
+    """GB/s of data-movement-only kernels on tensors of the chosen workload's shape, placed as the workload's are
+    (what is read as its inputs, what is written as its outputs)."""
     w = WORKLOADS[args.workload]
     B, T, M = w["batch"], w["steps"], w["neurons"]
     n = B * T * M
-    a = torch.randn(B, T, M, device=dev); b = torch.randn(B, T, M, device=dev); out = torch.empty_like(a)
+    a = place.empty((B, T, M), 0).normal_(); b = place.empty((B, T, M), 0).normal_(); out = place.empty((B, T, M), 1)
     alpha = torch.rand(B * M, device=dev) * 0.5 + 0.4
     zeros = torch.zeros(B * M, device=dev)
 
@@ -390,7 +391,8 @@ def measure_ceilings(args, torch, hip, dev):
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) / args.steps
 
-    res = {"workload": w["name"], "tensor_GB": n * 4 / 1e9, "peak_GBs": HBM_PEAK_GBS}
+    res = {"workload": w["name"], "tensor_GB": n * 4 / 1e9, "peak_GBs": HBM_PEAK_GBS, **place.describe()}
+    res.pop("placement_measured", None)
     probes = Probes(torch)
     ms = timed(lambda: probes.read(a))
     res["flat_read_only"] = {"ms": ms, "GBs": n * 4 / ms / 1e6}
@@ -707,7 +709,7 @@ def main():
         measure_reallocations(args, torch, hip, act, dev)
         return
     place = Placement(torch, dev)
-    if args.placement != "plain" and not (args.ceilings or args.conv_snn):
+    if args.placement != "plain" and not args.conv_snn:
         from sinabs.exodus import hbm
         try:
             if args.placement == "one-region":
@@ -738,15 +740,15 @@ def main():
         except RuntimeError as err:                     # device memory in use by something else: measure without
             plain_note = f"regions unavailable ({err}); ordinary allocator used"
             print("[bench] " + plain_note, file=sys.stderr, flush=True)
-    build = build_layer_workload if args.path == "layer" else build_workload
-    wl = build(args.workload, torch, hip, act, dev, place)
-    fwd, bwd, N, T = wl["fwd"], wl["bwd"], wl["N"], wl["T"]
     if args.ceilings:
-        print(json.dumps(measure_ceilings(args, torch, hip, dev)))
+        print(json.dumps(measure_ceilings(args, torch, hip, dev, place)))
         return
     if args.conv_snn:
         print(json.dumps(measure_conv_snn(args, torch, dev)))
         return
+    build = build_layer_workload if args.path == "layer" else build_workload
+    wl = build(args.workload, torch, hip, act, dev, place)
+    fwd, bwd, N, T = wl["fwd"], wl["bwd"], wl["N"], wl["T"]
 
     if args.copy_probe:
         src = torch.ones(1 << 28, device=dev)          # 2^28 floats = 1 GiB read + 1 GiB written
