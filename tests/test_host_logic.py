@@ -240,3 +240,35 @@ def test_parameter_validation_modes():
             val.set_mode("nonsense")
     finally:
         val.set_mode("sync")
+
+
+def test_hbm_range_bookkeeping_without_a_device():
+    """The free lists of sinabs.exodus.hbm (first fit, pieces of 2 MiB, neighbours joined on release) and its
+    argument checks, on an instance whose ranges are made up (no device memory behind them)."""
+    import threading
+    from sinabs.exodus import hbm
+    MIB = 2 ** 20
+    r = hbm.HbmRegions.__new__(hbm.HbmRegions)
+    r.bases = [1 << 40, 2 << 40, 3 << 40, 4 << 40]
+    r.sizes = [64 * MIB, 0, 64 * MIB, 256 * MIB]
+    r._free = [[[0, n]] for n in r.sizes]
+    r._lock, r._live, r._closing, r._closed = threading.Lock(), 0, False, True
+    a = r._take(3, 3 * MIB)                     # rounded up to 4 MiB
+    b = r._take(3, 2 * MIB)
+    c = r._take(3, 250 * MIB)
+    assert (a, b, c) == (0, 4 * MIB, 6 * MIB) and r.bytes_free(3) == 0 and r._live == 3
+    assert r._take(3, 1) is None and r._take(1, 1) is None          # full; a range that does not exist
+    r._give_back(3, b, 2 * MIB)
+    r._give_back(3, a, 4 * MIB)                 # joins the piece behind it
+    assert r._free[3] == [[0, 6 * MIB]] and r._take(3, 5 * MIB) == 0
+    r._give_back(3, c, 250 * MIB)
+    r._give_back(3, 0, 6 * MIB)                 # joins the piece after it: one free range again
+    assert r._free[3] == [[0, 256 * MIB]] and r._live == 0
+    assert r._take(0, 64 * MIB) == 0 and r._take(0, 2 * MIB) is None
+    for bad in (dict(gib_per_region=-1.0), dict(gib_per_region=0.0, gib_striped=0.0), dict(gib_per_region=70.0, gib_striped=48.0),
+                dict(gib_per_region=1.0, sort=False), dict(chunk_bytes=100 * MIB)):
+        with pytest.raises((ValueError, RuntimeError)):      # RuntimeError: no device in this process
+            hbm.HbmRegions(**bad)
+    assert hbm.active() is None
+    like = torch.zeros(4, 5)
+    assert hbm.empty_like(like).shape == like.shape and hbm.empty((2, 3), like).shape == (2, 3)   # not enabled: torch's
