@@ -235,3 +235,19 @@ def test_one_way_streaming_probes():
     assert torch.equal(dst, a)
     probes.stream(dst, a, b)
     assert torch.equal(dst, a + b)
+
+
+@pytest.mark.parametrize("n,t", [(64, 1 << 22), (65, (1 << 22) - 4), (3, (1 << 22) + 4)])
+def test_longest_rows_of_the_span_driver_and_the_first_beyond(hip, ref, n, t):
+    """Rows of 2^22 steps: a wave's 64 rows are exactly the 2^30 bytes that the raw-buffer driver's 32-bit
+    offsets cover; 2^22 - 4 steps puts row boundaries inside 64-byte sectors at that size; rows of 2^22 + 4 steps
+    take the driver with full address arithmetic.  Leaky integrator forward and its reverse pass, bit for bit."""
+    g = gen(t % 1000 + n)
+    x = torch.randn(n, t, generator=g) * 0.3; v0 = torch.randn(n, generator=g)
+    a = 0.9 + 0.1 * torch.rand(n, generator=g)
+    out = hip.leakyForward(D(x), D(v0), D(a))
+    want = ref.leaky_forward(x, v0, a)
+    assert torch.equal(out.cpu(), want)
+    del out
+    gi = hip.leakyBackward(D(x), D(a))                       # the same tensor as incoming gradient
+    assert torch.equal(gi.cpu(), ref.leaky_backward(x, a))
