@@ -37,13 +37,16 @@ namespace {
 #ifndef EXODUS_LAYER_BWD_BLOCK
 #define EXODUS_LAYER_BWD_BLOCK 256    // lanes per block of the spiking backward kernel (one neuron per lane)
 #endif
+#ifndef EXODUS_LAYER_CKPT
+#define EXODUS_LAYER_CKPT 32          // steps between checkpoints (a multiple of 2 * EXODUS_LAYER_FWD_UNROLL)
+#endif
 #ifndef EXODUS_WHOLE_NEURONS
 #define EXODUS_WHOLE_NEURONS 16       // neurons per step must be a multiple of this for the non-temporal kernel instances
 #endif
 #ifndef EXODUS_LAYER_BWD_WAVES
 #define EXODUS_LAYER_BWD_WAVES 3      // resident waves per SIMD the backward kernel is compiled for
 #endif
-constexpr int CKPT = 32;                             // steps between checkpoints = length of a backward chunk
+constexpr int CKPT = EXODUS_LAYER_CKPT;               // steps between checkpoints = length of a backward chunk
 constexpr int FWD_UNROLL = EXODUS_LAYER_FWD_UNROLL;  // forward steps per software-pipeline stage (divides CKPT)
 constexpr int BLOCK = EXODUS_LAYER_BLOCK;
 constexpr int BWD_BLOCK = EXODUS_LAYER_BWD_BLOCK;
