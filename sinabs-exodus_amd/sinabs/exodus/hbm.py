@@ -287,12 +287,13 @@ _active: Optional[HbmRegions] = None
 
 
 def enable(gib_per_region: float = 0.0, gib_striped: float = 48.0,
-           device: Optional[torch.device] = None) -> HbmRegions:
-    """Create the ranges and make the layer-layout kernels' wrappers allocate their outputs through them."""
+           device: Optional[torch.device] = None, **how) -> HbmRegions:
+    """Create the ranges (``HbmRegions(gib_per_region, gib_striped, device, **how)``) and make the kernels' wrappers
+    allocate their outputs through them."""
     global _active
     if _active is not None:
         disable()
-    _active = HbmRegions(gib_per_region, gib_striped, device)
+    _active = HbmRegions(gib_per_region, gib_striped, device, **how)
     return _active
 
 

@@ -41,6 +41,64 @@ def sorted_ranges(hbm, **sizes):
     return regions
 
 
+def test_outputs_go_to_another_pool_and_results_do_not_change(hbm):
+    """Ranges of single regions only (no striped range): the wrappers put what they write into another region than
+    what they read.  Runs first: it allocates in chunks of 4 GiB only, which leaves the driver's memory in order."""
+    from sinabs.exodus import _hip as hip
+    dev = torch.device("cuda:0")
+    B, T, M = 4, 300, 65536                                   # 300 MiB per tensor: large enough to be classified
+    n = B * M
+    x_plain = (torch.randn(B, T, M, generator=gen(3)) * 0.5 + 0.05).to(dev)
+    go_plain = torch.rand(B, T, M, generator=gen(4)).to(dev)
+    full = lambda v: torch.full((n,), float(v), device=dev)
+    zeros = torch.zeros(n, device=dev)
+    a_mem, a_syn, one, lo = full(0.95), full(0.8), full(1.0), full(-1.0)
+
+    def run(x, go):
+        f = hip.layerLifForward(x, zeros, zeros, a_mem, a_syn, one, one, lo, True, 2, True, True)
+        g = hip.layerLifBackward(go, None, None, x, f["ckpt_v"], f["ckpt_i"], zeros, zeros, a_mem, a_syn, one, one,
+                                 lo, True, 2, True, True, hip.SURR_SINGLE_EXP, 0.5, 1.0)
+        leak, _ = hip.layerLeakyForward(x, zeros, a_mem, False, False)
+        gl = hip.layerLeakyBackward(go, None, leak, x, zeros, a_mem, False, False, True)
+        return f, g, leak, gl
+
+    want_f, want_g, want_leak, want_gl = run(x_plain, go_plain)
+    assert want_f["spikes"].sum().item() > 0
+
+    regions = sorted_ranges(hbm, gib_per_region=8.0, gib_striped=0.0)
+    assert hbm.active() is regions
+    x = regions.empty((B, T, M), region=0).copy_(x_plain)
+    go = regions.empty((B, T, M), region=0).copy_(go_plain)
+    assert regions.pool_of(x) == 0 and regions.region_of(go) == 0 and regions.pool_of(x_plain) is None
+    f, g, leak, gl = run(x, go)
+    assert regions.pool_of(f["spikes"]) in (1, 2)
+    assert regions.pool_of(f["ckpt_v"]) in (1, 2) and regions.pool_of(f["ckpt_v"]) != regions.pool_of(f["spikes"])
+    assert regions.pool_of(g[0]) in (1, 2)                     # grad_input: away from grad_output and the input
+    assert regions.pool_of(leak) in (1, 2)
+    assert regions.pool_of(gl[0]) == 3 - regions.pool_of(leak)  # reads pool 0 and the output's pool, writes the third
+    for k in ("spikes", "v_last", "i_last", "ckpt_v", "ckpt_i", "spike_sum"):
+        assert torch.equal(f[k], want_f[k]), k
+    for got, want in zip(list(g) + [leak] + list(gl), list(want_g) + [want_leak] + list(want_gl)):
+        assert (got is None) == (want is None)
+        if got is not None:
+            assert torch.equal(got, want)
+
+    # inputs from the ordinary allocator are classified by timed copies, once per storage; the result still
+    # lands in one of the pools, and the values are the same
+    k = regions.region_of(x_plain)
+    assert k in (0, 1, 2) and regions.region_of(x_plain) == k
+    f2 = hip.layerLifForward(x_plain, zeros, zeros, a_mem, a_syn, one, one, lo, True, 2, True, True)
+    assert regions.pool_of(f2["spikes"]) not in (None, k)
+    assert torch.equal(f2["spikes"], want_f["spikes"])
+    small = torch.zeros(2, 8, 64, device=dev)
+    assert regions.region_of(small) is None                    # too small to time or to matter
+
+    hbm.disable()
+    assert hbm.active() is None
+    again = hip.layerLifForward(x_plain, zeros, zeros, a_mem, a_syn, one, one, lo, True, 2, True, True)
+    assert torch.equal(again["spikes"], want_f["spikes"])
+
+
 def test_ranges_of_one_region_each_and_a_striped_range_that_takes_writes_faster(hbm):
     """Copies between the regions' ranges beat copies inside one range, whatever this process and earlier ones have
     done to the order in which the driver hands out memory.  The striped range: the wrappers' outputs go there,
@@ -115,62 +173,6 @@ def test_ranges_of_one_region_each_and_a_striped_range_that_takes_writes_faster(
     assert x[:4].sum().isfinite() and regions.pool_of(regions.empty((2 ** 20,), region=0)) is None
 
 
-def test_outputs_go_to_another_pool_and_results_do_not_change(hbm):
-    from sinabs.exodus import _hip as hip
-    dev = torch.device("cuda:0")
-    B, T, M = 4, 300, 65536                                   # 300 MiB per tensor: large enough to be classified
-    n = B * M
-    x_plain = (torch.randn(B, T, M, generator=gen(3)) * 0.5 + 0.05).to(dev)
-    go_plain = torch.rand(B, T, M, generator=gen(4)).to(dev)
-    full = lambda v: torch.full((n,), float(v), device=dev)
-    zeros = torch.zeros(n, device=dev)
-    a_mem, a_syn, one, lo = full(0.95), full(0.8), full(1.0), full(-1.0)
-
-    def run(x, go):
-        f = hip.layerLifForward(x, zeros, zeros, a_mem, a_syn, one, one, lo, True, 2, True, True)
-        g = hip.layerLifBackward(go, None, None, x, f["ckpt_v"], f["ckpt_i"], zeros, zeros, a_mem, a_syn, one, one,
-                                 lo, True, 2, True, True, hip.SURR_SINGLE_EXP, 0.5, 1.0)
-        leak, _ = hip.layerLeakyForward(x, zeros, a_mem, False, False)
-        gl = hip.layerLeakyBackward(go, None, leak, x, zeros, a_mem, False, False, True)
-        return f, g, leak, gl
-
-    want_f, want_g, want_leak, want_gl = run(x_plain, go_plain)
-    assert want_f["spikes"].sum().item() > 0
-
-    regions = sorted_ranges(hbm, gib_per_region=8.0, gib_striped=0.0)
-    assert hbm.active() is regions
-    x = regions.empty((B, T, M), region=0).copy_(x_plain)
-    go = regions.empty((B, T, M), region=0).copy_(go_plain)
-    assert regions.pool_of(x) == 0 and regions.region_of(go) == 0 and regions.pool_of(x_plain) is None
-    f, g, leak, gl = run(x, go)
-    assert regions.pool_of(f["spikes"]) in (1, 2)
-    assert regions.pool_of(f["ckpt_v"]) in (1, 2) and regions.pool_of(f["ckpt_v"]) != regions.pool_of(f["spikes"])
-    assert regions.pool_of(g[0]) in (1, 2)                     # grad_input: away from grad_output and the input
-    assert regions.pool_of(leak) in (1, 2)
-    assert regions.pool_of(gl[0]) == 3 - regions.pool_of(leak)  # reads pool 0 and the output's pool, writes the third
-    for k in ("spikes", "v_last", "i_last", "ckpt_v", "ckpt_i", "spike_sum"):
-        assert torch.equal(f[k], want_f[k]), k
-    for got, want in zip(list(g) + [leak] + list(gl), list(want_g) + [want_leak] + list(want_gl)):
-        assert (got is None) == (want is None)
-        if got is not None:
-            assert torch.equal(got, want)
-
-    # inputs from the ordinary allocator are classified by timed copies, once per storage; the result still
-    # lands in one of the pools, and the values are the same
-    k = regions.region_of(x_plain)
-    assert k in (0, 1, 2) and regions.region_of(x_plain) == k
-    f2 = hip.layerLifForward(x_plain, zeros, zeros, a_mem, a_syn, one, one, lo, True, 2, True, True)
-    assert regions.pool_of(f2["spikes"]) not in (None, k)
-    assert torch.equal(f2["spikes"], want_f["spikes"])
-    small = torch.zeros(2, 8, 64, device=dev)
-    assert regions.region_of(small) is None                    # too small to time or to matter
-
-    hbm.disable()
-    assert hbm.active() is None
-    again = hip.layerLifForward(x_plain, zeros, zeros, a_mem, a_syn, one, one, lo, True, 2, True, True)
-    assert torch.equal(again["spikes"], want_f["spikes"])
-
-
 def test_striped_range_alone_is_made_of_whatever_memory_there_is(hbm):
     """Only a striped range: made whether or not the memory shows regions, usable, and given back."""
     regions = hbm.enable(gib_per_region=0.0, gib_striped=12.0)
@@ -185,6 +187,47 @@ def test_striped_range_alone_is_made_of_whatever_memory_there_is(hbm):
     assert regions.pool_of(u) is None
     del t, u
     hbm.disable()
+
+
+def test_layers_and_functions_give_the_same_results_from_the_striped_range(hbm):
+    """A small network of the public layers and the IntegrateAndFire Function, forward and backward, with and without
+    ``hbm.enable()``: every output and gradient bit for bit the same (the range only changes where tensors lie)."""
+    import torch.nn as nn
+    import sinabs.exodus.layers as el
+    from sinabs.exodus.spike import IntegrateAndFire
+    from sinabs.exodus._compat import activation as act
+    dev = torch.device("cuda:0")
+    torch.manual_seed(3)
+    net = nn.Sequential(el.LIF(tau_mem=20.0, tau_syn=5.0, min_v_mem=-1.0, spike_fn=act.MaxSpike(2), train_alphas=True),
+                        el.IAF()).to(dev)
+    x = (torch.rand(8, 200, 4096, generator=gen(12)) * 0.8).to(dev).requires_grad_(True)    # 26 MB per tensor
+    rows = (torch.randn(4096, 512, generator=gen(13)) * 0.6 + 0.2).to(dev)  # (rows, time) tensors of 8 MiB
+    alpha = torch.full((4096,), 0.9, device=dev); ones = torch.ones(4096, device=dev)
+
+    def run():
+        for m in net:
+            if hasattr(m, "reset_states"):
+                m.reset_states()
+        net.zero_grad(set_to_none=True)
+        x.grad = None
+        out = net(x)
+        out.sum().backward()
+        inp = rows.clone().requires_grad_(True)
+        s, v = IntegrateAndFire.apply(inp, alpha, torch.zeros_like(alpha), ones, ones, None, act.SingleExponential(), None)
+        (s.sum() + 0.1 * v.sum()).backward()
+        return [out.detach(), x.grad, s.detach(), v.detach(), inp.grad] + [p.grad for p in net.parameters()], (out, s)
+
+    want, _ = run()
+    assert want[0].sum().item() > 0 and want[2].sum().item() > 0 and want[1].abs().sum().item() > 0
+    regions = hbm.enable(gib_per_region=0.0, gib_striped=6.0, sort=False)
+    got, (out, s) = run()
+    assert regions.pool_of(s) == hbm.STRIPED and regions.pool_of(out) == hbm.STRIPED
+    assert regions.pool_of(net[1].v_mem) is None               # states are small: the ordinary allocator
+    same = lambda p, q: all((a is None and b is None) or torch.equal(a, b) for a, b in zip(p, q))
+    assert len(got) == len(want) and same(got, want) and sum(g is not None for g in got) >= 7
+    hbm.disable()
+    again, _ = run()
+    assert same(again, want)
 
 
 def test_striped_range_without_sorting(hbm):
