@@ -220,6 +220,36 @@ def test_bench_child_command_line_drops_the_cycle_option():
     assert f(["--workload", "c3"]) == ["--workload", "c3"]
 
 
+def test_bench_placement_modes_choose_the_ranges():
+    """bench.py's Placement: which range of sinabs.exodus.hbm each kind of tensor (0 = read, 1 / 2 = written) is asked
+    from in every mode, and that the roofline's traffic figures name a committed profile."""
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("bench", os.path.join(ROOT, "bench.py"))
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+
+    class Ranges:
+        verified, report = True, {"chunks_examined": 70, "inside_one_range_GBs": [5900.4, 6000.0, 6100.0]}
+
+        def empty(self, shape, region):
+            return ("range", region, tuple(shape))
+
+    asked = lambda mode, k: bench.Placement(torch, "cpu", Ranges(), mode=mode).empty((2, 3), k)[1]
+    assert [asked("striped", k) for k in (0, 1, 2)] == [0, 3, 3]
+    assert [asked("all-striped", k) for k in (0, 1, 2)] == [3, 3, 3]
+    assert [asked("regions", k) for k in (0, 1, 2)] == [0, 1, 2]
+    assert [asked("one-region", k) for k in (0, 1, 2)] == [0, 0, 0]
+    plain = bench.Placement(torch, "cpu")
+    assert plain.empty((2, 3), 1).shape == (2, 3) and plain.describe() == {"placement": "ordinary allocator"}
+    d = bench.Placement(torch, "cpu", Ranges(), mode="striped").describe()
+    assert "striped" not in d["placement"] or "alternate" in d["placement"]
+    assert d["placement_measured"]["inside_one_range_GBs"] == [5900, 6000, 6100] and d["placement_verified_by_timed_copies"]
+    for (_, _), (nbytes, source) in bench.MEASURED_TRAFFIC.items():
+        assert nbytes > 1e9 and source.startswith("profiles/")
+        if os.path.isdir(os.path.join(ROOT, "profiles")):       # (the summaries do not travel to the GPU box)
+            assert os.path.exists(os.path.join(ROOT, source)), source
+
+
 def test_parameter_validation_modes():
     from sinabs.exodus import _validate as val
     good, bad = torch.tensor([0.0, 0.5, 1.0]), torch.tensor([0.5, 1.5])
