@@ -39,6 +39,10 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));    // one 16-byte chunk
 #ifndef EXODUS_SPAN_UNROLL_Q
 #define EXODUS_SPAN_UNROLL_Q 2
 #endif
+// bytes of LDS asked for beyond what the span driver uses (an experiment's knob: fewer waves fit a CU)
+#ifndef EXODUS_SPAN_EXTRA_LDS
+#define EXODUS_SPAN_EXTRA_LDS 0
+#endif
 // 64-byte sectors shared by two rows of a wave are written in one piece (0: each row writes its part)
 #ifndef EXODUS_WHOLE_SECTORS
 #define EXODUS_WHOLE_SECTORS 1

@@ -941,7 +941,7 @@ int launch_rows(const Op &op, int64_t n, int64_t t, bool vec, void *stream)
             const int whole_sectors = EXODUS_WHOLE_SECTORS && Op::NOUT > 0 && t > TT && (t % 16 != 0 || base_shift % 16 != 0);
             const size_t lds_kept = whole_sectors ? static_cast<size_t>(Op::NOUT) * WAVE * 16 * sizeof(float) : 0;
             hipLaunchKernelGGL((scan_span_kernel<Op, TT, SpanPlan<Op>::UQ, SpanPlan<Op>::WPE>), grid, block,
-                               lds_bytes + lds_kept, s, op, n, static_cast<int>(t), static_cast<int>(n_tiles), base_shift,
+                               lds_bytes + lds_kept + EXODUS_SPAN_EXTRA_LDS, s, op, n, static_cast<int>(t), static_cast<int>(n_tiles), base_shift,
                                whole_sectors);
             return static_cast<int>(hipGetLastError());
         }
