@@ -680,10 +680,13 @@ def main():
         import subprocess
 
         def child_run(placement):
-            child = subprocess.run([sys.executable, os.path.abspath(__file__), "--placement", placement, "--no-others",
-                                    "--no-cpu-baseline", "--workload", args.workload, "--path", args.path,
-                                    "--steps", str(args.steps), "--warmup", str(args.warmup)],
-                                   capture_output=True, text=True)
+            try:
+                child = subprocess.run([sys.executable, os.path.abspath(__file__), "--placement", placement, "--no-others",
+                                        "--no-cpu-baseline", "--workload", args.workload, "--path", args.path,
+                                        "--steps", str(args.steps), "--warmup", str(args.warmup)],
+                                       capture_output=True, text=True, timeout=240)
+            except subprocess.TimeoutExpired:
+                return {"error": "no result within 240 s"}
             try:
                 r = json.loads(child.stdout.strip().splitlines()[-1])["roofline"]
                 return {"frac": r["frac"], "fwd_bwd_combined_frac": r["fwd_bwd_combined_frac"],
