@@ -37,6 +37,9 @@ namespace {
 #ifndef EXODUS_LAYER_BWD_BLOCK
 #define EXODUS_LAYER_BWD_BLOCK 256    // lanes per block of the spiking backward kernel (one neuron per lane)
 #endif
+#ifndef EXODUS_LEAKY_WAVES
+#define EXODUS_LEAKY_WAVES 8          // waves per CU the leaky kernels want before a lane takes more than one neuron
+#endif
 #ifndef EXODUS_LAYER_CKPT
 #define EXODUS_LAYER_CKPT 32          // steps between checkpoints (a multiple of 2 * EXODUS_LAYER_FWD_UNROLL)
 #endif
@@ -1185,7 +1188,7 @@ EXODUS_API int exodus_layer_leaky_forward(float *out, float *v_last, double *out
     p.alpha = alpha;
     p.decay_early = decay_early ? 1 : 0;
     p.norm_input = norm_input ? 1 : 0;
-    const int npl = pick_neurons_per_lane(batch, neurons, common_alignment({input, out}), 4, 8);
+    const int npl = pick_neurons_per_lane(batch, neurons, common_alignment({input, out}), 4, EXODUS_LEAKY_WAVES);
     const int64_t blocks_per_batch = (neurons + BLOCK * npl - 1) / (BLOCK * npl);
     if (blocks_per_batch > 0x7fffffffLL / batch) return hipErrorInvalidValue;
     const dim3 grid(static_cast<unsigned>(blocks_per_batch * batch)), block(BLOCK);
@@ -1226,7 +1229,7 @@ EXODUS_API int exodus_layer_leaky_backward(float *grad_input, float *alpha_grad,
     p.norm_input = norm_input ? 1 : 0;
     // with the alpha gradient two or three tensors are double-buffered: two neurons per lane at most
     const int npl = pick_neurons_per_lane(batch, neurons, common_alignment({grad_input, grad_out, out, input}),
-                                          want_alpha ? 2 : 4, 8);
+                                          want_alpha ? 2 : 4, EXODUS_LEAKY_WAVES);
     const int64_t blocks_per_batch = (neurons + BLOCK * npl - 1) / (BLOCK * npl);
     if (blocks_per_batch > 0x7fffffffLL / batch) return hipErrorInvalidValue;
     const dim3 grid(static_cast<unsigned>(blocks_per_batch * batch)), block(BLOCK);
