@@ -36,6 +36,9 @@ import torch
 
 GIB = 2 ** 30
 CHUNK = 4 * GIB                 # physical memory is sorted in pieces of this size: shorter copies tell less
+FINER_CHUNK = 256 * 2 ** 20     # ... and in pieces of this size when the big ones show no regions (memory that earlier
+                                # processes left mixed below 4 GiB is mostly still in order at this scale)
+REGIONS_NOT_FOUND = -3          # EXODUS_ERROR_REGIONS_NOT_FOUND of include/exodus_hip.h
 ALIGN = 2 * 2 ** 20             # every tensor of a range starts on a 2 MiB boundary
 PROBES = 15                     # EXODUS_HBM_PROBES of include/exodus_hip.h
 ARENAS = 4                      # EXODUS_HBM_ARENAS: one range per region and the striped one
@@ -73,6 +76,22 @@ class _Block:
             pass
 
 
+def _create(lib, device_index: int, bytes_per_region: int, bytes_striped: int, chunk_sizes: Sequence[int], sort: bool):
+    """``exodus_hbm_regions_create`` with each of ``chunk_sizes`` in turn until one shows the regions (or none is
+    left); returns (status, report, chunk size used).  A striped range that came out unsorted is given back before
+    the next try."""
+    for attempt, size in enumerate(chunk_sizes):
+        rep = _Report()
+        rc = lib.exodus_hbm_regions_create(device_index, bytes_per_region, bytes_striped, int(size), int(sort),
+                                           ctypes.byref(rep))
+        no_regions = rc == REGIONS_NOT_FOUND or (rc == 0 and sort and rep.kinds_found != 3)
+        if not no_regions or attempt + 1 == len(chunk_sizes):
+            break
+        if rc == 0:
+            lib.exodus_hbm_regions_destroy(device_index)
+    return rc, rep, int(size)
+
+
 def _copy_rate(dst: torch.Tensor, src: torch.Tensor, reps: int = 5) -> float:
     """bytes moved per millisecond by dst.copy_(src), median of `reps` (events on the current stream)"""
     dst.copy_(src)
@@ -95,7 +114,8 @@ class HbmRegions:
     serve is passed to the ordinary allocator, which is harmless but loses the placement.  Creating the ranges
     takes nearly all free device memory for a second or two and gives back what it does not keep, so do it
     early, before the program's big allocations.  ``chunk_bytes`` is the amount of memory judged as one piece
-    (4 GiB; smaller pieces copy too quickly to tell the regions apart reliably).  ``report`` holds what the sorting
+    (4 GiB; smaller pieces copy too quickly to tell the regions apart as reliably); when pieces of that size show no
+    regions -- memory that earlier processes left mixed -- the sorting is repeated once with ``finer_chunk_bytes``.  ``report`` holds what the sorting
     measured; ``sort=False`` skips the timed copies and makes the striped range from chunks spread evenly over the
     free memory (what is done anyway when the memory shows no regions); ``verified`` says
     whether copies between regions beat copies inside them on the finished ranges (on the probe chunks when there
@@ -105,7 +125,8 @@ class HbmRegions:
     """
 
     def __init__(self, gib_per_region: float = 0.0, gib_striped: float = 48.0,
-                 device: Optional[torch.device] = None, chunk_bytes: int = CHUNK, sort: bool = True):
+                 device: Optional[torch.device] = None, chunk_bytes: int = CHUNK, sort: bool = True,
+                 finer_chunk_bytes: Optional[int] = FINER_CHUNK):
         from . import _hip
         self.device = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
         if self.device.type != "cuda":
@@ -122,14 +143,16 @@ class HbmRegions:
             raise ValueError("gib_per_region + gib_striped / 3 must not exceed 80 (rounded up to whole chunks of "
                              "4 GiB): that much is taken from each region, and a region has 96 GiB")
         self._lib = _hip.lib
-        rep = _Report()
+        sizes = [int(chunk_bytes)]
+        if sort and finer_chunk_bytes and finer_chunk_bytes < chunk_bytes:
+            sizes.append(int(finer_chunk_bytes))
         with torch.cuda.device(self.device):
             torch.zeros(1, device=self.device)             # the device's context exists
             torch.cuda.empty_cache()                       # what torch has cached cannot be sorted
             torch.cuda.synchronize()
-            rc = self._lib.exodus_hbm_regions_create(self.device.index, int(gib_per_region * GIB),
-                                                     int(gib_striped * GIB), int(chunk_bytes), int(bool(sort)),
-                                                     ctypes.byref(rep))
+            rc, rep, size = _create(self._lib, self.device.index, int(gib_per_region * GIB), int(gib_striped * GIB),
+                                    sizes, bool(sort))
+        self.chunk_bytes = size                            # the size the ranges were sorted in
         self.report: Dict[str, object] = {
             "chunks_examined": rep.chunks_examined, "kinds_found": rep.kinds_found,
             "chunks_ambiguous": rep.chunks_ambiguous, "chunks_of_region": list(rep.chunks_of_region),

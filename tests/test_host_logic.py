@@ -299,6 +299,34 @@ def test_hbm_range_bookkeeping_without_a_device():
                 dict(gib_per_region=1.0, sort=False), dict(chunk_bytes=100 * MIB)):
         with pytest.raises((ValueError, RuntimeError)):      # RuntimeError: no device in this process
             hbm.HbmRegions(**bad)
+    # sorting is tried again with finer pieces when the big ones show no regions
+    class Lib:
+        def __init__(self, outcomes):
+            self.outcomes, self.calls, self.destroyed = list(outcomes), [], 0
+
+        def exodus_hbm_regions_create(self, dev, per_region, striped, chunk, sort, rep_ref):
+            self.calls.append(chunk)
+            rc, kinds = self.outcomes.pop(0)
+            rep_ref._obj.kinds_found = kinds
+            return rc
+
+        def exodus_hbm_regions_destroy(self, dev):
+            self.destroyed += 1
+            return 0
+
+    sizes = [4096 * MIB, 256 * MIB]
+    lib = Lib([(0, 3)])
+    assert hbm._create(lib, 0, 0, 1, sizes, True)[::2] == (0, 4096 * MIB) and lib.calls == [4096 * MIB]
+    lib = Lib([(hbm.REGIONS_NOT_FOUND, 2), (0, 3)])
+    rc, rep, size = hbm._create(lib, 0, 1, 1, sizes, True)
+    assert (rc, rep.kinds_found, size) == (0, 3, 256 * MIB) and lib.destroyed == 0
+    lib = Lib([(0, 2), (0, 1)])                                   # a striped range alone, unsorted both times
+    rc, rep, size = hbm._create(lib, 0, 0, 1, sizes, True)
+    assert (rc, rep.kinds_found, size) == (0, 1, 256 * MIB) and lib.destroyed == 1
+    lib = Lib([(2, 0)])                                           # any other error ends the tries
+    assert hbm._create(lib, 0, 1, 1, sizes, True)[0] == 2 and lib.calls == [4096 * MIB]
+    lib = Lib([(0, 0)])
+    assert hbm._create(lib, 0, 0, 1, sizes[:1], False)[::2] == (0, 4096 * MIB)   # no sorting asked for: one call
     assert hbm.active() is None
     like = torch.zeros(4, 5)
     assert hbm.empty_like(like).shape == like.shape and hbm.empty((2, 3), like).shape == (2, 3)   # not enabled: torch's
