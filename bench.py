@@ -8,7 +8,10 @@ already lives in HBM, called through the C ABI of libexodus_hip.so with prealloc
 Prints ONE JSON line: neuron-timesteps/s (rows * time steps / wall time of fwd+bwd), the HBM
 roofline of the slowest kernel (algorithmic bytes / its mean duration, measured with events on
 the launch stream) and a CPU baseline (the sinabs-style per-time-step torch loop with autograd,
-timed on this machine's host cores on a bounded sample of the same workload).
+timed on this machine's host cores on a bounded sample of the same workload).  Under "others" the
+same line carries the other configurations, the (rows, time) kernels, and every configuration
+through the public layer API (``sinabs.exodus.layers``: autograd, outputs allocated per call),
+each with the figures of the ordinary allocator beside those of ``sinabs.exodus.hbm.enable()``.
 """
 import argparse
 import contextlib
@@ -42,66 +45,66 @@ WORKLOADS = {
                batch=8, steps=100, neurons=256, mean=None, std=None, bytes=(12, 12)),
 }
 
-# HBM traffic per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (FETCH_SIZE x2 + WRITE_SIZE
-# x1 KiB, factors from a plain elementwise kernel over exactly 1 GiB in the same runs): bytes per launch
-# and the committed summary the figure comes from.  These are measurements of the kernels as they were
-# when the summary was made; a kernel that changes needs its counters taken again.
-MEASURED_TRAFFIC = {
-    ("c5", "exodus_layer_lif_backward"): (25.74e9, "profiles/all_workloads_striped_placement_kernel_stats_pmc.md"),
-    ("c5", "exodus_layer_lif_forward"): (17.34e9, "profiles/all_workloads_striped_placement_kernel_stats_pmc.md"),
-    ("c5", "exodus_synlif_backward"): (33.79e9, "profiles/all_workloads_striped_placement_kernel_stats_pmc.md"),
-    ("c5", "exodus_synlif_forward"): (33.64e9, "profiles/all_workloads_striped_placement_kernel_stats_pmc.md"),
-    ("c2", "exodus_layer_lif_backward"): (15.38e9, "profiles/all_workloads_striped_placement_kernel_stats_pmc.md"),
-    ("c2", "exodus_layer_lif_forward"): (10.30e9, "profiles/all_workloads_striped_placement_kernel_stats_pmc.md"),
-    ("c3", "exodus_layer_leaky_backward"): (3.15e9, "profiles/all_workloads_striped_placement_kernel_stats_pmc.md"),
-    ("c3", "exodus_layer_leaky_forward"): (2.10e9, "profiles/all_workloads_striped_placement_kernel_stats_pmc.md"),
-    ("c2", "exodus_lif_forward"): (15.75e9, "profiles/all_workloads_striped_placement_kernel_stats_pmc.md"),
-    ("c2", "exodus_lif_backward_fused"): (16.06e9, "profiles/all_workloads_striped_placement_kernel_stats_pmc.md"),
-    ("c3", "exodus_leaky_forward"): (2.12e9, "profiles/all_workloads_striped_placement_kernel_stats_pmc.md"),
-    ("c3", "exodus_leaky_backward_fused"): (3.20e9, "profiles/all_workloads_striped_placement_kernel_stats_pmc.md"),
-}
+# HBM traffic per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by what the same counters
+# read for a plain elementwise kernel over exactly 1 GiB in the same runs: bytes per launch by (workload, entry
+# point), and the committed summary each figure comes from.  bench_profile.py writes the file from the raw counter
+# output when it writes a summary, so the figures cannot drift from the summaries; a kernel that changes needs its
+# counters taken again.
+def load_measured_traffic():
+    path = os.path.join(ROOT, "profiles", "traffic.json")
+    try:
+        with open(path) as f:
+            raw = json.load(f)
+    except (OSError, ValueError):
+        return {}
+    return {(e["workload"], e["entry_point"]): (float(e["bytes_per_launch"]), e["source"]) for e in raw["kernels"]}
+
+
+MEASURED_TRAFFIC = load_measured_traffic()
 
 # what the default run reports next to its headline workload: (workload, path)
 OTHERS = [("c2", "layer"), ("c3", "layer"), ("c5", "rows"), ("c2", "rows"), ("c3", "rows")]
+# ... and through the public layer API: (workload, loss)
+API_RUNS = [("c5", "dense"), ("c5", "sum"), ("c2", "dense"), ("c2", "sum"), ("c3", "dense"), ("c3", "sum")]
 
 
 class Placement:
     """Where a workload's tensors are allocated (``mode``; ``regions`` = sinabs.exodus.hbm.HbmRegions):
-    striped      inputs (x, grad_output) in the range made of the first region of HBM, everything the kernels write
-                 in the striped range, whose 64 MiB pages alternate between the three regions
-    all-striped  every big tensor in the striped range
-    regions      every tensor in one region's range: inputs in the first, outputs in the second and -- where one
-                 range cannot hold them, and for the checkpoints -- the third
-    one-region   the control: every big tensor in the first region's range
+    striped      what a program gets that calls ``hbm.enable()`` and nothing else: its own inputs (x, grad_output) from
+                 the ordinary allocator, everything the kernels write in the striped range, whose 64 MiB pages
+                 alternate between the three regions of HBM
+    all-striped  every big tensor in the striped range (``hbm.enable(everything=True)``, or layers behind other layers)
+    regions      (needs sorted ranges) every tensor in one region's range: inputs in the first, outputs in the second
+                 and third
+    one-region   (needs sorted ranges) the control: every big tensor in the first region's range
     plain        torch's ordinary allocator"""
 
-    def __init__(self, torch, dev, regions=None, mode="plain", assign=(0, 0, 1, 1)):
+    def __init__(self, torch, dev, regions=None, mode="plain"):
         self.torch, self.dev, self.regions, self.mode = torch, dev, regions, mode
-        self.assign = assign        # mode "regions", layer workloads: region of input, grad_output, spikes, grad_input
 
     def empty(self, shape, k):
-        if self.regions is None:
+        """k = 0: a tensor the kernels read (input, incoming gradient); 1, 2: tensors they write"""
+        if self.regions is None or (self.mode == "striped" and k == 0):
             return self.torch.empty(tuple(shape), device=self.dev)
-        if self.mode == "striped":
-            return self.regions.empty(shape, region=0 if k == 0 else 3)
-        if self.mode == "all-striped":
-            return self.regions.empty(shape, region=3)
+        if self.mode in ("striped", "all-striped"):
+            return self.regions.empty(shape)
         return self.regions.empty(shape, region=0 if self.mode == "one-region" else k)
 
     def describe(self):
         if self.regions is None:
             return {"placement": "ordinary allocator"}
-        text = {"striped": "hbm regions (sinabs.exodus.hbm): inputs in one region of HBM, everything the kernels write in "
-                           "memory whose 64 MiB pages alternate between the three regions",
+        text = {"striped": "sinabs.exodus.hbm.enable(): inputs from the ordinary allocator, everything the kernels write in "
+                           "memory whose 64 MiB pages alternate between the three regions of HBM",
                 "all-striped": "every big tensor in memory whose 64 MiB pages alternate between the three regions of HBM",
                 "one-region": "all big tensors in ONE region of HBM (the control experiment)",
-                "regions": "hbm regions, one region per tensor: inputs in the first, outputs in the second, checkpoints in "
-                           "the third" if self.assign == (0, 0, 1, 1) else
-                           f"hbm regions, layer tensors (input, grad_output, spikes, grad_input) in regions {self.assign}"}
-        return {"placement": text[self.mode],
-                "placement_verified_by_timed_copies": self.regions.verified,
-                "placement_measured": {k: ([round(x) for x in v] if isinstance(v, list) else round(v))
-                                       for k, v in self.regions.report.items()}}
+                "regions": "one region of HBM per tensor: inputs in the first, outputs in the second and third"}
+        out = {"placement": text[self.mode], "placement_setup_s": round(self.regions.setup_s, 3),
+               "placement_sorted_by_timed_copies": bool(self.regions.sorted)}
+        if self.regions.sorted:
+            out["placement_verified_by_timed_copies"] = bool(self.regions.verified)
+            out["placement_measured"] = {k: ([round(x) for x in v] if isinstance(v, list) else round(v))
+                                         for k, v in self.regions.report.items()}
+        return out
 
 
 def build_layer_workload(key, torch, hip, act, dev, place=None):
@@ -114,7 +117,7 @@ def build_layer_workload(key, torch, hip, act, dev, place=None):
     B, T, M = w["batch"], w["steps"], w["neurons"]
     N = B * M
     g = torch.Generator(device=dev).manual_seed(list(WORKLOADS).index(key))
-    rx, rgo, rs, rgi = place.assign if place.mode == "regions" else (0, 0, 1, 1)
+    rx, rgo, rs, rgi = 0, 0, 1, 1                  # tensors the kernels read: 0; tensors they write: 1
     x = place.empty((B, T, M), rx)
     x.uniform_(0.0, 0.5, generator=g) if key == "c1" else x.normal_(w["mean"], w["std"], generator=g)
     go = place.empty((B, T, M), rgo).fill_(1.0)
@@ -409,9 +412,124 @@ def measure_ceilings(args, torch, hip, dev, place):
     return res
 
 
+def api_layer(key, torch, dev):
+    """The layer of ``sinabs.exodus.layers`` that a configuration names, and the shape of its input."""
+    import sinabs.exodus.layers as el
+    from sinabs.exodus._compat import activation as act
+    if key == "c5":
+        layer = el.LIF(tau_mem=20.0, tau_syn=5.0, min_v_mem=-1.0, spike_fn=act.MaxSpike(2), train_alphas=True)
+        shape = (16, 2000, 65536)
+    elif key == "c2":
+        layer = el.LIF(tau_mem=20.0, spike_fn=act.SingleSpike)
+        shape = (32, 300, 128, 32, 32)
+    elif key == "c3":
+        g = torch.Generator().manual_seed(2)
+        layer = el.ExpLeak(tau_mem=5.0 + 45.0 * torch.rand(4096, generator=g), train_alphas=True)
+        shape = (64, 1000, 4096)
+    else:
+        layer = el.IAF()
+        shape = (8, 100, 256)
+    return layer.to(dev), shape
+
+
+def measure_layer_api(key, loss, torch, dev, steps, warmup, place_all=False):
+    """One configuration through the public layer API: ``out = layer(x)`` followed by ``out.backward(grad)`` with a
+    dense gradient (``loss == "dense"``) or ``out.sum().backward()`` (``"sum"``): autograd, outputs allocated by every
+    call, the layer's state handling and firing rate included.  Wall time per step and the time of each direction
+    from events around the two calls.  ``place_all``: the input and the gradient are allocated inside
+    ``hbm.placement()`` as well (a layer behind other layers)."""
+    from sinabs.exodus import hbm
+    w = WORKLOADS[key]
+    layer, shape = api_layer(key, torch, dev)
+    g = torch.Generator(device=dev).manual_seed(list(WORKLOADS).index(key))
+    with (hbm.placement() if place_all else contextlib.nullcontext()):
+        x = torch.empty(shape, device=dev)
+        x.uniform_(0.0, 0.5, generator=g) if key == "c1" else x.normal_(w["mean"], w["std"], generator=g)
+        go = torch.empty(shape, device=dev).uniform_(0.5, 1.5, generator=g) if loss == "dense" else None
+    x.requires_grad_(True)
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps)]
+
+    def step(e=None):
+        layer.reset_states()
+        layer.zero_grad(set_to_none=True)
+        x.grad = None
+        if e:
+            e[0].record()
+        out = layer(x)
+        if e:
+            e[1].record()
+        if loss == "dense":
+            out.backward(go)
+        else:
+            out.sum().backward()
+        if e:
+            e[2].record()
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for k in range(steps):
+        step(ev[k])
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) / steps
+    fwd_ms = sum(e[0].elapsed_time(e[1]) for e in ev) / steps
+    bwd_ms = sum(e[1].elapsed_time(e[2]) for e in ev) / steps
+    n_t = 1
+    for v in shape:
+        n_t *= v
+    # bytes that have to move: forward x in, output out (8); backward with a dense gradient: gradient and x in, grad_x
+    # out (12); with the sum as the loss: torch's sum reads the output (4), the backward reads x and writes grad_x (8)
+    return {"workload": w["name"], "path": "public layer API (sinabs.exodus.layers, autograd, outputs allocated per call)",
+            "layer": repr(layer).split("(")[0].strip(), "loss": "out.backward(dense gradient)" if loss == "dense" else "out.sum().backward()",
+            "rows": n_t // shape[1], "time_steps": shape[1], "steps": steps, "ms_per_step": wall * 1e3,
+            "fwd_ms": fwd_ms, "bwd_ms": bwd_ms, "value": n_t / wall, "unit": "neuron-timesteps/s",
+            "algorithmic_bytes_per_neuron_timestep": 20,
+            "fwd_bwd_combined_frac": n_t * 20 / ((fwd_ms + bwd_ms) * 1e-3) / 1e9 / HBM_PEAK_GBS}
+
+
+def measure_small_layer(torch, dev, steps, warmup):
+    """C1 (8 x 100 x 256, IAF, loss = sum of spikes) through the layer API: one step eagerly, and the same step
+    recorded into a HIP graph and replayed (sinabs.exodus.graph.GraphedStep); the two kernels alone from events."""
+    from sinabs.exodus.graph import GraphedStep
+    import torch.nn as nn
+    w = WORKLOADS["c1"]
+    layer, shape = api_layer("c1", torch, dev)
+    model = nn.Sequential(layer)
+    g = torch.Generator(device=dev).manual_seed(3)
+    x = torch.empty(shape, device=dev).uniform_(0.0, 0.5, generator=g).requires_grad_(True)
+
+    def step():
+        layer.reset_states()
+        x.grad = None
+        out = model(x)
+        out.sum().backward()
+        return out
+
+    def wall(fn, n):
+        for _ in range(max(3, warmup)):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(n):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / n * 1e3
+
+    n = max(200, steps * 10)
+    eager_ms = wall(step, n)
+    graphed = GraphedStep(model, step)
+    replay_ms = wall(graphed.replay, n)
+    n_t = shape[0] * shape[1] * shape[2]
+    return {"workload": w["name"], "path": "public layer API (sinabs.exodus.layers)", "rows": shape[0] * shape[2],
+            "time_steps": shape[1], "steps": n, "ms_per_step_eager": eager_ms, "ms_per_step_hip_graph_replay": replay_ms,
+            "value": n_t / (replay_ms * 1e-3), "value_eager": n_t / (eager_ms * 1e-3), "unit": "neuron-timesteps/s"}
+
+
 def measure_conv_snn(args, torch, dev):
-    """Wall clock of one forward + backward of the convolutional spiking network, PyTorch-ROCm for the
-    convolution / pooling / linear layers, this package's layers in between."""
+    """Wall clock of one forward + backward of the convolutional spiking network (C4), PyTorch-ROCm for the
+    convolution / pooling / linear layers, this package's layers in between; and, from a second run with events
+    around every neuron layer's forward and backward pass, the share of the neuron layers."""
     import torch.nn as nn
     import sinabs.exodus.layers as el
     B, T = 64, 300
@@ -425,7 +543,7 @@ def measure_conv_snn(args, torch, dev):
     x = (torch.rand(B, T, 2, 34, 34, device=dev) < 0.02).float()
     labels = torch.randint(0, 10, (B,), device=dev)
 
-    def timed(model, spiking=True):
+    def make_step(model, spiking=True):
         def step():
             for m in model:
                 if hasattr(m, "reset_states"):
@@ -437,6 +555,9 @@ def measure_conv_snn(args, torch, dev):
             else:
                 loss = out.sum()
             loss.backward()
+        return step
+
+    def timed(step):
         for _ in range(max(1, args.warmup)):
             step()
         torch.cuda.synchronize()
@@ -450,14 +571,43 @@ def measure_conv_snn(args, torch, dev):
     with torch.no_grad():
         for i in (0, 3, 6):
             fast[i].weight.mul_(3.0)                # enough drive for all three layers to spike
-    res = {"workload": "C4 conv SNN fwd+bwd (B=64,T=300, 2x34x34 Bernoulli(0.02) input)",
-           "neuron_layer_rows": [64 * 32 * 32 * 32, 64 * 64 * 14 * 14, 64 * 10], "time_steps": T}
-    res["ms_layer_kernels"] = timed(fast)
+    res = {"workload": "C4 conv SNN fwd+bwd (B=64,T=300, 2x34x34 Bernoulli(0.02) input)", "path": "public layer API",
+           "neuron_layer_rows": [64 * 32 * 32 * 32, 64 * 64 * 14 * 14, 64 * 10], "time_steps": T, "steps": args.steps}
+    res["ms_per_step"] = timed(make_step(fast))
+    # the neuron layers' share: events when each layer's forward starts and ends, when the gradient of its output
+    # arrives and when the gradient of its input leaves (hooks; they add a little host work, so the end-to-end
+    # figure above comes from the run without them)
+    spans = []
+    handles = []
+    for m in fast:
+        if not hasattr(m, "reset_states"):
+            continue
+        ev = {k: torch.cuda.Event(enable_timing=True) for k in ("f0", "f1", "b0", "b1")}
+        spans.append(ev)
+        handles += [m.register_forward_pre_hook(lambda mod, a, ev=ev: ev["f0"].record()),
+                    m.register_forward_hook(lambda mod, a, o, ev=ev: ev["f1"].record()),
+                    m.register_full_backward_pre_hook(lambda mod, go, ev=ev: ev["b0"].record()),
+                    m.register_full_backward_hook(lambda mod, gi, go, ev=ev: ev["b1"].record())]
+    hooked = make_step(fast)
+    x.requires_grad_(True)                          # so that the first layer's backward hook has a gradient to wait for
+    for _ in range(2):
+        hooked()
+    total = 0.0
+    for _ in range(args.steps):
+        hooked()
+        torch.cuda.synchronize()
+        total += sum(ev["f0"].elapsed_time(ev["f1"]) + ev["b0"].elapsed_time(ev["b1"]) for ev in spans)
+    x.requires_grad_(False)
+    for h in handles:
+        h.remove()
+    res["ms_neuron_layers"] = total / args.steps
     for m in fast:
         if hasattr(m, "native_layout"):
             m.native_layout = False
-    res["ms_rows_functions_with_transposes"] = timed(fast)
-    res["ms_conv_pool_linear_alone"] = timed(network(lambda: None), spiking=False)
+    res["ms_per_step_rows_functions_with_transposes"] = timed(make_step(fast))
+    res["ms_conv_pool_linear_alone"] = timed(make_step(network(lambda: None), spiking=False))
+    res["value"] = sum(res["neuron_layer_rows"]) * T / (res["ms_per_step"] * 1e-3)
+    res["unit"] = "neuron-timesteps/s"
     return res
 
 
@@ -550,43 +700,18 @@ def measure_region_map(args, torch, dev):
         "pairs_on_the_wrong_side_of_the_threshold": sum(v >= threshold for v in inside) + sum(v < threshold for v in across)}))
 
 
-def measure_reallocations(args, torch, hip, act, dev):
-    """The chosen workload measured again and again on freshly allocated tensors."""
-    import random
-    rnd = random.Random(5)
-    junk = []
-    build = build_layer_workload if args.path == "layer" else build_workload
-    for k in range(args.reallocations):
-        torch.cuda.empty_cache()
-        wl = build(args.workload, torch, hip, act, dev)
-        m = measure(wl, args.steps, args.warmup, torch)
-        bf, bb = wl.get("bytes", WORKLOADS[args.workload]["bytes"])
-        n_t = wl["N"] * wl["T"]
-        print(json.dumps({"round": k, "other_allocations_held_GiB": round(sum(j.numel() for j in junk) / 2 ** 30, 2),
-                          "fwd_ms": m["fwd_ms"], "bwd_ms": m["bwd_ms"],
-                          "fwd_GBs": n_t * bf / m["fwd_ms"] / 1e6, "bwd_GBs": n_t * bb / m["bwd_ms"] / 1e6,
-                          "fwd_bwd_combined_frac": n_t * (bf + bb) / ((m["fwd_ms"] + m["bwd_ms"]) * 1e-3) / 1e9 / HBM_PEAK_GBS}),
-              flush=True)
-        del wl
-        torch.cuda.empty_cache()
-        # change what the driver has to give out next: hold one more block of another size, or drop one
-        if k % 2 == 0 or not junk:
-            junk.append(torch.empty(int(rnd.uniform(0.3, 9.0) * 2 ** 30), dtype=torch.uint8, device=dev))
-        elif rnd.random() < 0.5:
-            junk.pop(rnd.randrange(len(junk)))
-
-
-def without_cycle_option(argv):
-    """The command line without ``--after-hbm-cycle [N]`` (for the child process that measures)."""
-    rest, skip = [], False
-    for k, a in enumerate(argv):
-        if skip:
-            skip = False
-        elif a == "--after-hbm-cycle":
-            skip = k + 1 < len(argv) and argv[k + 1].isdigit()
-        elif not a.startswith("--after-hbm-cycle="):
-            rest.append(a)
-    return rest
+def child_json(argv, timeout=300):
+    """The last line a child run of this script printed, parsed, or {"error": ...}."""
+    import subprocess
+    try:
+        child = subprocess.run([sys.executable, os.path.abspath(__file__)] + argv, capture_output=True, text=True,
+                               timeout=timeout)
+    except subprocess.TimeoutExpired:
+        return {"error": f"no result within {timeout} s"}
+    try:
+        return json.loads(child.stdout.strip().splitlines()[-1])
+    except (IndexError, ValueError):
+        return {"error": (child.stderr or child.stdout)[-400:]}
 
 
 def main():
@@ -603,9 +728,12 @@ def main():
                          "e.g. a neuron count that does not fill 128-byte memory lines; such a run is a measurement "
                          "aid, not the benchmark (roofline.traffic is then null)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-others", dest="others", action="store_false",
-                    help="report only the chosen workload (the default run also times the other configurations "
-                         "and the (rows, time) kernels for a few steps each and lists them under \"others\")")
+    ap.add_argument("--others", default="all", choices=["all", "api", "none"],
+                    help="all (default): also time the other configurations and the (rows, time) kernels for a few steps "
+                         "each, every configuration through the public layer API, the small layer (C1) eagerly and as a "
+                         "HIP graph, and the convolutional network (C4), and list them under \"others\"; api: only the "
+                         "runs through the public layer API; none: only the chosen workload")
+    ap.add_argument("--no-others", dest="others", action="store_const", const="none")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also launch one plain elementwise kernel (torch.neg) over exactly 1 GiB before the timed region, so that a "
                          "counter run (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE) has a kernel of known traffic "
@@ -619,36 +747,25 @@ def main():
                          "layer API (Conv2d -> IAFSqueeze -> AvgPool -> Conv2d -> IAFSqueeze -> Flatten -> Linear -> "
                          "IAFSqueeze, batch 64 x 300 steps, cross-entropy on spike counts): layer-layout kernels, the "
                          "transposing (rows, time) Functions, and the convolution / pooling / linear layers alone")
-    ap.add_argument("--placement", default="striped", choices=["striped", "all-striped", "regions", "one-region", "plain"],
-                    help="striped (default): allocate through sinabs.exodus.hbm, which sorts device memory by the three "
-                         "regions of this GPU's HBM -- inputs in the first region's range, everything the kernels write in the "
-                         "striped range, whose 64 MiB pages alternate between the regions (a kernel's writes are held back by "
-                         "the region they go to; spread over all three they are not).  all-striped: every big tensor in the "
-                         "striped range -- what a program gets that allocates everything there without further thought.  "
-                         "regions: one region per tensor (inputs in the first, outputs in the others; see --assign).  "
-                         "one-region: the control -- the same sorted memory, every big tensor in the first region.  "
-                         "plain: the ordinary allocator.  The default run reports striped, all-striped and plain "
-                         "(roofline.frac_by_placement); the plain figure is measured first, in a child process, before this "
-                         "process touches the GPU")
-    ap.add_argument("--assign", default="0,0,1,1", metavar="X,GO,S,GI",
-                    help="with --placement regions and --path layer: the region (0, 1, 2) that the input, the incoming "
-                         "gradient, the spikes and the input gradient are allocated in (default 0,0,1,1: each kernel reads one "
-                         "region and writes another; the checkpoints go where the wrappers put them)")
+    ap.add_argument("--setup-only", action="store_true",
+                    help="instead of the benchmark, make the ranges of the chosen --placement, print how long that took "
+                         "and give them back")
+    ap.add_argument("--placement", default="striped",
+                    choices=["striped", "all-striped", "sorted-striped", "regions", "one-region", "plain"],
+                    help="striped (default): sinabs.exodus.hbm.enable() as a program would call it -- the workload's inputs "
+                         "come from the ordinary allocator, everything the kernels write lies in the striped range, whose "
+                         "64 MiB pages alternate between the three regions of this GPU's HBM (a kernel's writes are held back "
+                         "by the region they go to; spread over all three they are not).  all-striped: every big tensor in "
+                         "the striped range -- a layer behind other layers, or hbm.enable(everything=True).  sorted-striped: "
+                         "as striped, the ranges made with sort=True (timed copies decide which memory belongs to which "
+                         "region).  regions / one-region: sorted ranges of one region each -- one region per tensor, and the "
+                         "control with every tensor in the first region.  plain: the ordinary allocator.  The default run "
+                         "reports striped, all-striped and plain (roofline.frac_by_placement); the plain figures are "
+                         "measured first, in a child process, before this process touches the GPU")
     ap.add_argument("--region-map", type=float, nargs="?", const=4.0, default=0.0, metavar="GIB",
                     help="instead of the benchmark, fill device memory with buffers of GIB (default 4) GiB in the order "
                          "the driver hands them out, copy every buffer into every other with a flat copy kernel and print "
                          "the matrix of rates as text plus one JSON line with the region boundaries found")
-    ap.add_argument("--reallocations", type=int, default=0, metavar="N",
-                    help="instead of the benchmark, build and measure the chosen workload N times in this process, "
-                         "releasing its tensors to the driver and allocating other memory of varying size in between, "
-                         "and print one JSON line per round: the same kernels on the same shapes run at different rates "
-                         "depending on which physical memory their tensors were given (a process that has allocated "
-                         "nothing before, as the default run, gets one fixed placement)")
-    ap.add_argument("--after-hbm-cycle", type=int, nargs="?", const=2, default=0, metavar="N",
-                    help="first let N (default 2) child processes in turn allocate nearly all device memory and exit, "
-                         "then run the chosen measurement in another child process (this process starts no GPU work "
-                         "itself).  The physical memory a process is handed after such cycles serves the time-strided "
-                         "kernels 5-10 %% faster than on a box that has run nothing yet; the default run does not do this")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (rows shard across GPUs without exchange; "
@@ -659,44 +776,16 @@ def main():
         w_ = WORKLOADS[args.workload]
         WORKLOADS[args.workload] = dict(w_, batch=b_, steps=t_, neurons=m_,
                                         name=w_["name"] + f" -- at shape ({b_},{t_},{m_})")
-    if args.after_hbm_cycle:
-        import subprocess
-        cycle = ("import torch; free, _ = torch.cuda.mem_get_info(); n = int((free - 6 * 2**30) // (4 * 2**30)); "
-                 "held = [torch.empty(4 * 2**30, dtype=torch.uint8, device='cuda') for _ in range(n)]; "
-                 "torch.cuda.synchronize(); print(f'[hbm cycle] {n} x 4 GiB allocated, released on exit', flush=True)")
-        for _ in range(args.after_hbm_cycle):
-            subprocess.run([sys.executable, "-c", cycle], check=True, stdout=sys.stderr)
-        rest = without_cycle_option(sys.argv[1:])
-        env = dict(os.environ, EXODUS_BENCH_AFTER_HBM_CYCLE=str(args.after_hbm_cycle))
-        sys.exit(subprocess.run([sys.executable, os.path.abspath(__file__)] + rest, env=env).returncode)
 
-    plain_first, plain_note = None, None
-    special = (args.region_map or args.reallocations or args.ceilings or args.conv_snn or args.shape or args.copy_probe
-               or args.assign != "0,0,1,1")
-    if args.placement == "striped" and args.others and not special:
-        # the same measurement with the ordinary allocator, in a process of its own and before this one touches
-        # the GPU, so that it sees what a program that allocates without further thought is handed; then with
-        # every tensor in the striped range
-        import subprocess
-
-        def child_run(placement):
-            try:
-                child = subprocess.run([sys.executable, os.path.abspath(__file__), "--placement", placement, "--no-others",
-                                        "--no-cpu-baseline", "--workload", args.workload, "--path", args.path,
-                                        "--steps", str(args.steps), "--warmup", str(args.warmup)],
-                                       capture_output=True, text=True, timeout=240)
-            except subprocess.TimeoutExpired:
-                return {"error": "no result within 240 s"}
-            try:
-                r = json.loads(child.stdout.strip().splitlines()[-1])["roofline"]
-                return {"frac": r["frac"], "fwd_bwd_combined_frac": r["fwd_bwd_combined_frac"],
-                        "kernel_ms": r["kernel_ms"], "other_kernel_ms": r["other_kernel"]["kernel_ms"]}
-            except (IndexError, KeyError, ValueError):
-                return {"error": (child.stderr or child.stdout)[-400:]}
-
-        plain_first = child_run("plain")
-        # (the all-striped figure is measured last, after this process has given its memory back: a process that
-        # has allocated device memory in pages leaves it to the next one as a mixture of the regions)
+    plain_first = None
+    special = args.region_map or args.ceilings or args.conv_snn or args.shape or args.copy_probe or args.setup_only
+    full_run = args.placement == "striped" and args.others == "all" and not special
+    common = ["--no-cpu-baseline", "--workload", args.workload, "--path", args.path, "--steps", str(args.steps),
+              "--warmup", str(args.warmup)]
+    if full_run:
+        # the same measurements with the ordinary allocator, in a process of its own and before this one touches
+        # the GPU, so that it sees what a program that allocates without further thought is handed
+        plain_first = child_json(["--placement", "plain", "--others", "api"] + common)
 
     import torch
     assert torch.cuda.is_available(), "bench.py needs the GPU"
@@ -708,46 +797,35 @@ def main():
     if args.region_map:
         measure_region_map(args, torch, dev)
         return
-    if args.reallocations:
-        measure_reallocations(args, torch, hip, act, dev)
-        return
     place = Placement(torch, dev)
-    if args.placement != "plain" and not args.conv_snn:
+    placement_note = None
+    if args.placement != "plain":
         from sinabs.exodus import hbm
         try:
             if args.placement == "one-region":
-                # the wrappers' own choices (checkpoints) stay off: they would move tensors out of the region
-                place = Placement(torch, dev, hbm.HbmRegions(gib_per_region=40.0, gib_striped=0.0, device=dev),
+                place = Placement(torch, dev, hbm.enable(gib_per_region=40.0, gib_striped=0.0, device=dev, sort=True),
                                   mode="one-region")
             elif args.placement == "regions":
-                assign = tuple(int(v) for v in args.assign.split(","))
-                assert len(assign) == 4 and all(0 <= v <= 2 for v in assign), "--assign takes four regions out of 0, 1, 2"
-                place = Placement(torch, dev, hbm.enable(gib_per_region=32.0, gib_striped=0.0, device=dev),
-                                  mode="regions", assign=assign)
-            elif args.placement == "all-striped":
-                place = Placement(torch, dev, hbm.enable(gib_per_region=0.0, gib_striped=72.0, device=dev),
-                                  mode="all-striped")
+                place = Placement(torch, dev, hbm.enable(gib_per_region=32.0, gib_striped=0.0, device=dev, sort=True),
+                                  mode="regions")
+            elif args.placement == "sorted-striped":
+                place = Placement(torch, dev, hbm.enable(gib_striped=72.0, device=dev, sort=True), mode="striped")
             else:
-                try:
-                    place = Placement(torch, dev, hbm.enable(gib_per_region=24.0, gib_striped=48.0, device=dev),
-                                      mode="striped")
-                except RuntimeError as err:
-                    if "did not show three kinds" not in str(err):
-                        raise
-                    # memory that earlier processes left as a mixture of the regions: no region to put the inputs
-                    # in; everything goes into the striped range, made of that memory as it is
-                    plain_note = "no regions found in device memory (earlier processes left it mixed): all-striped used"
-                    print("[bench] " + plain_note, file=sys.stderr, flush=True)
-                    place = Placement(torch, dev, hbm.enable(gib_per_region=0.0, gib_striped=72.0, device=dev),
-                                      mode="all-striped")
+                place = Placement(torch, dev, hbm.enable(gib_striped=72.0, device=dev), mode=args.placement)
         except RuntimeError as err:                     # device memory in use by something else: measure without
-            plain_note = f"regions unavailable ({err}); ordinary allocator used"
-            print("[bench] " + plain_note, file=sys.stderr, flush=True)
+            placement_note = f"ranges unavailable ({err}); ordinary allocator used"
+            print("[bench] " + placement_note, file=sys.stderr, flush=True)
+    if args.setup_only:
+        out = dict(place.describe())
+        if place.regions is not None:
+            out["gave_memory_back"] = hbm.disable()
+        print(json.dumps(out))
+        return
     if args.ceilings:
         print(json.dumps(measure_ceilings(args, torch, hip, dev, place)))
         return
     if args.conv_snn:
-        print(json.dumps(measure_conv_snn(args, torch, dev)))
+        print(json.dumps(dict(measure_conv_snn(args, torch, dev), **place.describe())))
         return
     build = build_layer_workload if args.path == "layer" else build_workload
     wl = build(args.workload, torch, hip, act, dev, place)
@@ -786,23 +864,28 @@ def main():
         "dtype": "f32",
         "data": "synthetic",
         "config": {"workload": WORKLOADS[args.workload]["name"], "path": args.path, "rows": N, "time_steps": T,
-                   "algorithmic_bytes_per_neuron_timestep": bf + bb,
-                   **place.describe(),
-                   **({"after_hbm_cycles": int(os.environ["EXODUS_BENCH_AFTER_HBM_CYCLE"])}
-                      if os.environ.get("EXODUS_BENCH_AFTER_HBM_CYCLE") else {})},
+                   "algorithmic_bytes_per_neuron_timestep": bf + bb, **place.describe()},
         "roofline": roof,
     }
+    if placement_note:
+        result["config"]["placement_note"] = placement_note
     if plain_first is not None:
+        # the ordinary allocator's figures beside the headline: what the same kernels reach without hbm.enable()
+        pr = plain_first.get("roofline", {})
+        result["value_ordinary_allocator"] = plain_first.get("value")
+        roof["frac_ordinary_allocator"] = pr.get("frac")
         roof["frac_by_placement"] = {
-            ("striped: inputs in one region, outputs striped over the three (this run's figures)" if place.mode == "striped"
-             else f"{place.mode} (this run's figures; {plain_note})"):
+            "hbm.enable(): outputs striped over the three regions of HBM (this run's figures; the >= 70 % claim rests on it)":
                 {"frac": roof["frac"], "fwd_bwd_combined_frac": roof["fwd_bwd_combined_frac"]},
-            "ordinary allocator, first allocations of a process (measured before this one touched the GPU)": plain_first}
-    if args.others and not args.shape:
+            "ordinary allocator, first allocations of a process (measured before this one touched the GPU)":
+                ({"frac": pr.get("frac"), "fwd_bwd_combined_frac": pr.get("fwd_bwd_combined_frac"),
+                  "kernel_ms": pr.get("kernel_ms"), "other_kernel_ms": pr.get("other_kernel", {}).get("kernel_ms")}
+                 if pr else plain_first)}
+    del wl, fwd, bwd
+    result["others"] = []
+    if args.others == "all" and not args.shape:
         # the other configurations and the (rows, time) kernels behind the autograd Functions, a few
         # steps each: same measurement and placement, reported beside the headline workload
-        del wl, fwd, bwd
-        result["others"] = []
         for key, path in OTHERS:
             if (key, path) == (args.workload, args.path):
                 continue
@@ -816,21 +899,46 @@ def main():
                 "algorithmic_bytes_per_neuron_timestep": obf + obb,
                 "roofline": roofline(key, other, mo["fwd_ms"], mo["bwd_ms"], obf, obb)})
             del other
-    if plain_note:
-        result["config"]["placement_note"] = plain_note
+    if args.others in ("all", "api") and not args.shape:
+        # every configuration through the public layer API, with the ordinary allocator's figures (from the child
+        # run) beside those of this process's placement
+        plain_api = {(e.get("workload"), e.get("loss")): e for e in (plain_first or {}).get("others", [])
+                     if str(e.get("path", "")).startswith("public layer API") and "loss" in e}
+        steps_api, warm_api = max(3, args.steps // 2), max(2, args.warmup // 2)
+        for key, loss in API_RUNS:
+            e = measure_layer_api(key, loss, torch, dev, steps_api, warm_api, place_all=place.mode == "all-striped")
+            e.update(place.describe())
+            e.pop("placement_measured", None)
+            twin = plain_api.get((e["workload"], e["loss"]))
+            if twin:
+                e["ordinary_allocator"] = {k: twin[k] for k in ("ms_per_step", "fwd_ms", "bwd_ms", "value",
+                                                                 "fwd_bwd_combined_frac")}
+            result["others"].append(e)
+    if args.others == "all" and not args.shape:
+        small = measure_small_layer(torch, dev, args.steps, args.warmup)
+        result["others"].append(small)
+        conv = measure_conv_snn(argparse.Namespace(steps=max(3, args.steps // 4), warmup=2), torch, dev)
+        result["others"].append(conv)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(args.workload, torch)
-    if plain_first is not None:
-        # every tensor in the striped range, in a process of its own, once this one has given its memory back
-        wl = fwd = bwd = place = None
-        if args.placement != "plain":
-            hbm.disable()
+    if full_run:
+        # every tensor in the striped range, and the set-up time of ranges sorted by timed copies, each in a process
+        # of its own once this one has given its memory back
+        place = None
         import gc
         gc.collect()
+        if not hbm.disable():
+            print("[bench] the ranges could not be given back (tensors alive)", file=sys.stderr, flush=True)
         torch.cuda.empty_cache()
         torch.cuda.synchronize()
-        roof["frac_by_placement"]["all-striped: every tensor striped over the three regions "
-                                  "(measured last, in a process of its own)"] = child_run("all-striped")
+        allst = child_json(["--placement", "all-striped", "--others", "none"] + common)
+        ar = allst.get("roofline")
+        roof["frac_by_placement"]["every tensor striped over the three regions (measured last, in a process of its own)"] = (
+            {"frac": ar["frac"], "fwd_bwd_combined_frac": ar["fwd_bwd_combined_frac"], "kernel_ms": ar["kernel_ms"],
+             "other_kernel_ms": ar["other_kernel"]["kernel_ms"]} if ar else allst)
+        result["placement_setup"] = {
+            "hbm.enable() (default: sort=False)": {"setup_s": result["config"].get("placement_setup_s")},
+            "hbm.enable(sort=True)": child_json(["--placement", "sorted-striped", "--setup-only"])}
     print(json.dumps(result))
 
 

@@ -22,6 +22,7 @@
 #ifndef EXODUS_HIP_H
 #define EXODUS_HIP_H
 
+#include <stddef.h>
 #include <stdint.h>
 
 #ifdef __cplusplus
@@ -29,7 +30,7 @@ extern "C" {
 #endif
 
 /* ABI version of this header; bumped on any signature change. */
-#define EXODUS_HIP_ABI_VERSION 7
+#define EXODUS_HIP_ABI_VERSION 8
 
 int exodus_hip_abi_version(void);
 const char *exodus_hip_error_string(int status);
@@ -37,6 +38,7 @@ const char *exodus_hip_error_string(int status);
 /* Status values of this library's own (negative, so that they cannot collide with a hipError_t). */
 #define EXODUS_ERROR_SCRATCH_TOO_SMALL (-2)
 #define EXODUS_ERROR_REGIONS_NOT_FOUND (-3)
+#define EXODUS_ERROR_RANGE_IN_USE (-4)
 
 /* ---------------------------------------------------------------------------------------------
  * One-to-one counterparts of the reference bindings
@@ -204,7 +206,12 @@ int exodus_layer_lif_forward(float *out_spikes, float *out_vmem_rec, float *out_
  * arbitrary Python callable there, sinabs/exodus/spike.py:251); otherwise `surr` is ignored.
  * grad_v_rec / grad_i_rec (batch,t,neurons, optional; with synapse both or none) are gradients
  * arriving at the forward's per-step records of the post-reset potential and the synaptic current
- * (the layer's `recordings` are differentiable, reference sinabs/exodus/layers/lif.py:256,290-293). */
+ * (the layer's `recordings` are differentiable, reference sinabs/exodus/layers/lif.py:256,290-293).
+ * grad_spikes_uniform != 0: `grad_spikes` points at ONE float that is the gradient of every spike -- what the loss
+ * `out.sum()` of the reference's own tests (reference tests/test_spike_functions.py:50, tests/test_leak_functions.py:22) hands back, which
+ * autograd represents as a broadcast scalar.  The kernel then streams one tensor less (8 instead of 12 bytes per
+ * neuron-timestep).  Only with an in-kernel surrogate (kind 1..3) and without grad_v_rec / grad_i_rec
+ * (hipErrorInvalidValue otherwise). */
 int exodus_layer_lif_backward(float *grad_input, float *alpha_mem_grad, float *alpha_syn_grad,
                               float *vmem_init_grad, float *isyn_init_grad, const float *grad_spikes,
                               const float *grad_v_last, const float *grad_i_last, const float *input,
@@ -213,8 +220,8 @@ int exodus_layer_lif_backward(float *grad_input, float *alpha_mem_grad, float *a
                               const float *membr_subtract, const float *theta, const float *theta_low,
                               int apply_theta_low, int max_num_spikes, int decay_early, int norm_input,
                               int surrogate_kind, float surr_p0, float surr_p1, const float *surr,
-                              const float *grad_v_rec, const float *grad_i_rec, int64_t batch, int64_t t,
-                              int64_t neurons, void *stream);
+                              const float *grad_v_rec, const float *grad_i_rec, int grad_spikes_uniform,
+                              int64_t batch, int64_t t, int64_t neurons, void *stream);
 
 /* exodus_layer_lif_backward for callers that cannot allocate device memory -- code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the
@@ -239,8 +246,8 @@ int exodus_layer_lif_backward_from_input(float *grad_input, float *alpha_mem_gra
                                          const float *theta, const float *theta_low, int apply_theta_low,
                                          int max_num_spikes, int decay_early, int norm_input, int surrogate_kind,
                                          float surr_p0, float surr_p1, const float *surr, const float *grad_v_rec,
-                                         const float *grad_i_rec, int64_t batch, int64_t t, int64_t neurons,
-                                         void *stream);
+                                         const float *grad_i_rec, int grad_spikes_uniform, int64_t batch, int64_t t,
+                                         int64_t neurons, void *stream);
 
 /* Forward of the non-spiking leaky-integrator layer (ExpLeak) on (batch,t,neurons): per neuron
  *   xin = norm_input ? (1 - alpha) * input : input;  xin = decay_early ? xin * alpha : xin;
@@ -254,11 +261,13 @@ int exodus_layer_leaky_forward(float *out, float *v_last, double *out_sum, const
 
 /* Backward of the above: grad_input (batch,t,neurons); optional per-neuron alpha_grad (needs `out`
  * and `vmem_initial`, and `input` when one of the input scalings is on) and vmem_init_grad;
- * grad_v_last (batch*neurons, optional) is a gradient arriving at the final state. */
+ * grad_v_last (batch*neurons, optional) is a gradient arriving at the final state.
+ * grad_out_uniform != 0: `grad_out` points at ONE float that stands for every element (as grad_spikes_uniform of
+ * exodus_layer_lif_backward). */
 int exodus_layer_leaky_backward(float *grad_input, float *alpha_grad, float *vmem_init_grad,
                                 const float *grad_out, const float *grad_v_last, const float *out,
                                 const float *input, const float *vmem_initial, const float *alpha,
-                                int decay_early, int norm_input, int64_t batch, int64_t t,
+                                int decay_early, int norm_input, int grad_out_uniform, int64_t batch, int64_t t,
                                 int64_t neurons, void *stream);
 
 /* ---- experimental spike generation on a precomputed membrane potential -------------------------
@@ -308,7 +317,12 @@ int exodus_spike_backward(float *input_grad, const float *surr, const float *out
  * (kinds_found = 0; bytes_per_region must be 0): cheaper, and enough on a machine whose memory is known to come back
  * mixed.  hipErrorOutOfMemory when too little memory is free to find or fill the ranges,
  * hipErrorInvalidValue for bad arguments or a device that already has its ranges.  Takes a second or two;
- * synchronises the device. */
+ * synchronises the device.
+ * While it works the call holds nearly all free memory of the device (all but 6 GiB, then all but 512 MiB): another
+ * process that allocates on the same GPU in that second can run out of memory.  take_limit_bytes > 0 bounds what is
+ * held (rounded down to whole chunks; hipErrorOutOfMemory when that is less than the ranges plus the 15 probe chunks
+ * need): memory beyond the bound is neither sorted nor kept from supplying pages, so on a machine that hands memory
+ * out in address order a bound below two thirds of the device leaves the ranges in one or two regions. */
 #define EXODUS_HBM_REGIONS 3
 #define EXODUS_HBM_ARENAS 4                          /* one range per region, and the striped one */
 #define EXODUS_HBM_PAGE_BYTES (64ull << 20)          /* stripe width; 32-128 MiB measured alike, 8 and 512 MiB worse */
@@ -329,10 +343,33 @@ typedef struct exodus_hbm_report {
     int32_t probe_chunk[EXODUS_HBM_PROBES];          /* the probe chunks (position in the order of creation), */
     int32_t probe_kind[EXODUS_HBM_PROBES];           /* the group each was put in, and the copy rate between every */
     float probe_pair_GBs[EXODUS_HBM_PROBES][EXODUS_HBM_PROBES];   /* two of them (mean of both directions) */
+    float phase_s[4];                                /* seconds spent taking the memory, sorting it, building the ranges, checking them */
 } exodus_hbm_report;
 int exodus_hbm_regions_create(int device, uint64_t bytes_per_region, uint64_t bytes_striped, uint64_t chunk_bytes,
-                              int sort, exodus_hbm_report *report);
+                              int sort, uint64_t take_limit_bytes, exodus_hbm_report *report);
+/* Gives the ranges' memory back to the driver.  EXODUS_ERROR_RANGE_IN_USE, and nothing happens, while any piece
+ * handed out by exodus_hbm_alloc_* has not come back through exodus_hbm_free. */
 int exodus_hbm_regions_destroy(int device);
+
+/* Pieces of the ranges, in the signature PyTorch's pluggable allocator binds
+ * (torch.cuda.memory.CUDAPluggableAllocator(path, "exodus_hbm_alloc_striped", "exodus_hbm_free")), so that a
+ * torch.cuda.MemPool can sit on top of a range: PyTorch's caching allocator then asks these functions for whole
+ * segments, splits and reuses them itself and keeps track of which stream still uses what, as it does for ordinary
+ * memory -- the tensors of such a pool are as safe across streams as any other tensor.  exodus_hbm_alloc_striped
+ * takes from the striped range, _region0/1/2 from the range of one region: first fit from the lowest address, sizes
+ * rounded up to 2 MiB, neighbours joined on release.  When the device has no such range (never created, destroyed,
+ * size 0) or the range has no room, the memory comes from hipMalloc instead and exodus_hbm_free returns it with
+ * hipFree: the caller always gets memory, only the placement is lost.  NULL only when hipMalloc fails too.  `stream`
+ * is ignored (nothing here is ordered by streams: a caller without an allocator like PyTorch's on top must free a
+ * piece only after all work that uses it has finished).  exodus_hbm_free ignores pointers it did not hand out.
+ * Thread safe.  exodus_hbm_usage reports the bytes handed out from each range (bytes_in_use[4]) and, optionally,
+ * what was taken from hipMalloc instead. */
+void *exodus_hbm_alloc_striped(size_t size, int device, void *stream);
+void *exodus_hbm_alloc_region0(size_t size, int device, void *stream);
+void *exodus_hbm_alloc_region1(size_t size, int device, void *stream);
+void *exodus_hbm_alloc_region2(size_t size, int device, void *stream);
+void exodus_hbm_free(void *ptr, size_t size, int device, void *stream);
+int exodus_hbm_usage(int device, uint64_t *bytes_in_use, uint64_t *bytes_elsewhere);
 
 #ifdef __cplusplus
 }

@@ -22,16 +22,23 @@
 // sorted chunk: with all other free memory held, the chunk is released and 64 pages are allocated at
 // once, which can only come from the hole it left.
 //
-//   exodus_hbm_regions_create(device, bytes_per_region, bytes_striped, chunk_bytes, sort, &report)
+//   exodus_hbm_regions_create(device, bytes_per_region, bytes_striped, chunk_bytes, sort, take_limit_bytes, &report)
 //   exodus_hbm_regions_destroy(device)
+//   exodus_hbm_alloc_striped / _region0 / _region1 / _region2 (size, device, stream), exodus_hbm_free(ptr, size, device, stream)
 //
-// Both calls synchronise the device.  One set of arenas per device; creating a second one fails with
-// hipErrorInvalidValue until the first is destroyed.
+// create and destroy synchronise the device.  One set of arenas per device; creating a second one fails with
+// hipErrorInvalidValue until the first is destroyed.  The alloc / free pair hands out pieces of the arenas (first
+// fit, pieces of 2 MiB, neighbours joined on release) in the signature of PyTorch's pluggable allocator, so that a
+// torch.cuda.MemPool can sit on top: PyTorch's caching allocator then keeps track of which stream still uses
+// what, and these functions only ever see whole segments come and go.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
 #include <algorithm>
+#include <chrono>
+#include <map>
 #include <mutex>
+#include <unordered_map>
 #include <vector>
 
 #include "exodus_common.hpp"
@@ -62,12 +69,71 @@ __global__ void __launch_bounds__(256) region_copy(f32x4 *__restrict__ dst, cons
         if (base + k * 256 < n_chunks) st_stream(v[k], dst + base + k * 256);
 }
 
+constexpr size_t GRANULE = size_t(2) << 20;   // pieces handed out by exodus_hbm_alloc_* are multiples of this
+
 struct Arenas {
     bool live = false;
     void *base[ARENAS] = {nullptr, nullptr, nullptr, nullptr};
     size_t reserved[ARENAS] = {0, 0, 0, 0};
     size_t unit[ARENAS] = {0, 0, 0, 0};     // bytes per allocation: a chunk in the regions' arenas, a page in the striped one
     std::vector<hipMemGenericAllocationHandle_t> handles[ARENAS];   // allocation j is mapped at base + j * unit
+    // what exodus_hbm_alloc_* has not handed out: offset -> bytes, neighbours joined; and what it has
+    std::map<size_t, size_t> free_pieces[ARENAS];
+    size_t in_use[ARENAS] = {0, 0, 0, 0};
+    size_t pieces_out[ARENAS] = {0, 0, 0, 0};
+
+    bool anything_out() const
+    {
+        for (int k = 0; k < ARENAS; ++k)
+            if (pieces_out[k]) return true;
+        return false;
+    }
+
+    // first fit from the lowest address; nullptr when no piece of the range is large enough
+    void *take(int k, size_t bytes)
+    {
+        const size_t want = (bytes + GRANULE - 1) / GRANULE * GRANULE;
+        for (auto it = free_pieces[k].begin(); it != free_pieces[k].end(); ++it) {
+            if (it->second < want) continue;
+            const size_t off = it->first, rest = it->second - want;
+            free_pieces[k].erase(it);
+            if (rest) free_pieces[k].emplace(off + want, rest);
+            in_use[k] += want;
+            ++pieces_out[k];
+            return static_cast<char *>(base[k]) + off;
+        }
+        return nullptr;
+    }
+
+    // index of the range that holds p, or -1
+    int range_of(const void *p) const
+    {
+        for (int k = 0; k < ARENAS; ++k)
+            if (base[k] && p >= base[k] && p < static_cast<const char *>(base[k]) + reserved[k]) return k;
+        return -1;
+    }
+
+    void give_back(int k, void *p, size_t bytes)
+    {
+        const size_t want = (bytes + GRANULE - 1) / GRANULE * GRANULE;
+        size_t off = static_cast<size_t>(static_cast<char *>(p) - static_cast<char *>(base[k])), n = want;
+        auto next = free_pieces[k].lower_bound(off);
+        if (next != free_pieces[k].end() && off + n == next->first) {
+            n += next->second;
+            next = free_pieces[k].erase(next);
+        }
+        if (next != free_pieces[k].begin()) {
+            auto prev = std::prev(next);
+            if (prev->first + prev->second == off) {
+                off = prev->first;
+                n += prev->second;
+                free_pieces[k].erase(prev);
+            }
+        }
+        free_pieces[k].emplace(off, n);
+        in_use[k] -= want;
+        --pieces_out[k];
+    }
 
     // unmaps and releases everything; returns the first error
     hipError_t release()
@@ -100,6 +166,9 @@ struct Loose {
 
 std::mutex table_mutex;
 Arenas table[MAX_DEVICES];
+// what exodus_hbm_alloc_* took from the ordinary allocator because a range was absent or full: pointer -> bytes
+std::unordered_map<void *, size_t> elsewhere;
+size_t elsewhere_bytes[MAX_DEVICES] = {};
 
 // everything create() holds while it sorts; the destructor gives back whatever was not moved into an arena
 struct Sorting {
@@ -173,7 +242,7 @@ float two_group_threshold(const std::vector<float> &v)
 }
 
 int create(int device, uint64_t bytes_per_region, uint64_t bytes_striped, uint64_t chunk_bytes, bool sort,
-           exodus_hbm_report *rep)
+           uint64_t take_limit, exodus_hbm_report *rep)
 {
     HBM_TRY(hipSetDevice(device));
     HBM_TRY(hipDeviceSynchronize());
@@ -195,7 +264,14 @@ int create(int device, uint64_t bytes_per_region, uint64_t bytes_striped, uint64
     const size_t margin = size_t(6) << 30;                              // left to everybody else while sorting
     if (free_b < margin + (3 * need + PROBES) * chunk) return hipErrorOutOfMemory;
     size_t n = (free_b - margin) / chunk;
+    // a caller's bound on what may be held while the ranges are made (0 = none): the part of the memory that is
+    // never taken cannot be sorted, nor kept from supplying pages, so a bound trades placement for politeness
+    if (take_limit) n = std::min<size_t>(n, take_limit / chunk);
 
+    const auto clock0 = std::chrono::steady_clock::now();
+    auto since = [](std::chrono::steady_clock::time_point t) {
+        return std::chrono::duration<float>(std::chrono::steady_clock::now() - t).count();
+    };
     Sorting s;
     s.chunk = chunk;
     HBM_TRY(hipEventCreate(&s.e0));
@@ -215,10 +291,12 @@ int create(int device, uint64_t bytes_per_region, uint64_t bytes_striped, uint64
         if (e == hipErrorOutOfMemory) { (void)hipGetLastError(); break; }   // somebody else took memory meanwhile
         HBM_TRY(e);
         s.handle.push_back(h); s.owned.push_back(1); s.mapped.push_back(0);
+        if (!sort) continue;                       // only the timed copies need to reach the chunk's memory
         HBM_TRY(hipMemMap(s.at(i), chunk, 0, h, 0));
         s.mapped[i] = 1;
         HBM_TRY(hipMemSetAccess(s.at(i), chunk, &acc, 1));
     }
+    rep->phase_s[0] = since(clock0);
     n = s.handle.size();
     if (n < 3 * need + PROBES) return hipErrorOutOfMemory;
 
@@ -358,6 +436,8 @@ int create(int device, uint64_t bytes_per_region, uint64_t bytes_striped, uint64
     // machine finds region 0 where its ordinary allocations lie.
     Arenas built;
     HBM_TRY(hipDeviceSynchronize());
+    rep->phase_s[1] = since(clock0) - rep->phase_s[0];
+    const auto clock2 = std::chrono::steady_clock::now();
     int status = hipSuccess;
     std::vector<size_t> to_pages[REGIONS];                              // chunks that become pages, by kind
     for (int k = 0; k < REGIONS && status == hipSuccess && sorted; ++k) {
@@ -389,7 +469,9 @@ int create(int device, uint64_t bytes_per_region, uint64_t bytes_striped, uint64
         size_t free_now = 0, total_now = 0;
         status = hipMemGetInfo(&free_now, &total_now);
         const size_t spare = size_t(512) << 20;
-        while (status == hipSuccess && free_now > spare + PAGE) {
+        // (with a bound on what may be taken nothing more is held: the pages then come from wherever the driver
+        // finds room, which on a machine that hands memory out in address order is the hole all the same)
+        while (status == hipSuccess && !take_limit && free_now > spare + PAGE) {
             hipMemGenericAllocationHandle_t h;
             const hipError_t e = hipMemCreate(&h, PAGE, &prop, 0);
             if (e == hipErrorOutOfMemory) { (void)hipGetLastError(); break; }
@@ -398,15 +480,19 @@ int create(int device, uint64_t bytes_per_region, uint64_t bytes_striped, uint64
             free_now -= PAGE;
         }
         // the chunks whose pages take turns in the range: one of each kind after the other -- or, with no kinds,
-        // chunks spread evenly over the order of creation
+        // chunks spread evenly over the order of creation, taken from its first, second and last third in turn
+        // (on a machine that hands memory out in address order the thirds are the regions; on one that does not,
+        // any order is as good)
         const size_t lanes = REGIONS * need_striped;
         std::vector<size_t> turn;
-        for (size_t c = 0; c < lanes; ++c)
-            turn.push_back(sorted ? to_pages[c % REGIONS][c / REGIONS] : (n * (2 * c + 1)) / (2 * lanes));
+        for (size_t c = 0; c < lanes; ++c) {
+            const size_t spread = (c % REGIONS) * need_striped + c / REGIONS;    // position among `lanes` even steps
+            turn.push_back(sorted ? to_pages[c % REGIONS][c / REGIONS] : (n * (2 * spread + 1)) / (2 * lanes));
+        }
         std::vector<Loose> pages(lanes);
         for (size_t c = 0; c < lanes && status == hipSuccess; ++c) {
             const size_t i = turn[c];
-            if ((status = hipMemUnmap(s.at(i), chunk)) != hipSuccess) break;
+            if (s.mapped[i] && (status = hipMemUnmap(s.at(i), chunk)) != hipSuccess) break;
             s.mapped[i] = 0;
             if ((status = hipMemRelease(s.handle[i])) != hipSuccess) break;
             s.owned[i] = 0;
@@ -437,6 +523,8 @@ int create(int device, uint64_t bytes_per_region, uint64_t bytes_striped, uint64
     }                                                                   // what was held goes back here
     if (status != hipSuccess) { (void)built.release(); return status; }
 
+    rep->phase_s[2] = since(clock2);
+    const auto clock3 = std::chrono::steady_clock::now();
     // 4. the proof: copies inside each arena (first half to second half) and between the regions' arenas
     const size_t half = (need_pure / 2) * chunk;             // 0 when a range is one chunk or absent
     for (int k = 0; k < ARENAS; ++k) {
@@ -461,6 +549,9 @@ int create(int device, uint64_t bytes_per_region, uint64_t bytes_striped, uint64
         if (h) status = s.rate(static_cast<char *>(built.base[STRIPED]) + h, built.base[STRIPED], h, 3, &rep->copy_striped_GBs);
     }
     if (status != hipSuccess) { (void)hipDeviceSynchronize(); (void)built.release(); return status; }
+    rep->phase_s[3] = since(clock3);
+    for (int k = 0; k < ARENAS; ++k)
+        if (built.reserved[k]) built.free_pieces[k].emplace(size_t(0), built.reserved[k]);
     built.live = true;
     table[device] = std::move(built);
     return hipSuccess;          // ~Sorting returns the unused chunks
@@ -471,7 +562,8 @@ int create(int device, uint64_t bytes_per_region, uint64_t bytes_striped, uint64
 extern "C" {
 
 EXODUS_API int exodus_hbm_regions_create(int device, uint64_t bytes_per_region, uint64_t bytes_striped,
-                                         uint64_t chunk_bytes, int sort, exodus_hbm_report *report)
+                                         uint64_t chunk_bytes, int sort, uint64_t take_limit_bytes,
+                                         exodus_hbm_report *report)
 {
     if (device < 0 || device >= MAX_DEVICES || !report || (bytes_per_region == 0 && bytes_striped == 0) || chunk_bytes == 0)
         return hipErrorInvalidValue;
@@ -481,7 +573,7 @@ EXODUS_API int exodus_hbm_regions_create(int device, uint64_t bytes_per_region, 
     int before = 0;
     if (hipGetDevice(&before) != hipSuccess) return hipErrorInvalidDevice;
     *report = exodus_hbm_report{};
-    const int status = create(device, bytes_per_region, bytes_striped, chunk_bytes, sort != 0, report);
+    const int status = create(device, bytes_per_region, bytes_striped, chunk_bytes, sort != 0, take_limit_bytes, report);
     (void)hipSetDevice(before);
     return status;
 }
@@ -492,6 +584,7 @@ EXODUS_API int exodus_hbm_regions_destroy(int device)
     std::lock_guard<std::mutex> guard(table_mutex);
     Arenas &a = table[device];
     if (!a.live) return hipSuccess;
+    if (a.anything_out()) return EXODUS_ERROR_RANGE_IN_USE;     // memory that somebody still holds is never unmapped
     int before = 0;
     if (hipGetDevice(&before) != hipSuccess) return hipErrorInvalidDevice;
     int status = hipSetDevice(device);
@@ -500,6 +593,68 @@ EXODUS_API int exodus_hbm_regions_destroy(int device)
     if (status == hipSuccess) status = released;
     (void)hipSetDevice(before);
     return status;
+}
+
+// A piece of range `k` of `device`, or -- when the device has no such range, or the range no room -- plain device
+// memory (remembered, so that exodus_hbm_free knows what to do with it): a caller of these functions is an
+// allocator that cannot do anything useful with a null pointer.
+static void *alloc_from(int k, size_t size, int device)
+{
+    if (device < 0 || device >= MAX_DEVICES) return nullptr;
+    if (size == 0) size = 1;
+    std::lock_guard<std::mutex> guard(table_mutex);
+    Arenas &a = table[device];
+    if (a.live && a.base[k]) {
+        if (void *p = a.take(k, size)) return p;
+    }
+    int before = 0;
+    if (hipGetDevice(&before) != hipSuccess) return nullptr;
+    void *p = nullptr;
+    if (hipSetDevice(device) == hipSuccess && hipMalloc(&p, size) != hipSuccess) {
+        (void)hipGetLastError();
+        p = nullptr;
+    }
+    (void)hipSetDevice(before);
+    if (p) {
+        elsewhere[p] = size;
+        elsewhere_bytes[device] += size;
+    }
+    return p;
+}
+
+EXODUS_API void *exodus_hbm_alloc_striped(size_t size, int device, void *) { return alloc_from(STRIPED, size, device); }
+EXODUS_API void *exodus_hbm_alloc_region0(size_t size, int device, void *) { return alloc_from(0, size, device); }
+EXODUS_API void *exodus_hbm_alloc_region1(size_t size, int device, void *) { return alloc_from(1, size, device); }
+EXODUS_API void *exodus_hbm_alloc_region2(size_t size, int device, void *) { return alloc_from(2, size, device); }
+
+EXODUS_API void exodus_hbm_free(void *ptr, size_t size, int device, void *)
+{
+    if (!ptr || device < 0 || device >= MAX_DEVICES) return;
+    if (size == 0) size = 1;
+    std::lock_guard<std::mutex> guard(table_mutex);
+    Arenas &a = table[device];
+    const int k = a.live ? a.range_of(ptr) : -1;
+    if (k >= 0) {
+        a.give_back(k, ptr, size);
+        return;
+    }
+    auto it = elsewhere.find(ptr);
+    if (it == elsewhere.end()) return;                          // not from here: nothing this library may free
+    elsewhere_bytes[device] -= it->second;
+    elsewhere.erase(it);
+    int before = 0;
+    if (hipGetDevice(&before) != hipSuccess) return;
+    if (hipSetDevice(device) == hipSuccess) (void)hipFree(ptr);
+    (void)hipSetDevice(before);
+}
+
+EXODUS_API int exodus_hbm_usage(int device, uint64_t *bytes_in_use, uint64_t *bytes_elsewhere)
+{
+    if (device < 0 || device >= MAX_DEVICES || !bytes_in_use) return hipErrorInvalidValue;
+    std::lock_guard<std::mutex> guard(table_mutex);
+    for (int k = 0; k < ARENAS; ++k) bytes_in_use[k] = table[device].live ? table[device].in_use[k] : 0;
+    if (bytes_elsewhere) *bytes_elsewhere = elsewhere_bytes[device];
+    return hipSuccess;
 }
 
 }  // extern "C"

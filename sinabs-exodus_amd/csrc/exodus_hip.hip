@@ -1073,6 +1073,9 @@ EXODUS_API const char *exodus_hip_error_string(int status)
         return "timed copies between chunks of device memory did not show three kinds of chunks with a clear gap "
                "between them: this device's memory has no regions to sort tensors by, or something else was "
                "using it during the measurement";
+    if (status == EXODUS_ERROR_RANGE_IN_USE)
+        return "memory handed out by exodus_hbm_alloc_* has not come back through exodus_hbm_free yet: the ranges "
+               "stay as they are";
     return hipGetErrorString(static_cast<hipError_t>(status));
 }
 

@@ -17,6 +17,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
 #include <initializer_list>
 #include <mutex>
 #include <type_traits>
@@ -425,7 +426,10 @@ __global__ void __launch_bounds__(BLOCK) layer_lif_forward(
 // evaluate it from the rebuilt potential and ignore `surr`.
 // EXTRA: gradients also arrive at the per-step state records of the forward (grad_v_rec on the potential
 // after each reset, with synapse grad_i_rec on each synaptic current): two more streamed inputs.
-template <bool SYN, int KIND, int CAPK, bool NT, bool EXTRA>
+// GO1: the gradient of the spikes is one value for every neuron and step (the gradient of a sum of the
+// output, which autograd hands over as a broadcast scalar): `grad_spikes` then points at that one float and the
+// kernel streams one tensor less (8 instead of 12 bytes per neuron-timestep).
+template <bool SYN, int KIND, int CAPK, bool NT, bool EXTRA, bool GO1 = false>
 __global__ void __launch_bounds__(BWD_BLOCK)
     __attribute__((amdgpu_waves_per_eu((KIND == EXODUS_SURR_TENSOR || EXTRA) ? 2 : EXODUS_LAYER_BWD_WAVES,
                                        (KIND == EXODUS_SURR_TENSOR || EXTRA) ? 2 : EXODUS_LAYER_BWD_WAVES)))
@@ -448,7 +452,8 @@ layer_lif_backward(
     const int64_t n_ck = (T + CKPT - 1) / CKPT;
     // block-uniform bases; lane and step offsets are added by the buffer instructions
     const float *xp = x + (b * T) * M + m0;
-    const float *gp = grad_spikes + (b * T) * M + m0;
+    const float *gp = GO1 ? nullptr : grad_spikes + (b * T) * M + m0;
+    const float g1 = GO1 ? grad_spikes[0] : 0.f;
     float *op = grad_x + (b * T) * M + m0;
     constexpr bool FROM_TENSOR = KIND == EXODUS_SURR_TENSOR;
     const float *srp = FROM_TENSOR ? surr + (b * T) * M + m0 : nullptr;
@@ -495,7 +500,7 @@ layer_lif_backward(
         {
             // always CKPT loads per tensor (steps past the end re-read the last step): a constant number
             // of loads in flight lets each use wait for its own load only
-            const Rsrc rx = make_rsrc(xp + t0 * M), rg = make_rsrc(gp + t0 * M);
+            const Rsrc rx = make_rsrc(xp + t0 * M), rg = make_rsrc(GO1 ? nullptr : gp + t0 * M);
             const Rsrc rs = make_rsrc(FROM_TENSOR ? srp + t0 * M : nullptr);
             const Rsrc rqv = make_rsrc(EXTRA ? qvp + t0 * M : nullptr);
             const Rsrc rqi = make_rsrc((EXTRA && SYN) ? qip + t0 * M : nullptr);
@@ -504,7 +509,7 @@ layer_lif_backward(
             for (int k = 0; k < CKPT; ++k) {
                 const unsigned so = (GUARD ? (k < last ? k : last) : k) * step_bytes;
                 xr[k] = IO::load(rx, voff, so);
-                gr[k] = IO::load(rg, voff, so);
+                if (!GO1) gr[k] = IO::load(rg, voff, so);
                 if (FROM_TENSOR) sr[k] = IO::load(rs, voff, so);
                 if (EXTRA) qv[k] = IO::load(rqv, voff, so);
                 if (EXTRA && SYN) qi[k] = IO::load(rqi, voff, so);
@@ -536,7 +541,7 @@ layer_lif_backward(
                 const float through = __fsub_rn(1.0f, __fmul_rn(nr.c, sg));   // d vpost_t / d v_t
                 // a gradient on the recorded vpost_t joins what the next step sends down to vpost_t
                 const float below = EXTRA ? __fadd_rn(h, qv[EXTRA ? k : 0]) : h;
-                const float l = __fadd_rn(__fmul_rn(sg, gr[k]), __fmul_rn(through, below));
+                const float l = __fadd_rn(__fmul_rn(sg, GO1 ? g1 : gr[k]), __fmul_rn(through, below));
                 lam = v > nr.lo ? l : 0.f;                      // clamped (or NaN) steps pass nothing on
                 h = __fmul_rn(nr.am, lam);
                 acc_n.add(lam, cur_i);                          // lambda_t * i_t
@@ -701,7 +706,8 @@ __global__ void __launch_bounds__(BLOCK) layer_leaky_forward(float *__restrict__
 // grad_x_t = ((decay_early ? g_t alpha : g_t) * (norm_input ? 1 - alpha : 1))
 // grad_alpha = sum_t g_t out_{t-1}  +  (decay_early ? sum_t g_t (k x_t) : 0)  -  (norm_input ? sum_t (g_t [alpha]) x_t : 0)
 // `x` is only read when WITH_X (alpha gradient wanted and one of the input scalings is on).
-template <int NPL, bool ALPHA, bool WITH_X, bool NT>
+// GO1: grad_out points at one float that stands for every element (the gradient of a sum of the output).
+template <int NPL, bool ALPHA, bool WITH_X, bool NT, bool GO1 = false>
 __global__ void __launch_bounds__(BLOCK) layer_leaky_backward(
     float *__restrict__ grad_x, float *__restrict__ alpha_grad, float *__restrict__ v_init_grad,
     const float *__restrict__ grad_out, const float *__restrict__ grad_v_last, const float *__restrict__ out,
@@ -717,7 +723,10 @@ __global__ void __launch_bounds__(BLOCK) layer_leaky_backward(
     // accesses and all arithmetic sit behind `active`
     const bool active = m0 + lane_off < M;
     const int64_t first = b * M + m0 + lane_off;
-    const float *gp = grad_out + (b * T) * M + m0;
+    const float *gp = GO1 ? nullptr : grad_out + (b * T) * M + m0;
+    V g_all;                                                   // GO1: the one gradient value in every lane element
+#pragma unroll
+    for (int e = 0; e < NPL; ++e) lane_put<NPL>(g_all, e, GO1 ? grad_out[0] : 0.f);
     const float *outp = ALPHA ? out + (b * T) * M + m0 : nullptr;
     const float *xp = WITH_X ? x + (b * T) * M + m0 : nullptr;
     float *op = grad_x + (b * T) * M + m0;
@@ -758,15 +767,17 @@ __global__ void __launch_bounds__(BLOCK) layer_leaky_backward(
         return o;
     };
     struct Stage {
-        V g[U], o[ALPHA ? U : 1], x[WITH_X ? U : 1];
+        V g[GO1 ? 1 : U], o[ALPHA ? U : 1], x[WITH_X ? U : 1];
     };
     // steps t0 .. t0 + U - 1; `spread` = step_bytes, or 0 for a fetch whose data will not be used
     auto fetch = [&](Stage &s, int64_t t0, unsigned spread) {
         __syncthreads();                                   // keeps the block's waves at the same step
         if (!active) return;
-        const Rsrc rg = make_rsrc(gp + t0 * M);
+        if (!GO1) {
+            const Rsrc rg = make_rsrc(gp + t0 * M);
 #pragma unroll
-        for (int u = 0; u < U; ++u) s.g[u] = IO::load(rg, voff, u * spread);
+            for (int u = 0; u < U; ++u) s.g[GO1 ? 0 : u] = IO::load(rg, voff, u * spread);
+        }
         if (WITH_X) {
             const Rsrc rx = make_rsrc(xp + t0 * M);
 #pragma unroll
@@ -786,13 +797,14 @@ __global__ void __launch_bounds__(BLOCK) layer_leaky_backward(
 #pragma unroll
         for (int uu = 0; uu < U; ++uu) {
             const int u = U - 1 - uu;
-            IO::store(advance(t0 + u, s.g[u], s.o[ALPHA ? u : 0], s.x[WITH_X ? u : 0]), r, voff, u * step_bytes);
+            IO::store(advance(t0 + u, GO1 ? g_all : s.g[GO1 ? 0 : u], s.o[ALPHA ? u : 0], s.x[WITH_X ? u : 0]), r, voff,
+                      u * step_bytes);
         }
     };
     const int64_t pairs = T / (2 * U);
     // the steps that do not fill a pair are the newest ones: one at a time
     for (int64_t t = T - 1; active && t >= pairs * 2 * U; --t) {
-        const V gv = IO::load(make_rsrc(gp + t * M), voff, 0u);
+        const V gv = GO1 ? g_all : IO::load(make_rsrc(gp + t * M), voff, 0u);
         V ov = gv, xv = gv;
         if (ALPHA && t >= 1) ov = IO::load(make_rsrc(outp + (t - 1) * M), voff, 0u);
         if (WITH_X) xv = IO::load(make_rsrc(xp + t * M), voff, 0u);
@@ -828,12 +840,22 @@ __global__ void __launch_bounds__(BLOCK) layer_leaky_backward(
 // waves, so that small layers are not starved of parallelism (the spiking forward kernel has a long
 // dependent chain per step and wants 16; the leaky kernels measure best from 8 on).  `align` is the
 // common alignment (bytes) of all (batch, time, neurons) pointers involved.
+// compute units of the current device, asked for once per device
+inline int compute_units()
+{
+    static std::atomic<int> known[64] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    int cus = known[dev].load(std::memory_order_relaxed);
+    if (cus > 0) return cus;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
+    known[dev].store(cus, std::memory_order_relaxed);
+    return cus;
+}
+
 inline int pick_neurons_per_lane(int64_t batch, int64_t neurons, unsigned align, int widest, int waves_per_cu)
 {
-    int cus = 0, dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess ||
-        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
-        cus = 256;
+    const int cus = compute_units();
     const int64_t wanted_lanes = static_cast<int64_t>(cus) * waves_per_cu * WAVE;
     const int64_t n = batch * neurons;
 #ifdef EXODUS_FORCE_NPL
@@ -874,22 +896,32 @@ template <bool SYN, int KIND, int CAPK>
 int launch_bwd(float *grad_x, float *am_g, float *as_g, float *v0_g, float *i0_g, const float *grad_spikes,
                const float *gvl, const float *gil, const float *x, const float *surr, const float *gvr,
                const float *gir, const float *ckpt_v, const float *ckpt_i, const LayerConsts &p, float p0, float p1,
-               int64_t B, int64_t T, int64_t M, hipStream_t s)
+               bool uniform, int64_t B, int64_t T, int64_t M, hipStream_t s)
 {
     const int64_t blocks_per_batch = (M + BWD_BLOCK - 1) / BWD_BLOCK;
     if (blocks_per_batch > 0x7fffffffLL / B) return hipErrorInvalidValue;
     const int64_t blocks = blocks_per_batch * B;
-#define EXODUS_LAUNCH(CK, NT, EX)                                                                                  \
-    hipLaunchKernelGGL((layer_lif_backward<SYN, KIND, CK, NT, EX>), dim3(static_cast<unsigned>(blocks)),          \
+#define EXODUS_LAUNCH(CK, NT, EX, G1)                                                                              \
+    hipLaunchKernelGGL((layer_lif_backward<SYN, KIND, CK, NT, EX, G1>), dim3(static_cast<unsigned>(blocks)),      \
                        dim3(BWD_BLOCK), 0, s, grad_x, am_g, as_g, v0_g, i0_g, grad_spikes, gvl, gil, x, surr, gvr, \
                        gir, ckpt_v, ckpt_i, p, p0, p1, p0 != 0.f ? 1.f / p0 : 0.f, blocks_per_batch, T, M)
-    if (gvr) {
+    if (uniform) {
+        // one value as the gradient of every spike: instances exist for the in-kernel surrogates, without
+        // gradients on the state records
+        if constexpr (KIND == EXODUS_SURR_TENSOR) {
+            return hipErrorInvalidValue;
+        } else {
+            if (gvr) return hipErrorInvalidValue;
+            if (whole_lines(M, {grad_x, x})) EXODUS_LAUNCH(CAPK, true, false, true);
+            else EXODUS_LAUNCH(CAPK, false, false, true);
+        }
+    } else if (gvr) {
         // gradients on the state records: one general instance per surrogate kind
-        EXODUS_LAUNCH(0, false, true);
+        EXODUS_LAUNCH(0, false, true, false);
     } else if (whole_lines(M, {grad_x, grad_spikes, x, surr})) {
-        EXODUS_LAUNCH(CAPK, true, false);
+        EXODUS_LAUNCH(CAPK, true, false, false);
     } else {
-        EXODUS_LAUNCH(CAPK, false, false);
+        EXODUS_LAUNCH(CAPK, false, false, false);
     }
 #undef EXODUS_LAUNCH
     return static_cast<int>(hipGetLastError());
@@ -1062,13 +1094,15 @@ EXODUS_API int exodus_layer_lif_backward(float *grad_input, float *alpha_mem_gra
                                          const float *membr_subtract, const float *theta, const float *theta_low,
                                          int apply_theta_low, int max_num_spikes, int decay_early, int norm_input,
                                          int surrogate_kind, float surr_p0, float surr_p1, const float *surr,
-                                         const float *grad_v_rec, const float *grad_i_rec, int64_t batch, int64_t t,
-                                         int64_t neurons, void *stream)
+                                         const float *grad_v_rec, const float *grad_i_rec, int grad_spikes_uniform,
+                                         int64_t batch, int64_t t, int64_t neurons, void *stream)
 {
     if (bad3(batch, t, neurons)) return hipErrorInvalidValue;
     if (batch == 0 || t == 0 || neurons == 0) return hipSuccess;
     if (too_wide(neurons)) return hipErrorInvalidValue;
     const bool syn = alpha_syn != nullptr;
+    if (grad_spikes_uniform && (surrogate_kind == EXODUS_SURR_TENSOR || grad_v_rec || grad_i_rec))
+        return hipErrorInvalidValue;
     if (!grad_input || !grad_spikes || !input || !ckpt_v || !alpha_mem || !membr_subtract || !theta ||
         (apply_theta_low && !theta_low) || (syn && !ckpt_i) || (surrogate_kind == EXODUS_SURR_TENSOR && !surr))
         return hipErrorInvalidValue;
@@ -1093,8 +1127,8 @@ EXODUS_API int exodus_layer_lif_backward(float *grad_input, float *alpha_mem_gra
 #define EXODUS_BWD(SYN, K)                                                                                        \
     return dispatch_bwd_cap<SYN, K>(p.cap, grad_input, alpha_mem_grad, alpha_syn_grad, vmem_init_grad,            \
                                     isyn_init_grad, grad_spikes, grad_v_last, grad_i_last, input, surr,           \
-                                    grad_v_rec, grad_i_rec, ckpt_v, ckpt_i, p, surr_p0, surr_p1, batch, t,        \
-                                    neurons, s)
+                                    grad_v_rec, grad_i_rec, ckpt_v, ckpt_i, p, surr_p0, surr_p1,                  \
+                                    grad_spikes_uniform != 0, batch, t, neurons, s)
     switch (surrogate_kind) {
         case EXODUS_SURR_TENSOR: if (syn) EXODUS_BWD(true, EXODUS_SURR_TENSOR); EXODUS_BWD(false, EXODUS_SURR_TENSOR);
         case EXODUS_SURR_SINGLE_EXP: if (syn) EXODUS_BWD(true, EXODUS_SURR_SINGLE_EXP); EXODUS_BWD(false, EXODUS_SURR_SINGLE_EXP);
@@ -1113,7 +1147,8 @@ EXODUS_API int exodus_layer_lif_backward_from_input(
     const float *vmem_post_initial, const float *isyn_initial, const float *alpha_mem, const float *alpha_syn,
     const float *membr_subtract, const float *theta, const float *theta_low, int apply_theta_low, int max_num_spikes,
     int decay_early, int norm_input, int surrogate_kind, float surr_p0, float surr_p1, const float *surr,
-    const float *grad_v_rec, const float *grad_i_rec, int64_t batch, int64_t t, int64_t neurons, void *stream)
+    const float *grad_v_rec, const float *grad_i_rec, int grad_spikes_uniform, int64_t batch, int64_t t,
+    int64_t neurons, void *stream)
 {
     if (bad3(batch, t, neurons)) return hipErrorInvalidValue;
     if (batch == 0 || t == 0 || neurons == 0) return hipSuccess;
@@ -1122,7 +1157,8 @@ EXODUS_API int exodus_layer_lif_backward_from_input(
     if (!grad_input || !grad_spikes || !input || !vmem_post_initial || !alpha_mem || !membr_subtract || !theta ||
         (apply_theta_low && !theta_low) || (syn && !isyn_initial) ||
         (surrogate_kind == EXODUS_SURR_TENSOR && !surr) || surrogate_kind < EXODUS_SURR_TENSOR ||
-        surrogate_kind > EXODUS_SURR_HEAVISIDE)
+        surrogate_kind > EXODUS_SURR_HEAVISIDE ||
+        (grad_spikes_uniform && (surrogate_kind == EXODUS_SURR_TENSOR || grad_v_rec || grad_i_rec)))
         return hipErrorInvalidValue;
     if (syn ? ((grad_v_rec != nullptr) != (grad_i_rec != nullptr)) : grad_i_rec != nullptr) return hipErrorInvalidValue;
     // checkpoints of one batch element; the batch is walked in slices of as many elements as fit
@@ -1166,10 +1202,11 @@ EXODUS_API int exodus_layer_lif_backward_from_input(
         if (rc) return rc;
         const int rb = exodus_layer_lif_backward(
             at(grad_input, el), at(alpha_mem_grad, row), at(alpha_syn_grad, row), at(vmem_init_grad, row),
-            at(isyn_init_grad, row), at(grad_spikes, el), at(grad_v_last, row), at(grad_i_last, row), input + el,
+            at(isyn_init_grad, row), grad_spikes_uniform ? grad_spikes : at(grad_spikes, el), at(grad_v_last, row),
+            at(grad_i_last, row), input + el,
             ckpt_v, ckpt_i, q.v_init, q.i_init, q.alpha_mem, q.alpha_syn, q.c, q.theta, q.theta_low, apply_theta_low,
             max_num_spikes, decay_early, norm_input, surrogate_kind, surr_p0, surr_p1, at(surr, el), at(grad_v_rec, el),
-            at(grad_i_rec, el), nb, t, neurons, stream);
+            at(grad_i_rec, el), grad_spikes_uniform, nb, t, neurons, stream);
         if (rb) return rb;
     }
     return hipSuccess;
@@ -1211,8 +1248,8 @@ EXODUS_API int exodus_layer_leaky_forward(float *out, float *v_last, double *out
 EXODUS_API int exodus_layer_leaky_backward(float *grad_input, float *alpha_grad, float *vmem_init_grad,
                                            const float *grad_out, const float *grad_v_last, const float *out,
                                            const float *input, const float *vmem_initial, const float *alpha,
-                                           int decay_early, int norm_input, int64_t batch, int64_t t,
-                                           int64_t neurons, void *stream)
+                                           int decay_early, int norm_input, int grad_out_uniform, int64_t batch,
+                                           int64_t t, int64_t neurons, void *stream)
 {
     if (bad3(batch, t, neurons)) return hipErrorInvalidValue;
     if (batch == 0 || t == 0 || neurons == 0) return hipSuccess;
@@ -1228,19 +1265,24 @@ EXODUS_API int exodus_layer_leaky_backward(float *grad_input, float *alpha_grad,
     p.decay_early = decay_early ? 1 : 0;
     p.norm_input = norm_input ? 1 : 0;
     // with the alpha gradient two or three tensors are double-buffered: two neurons per lane at most
-    const int npl = pick_neurons_per_lane(batch, neurons, common_alignment({grad_input, grad_out, out, input}),
+    const bool g1 = grad_out_uniform != 0;
+    const int npl = pick_neurons_per_lane(batch, neurons, common_alignment({grad_input, g1 ? nullptr : grad_out, out, input}),
                                           want_alpha ? 2 : 4, EXODUS_LEAKY_WAVES);
     const int64_t blocks_per_batch = (neurons + BLOCK * npl - 1) / (BLOCK * npl);
     if (blocks_per_batch > 0x7fffffffLL / batch) return hipErrorInvalidValue;
     const dim3 grid(static_cast<unsigned>(blocks_per_batch * batch)), block(BLOCK);
     hipStream_t s = static_cast<hipStream_t>(stream);
-    const bool nt = whole_lines(neurons, {grad_input, grad_out, out, input});
-#define EXODUS_LK1(NPL, AL, WX, NT)                                                                            \
-    hipLaunchKernelGGL((layer_leaky_backward<NPL, AL, WX, NT>), grid, block, 0, s, grad_input, alpha_grad,    \
+    const bool nt = whole_lines(neurons, {grad_input, g1 ? nullptr : grad_out, out, input});
+#define EXODUS_LK1(NPL, AL, WX, NT, G1)                                                                        \
+    hipLaunchKernelGGL((layer_leaky_backward<NPL, AL, WX, NT, G1>), grid, block, 0, s, grad_input, alpha_grad, \
                        vmem_init_grad, grad_out, grad_v_last, out, input, p, blocks_per_batch, t, neurons)
 #define EXODUS_LK(NPL, AL, WX)                                                                                 \
     do {                                                                                                       \
-        if (nt) EXODUS_LK1(NPL, AL, WX, true); else EXODUS_LK1(NPL, AL, WX, false);                            \
+        if (g1) {                                                                                              \
+            if (nt) EXODUS_LK1(NPL, AL, WX, true, true); else EXODUS_LK1(NPL, AL, WX, false, true);            \
+        } else {                                                                                               \
+            if (nt) EXODUS_LK1(NPL, AL, WX, true, false); else EXODUS_LK1(NPL, AL, WX, false, false);          \
+        }                                                                                                      \
     } while (0)
     if (npl == 4) {
         EXODUS_LK(4, false, false);

@@ -23,7 +23,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("EXODUS_HIP_LIBRARY") or os.path.join(_HERE, "libexodus_hip.so")
 
 SURR_TENSOR, SURR_SINGLE_EXP, SURR_PERIODIC_EXP, SURR_HEAVISIDE = 0, 1, 2, 3
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 _p = ctypes.c_void_p
 _i64 = ctypes.c_int64
@@ -47,13 +47,19 @@ _SIGNATURES = {
     "exodus_spike_backward": ([_p] * 4 + [_f, _f, _i64, _i64, _p], _int),
     "exodus_layer_checkpoint_interval": ([], _int),
     "exodus_layer_lif_forward": ([_p] * 16 + [_int, _int, _int, _int, _int, _i64, _i64, _i64, _p], _int),
-    "exodus_layer_lif_backward": ([_p] * 18 + [_int, _int, _int, _int, _int, _f, _f, _p, _p, _p, _i64, _i64, _i64, _p], _int),
+    "exodus_layer_lif_backward": ([_p] * 18 + [_int, _int, _int, _int, _int, _f, _f, _p, _p, _p, _int, _i64, _i64, _i64, _p], _int),
     "exodus_layer_scratch_floats": ([], _i64),
-    "exodus_layer_lif_backward_from_input": ([_p] * 16 + [_int, _int, _int, _int, _int, _f, _f, _p, _p, _p, _i64, _i64, _i64, _p], _int),
+    "exodus_layer_lif_backward_from_input": ([_p] * 16 + [_int, _int, _int, _int, _int, _f, _f, _p, _p, _p, _int, _i64, _i64, _i64, _p], _int),
     "exodus_layer_leaky_forward": ([_p] * 6 + [_int, _int, _i64, _i64, _i64, _p], _int),
-    "exodus_layer_leaky_backward": ([_p] * 9 + [_int, _int, _i64, _i64, _i64, _p], _int),
-    "exodus_hbm_regions_create": ([_int, ctypes.c_uint64, ctypes.c_uint64, ctypes.c_uint64, _int, _p], _int),
+    "exodus_layer_leaky_backward": ([_p] * 9 + [_int, _int, _int, _i64, _i64, _i64, _p], _int),
+    "exodus_hbm_regions_create": ([_int, ctypes.c_uint64, ctypes.c_uint64, ctypes.c_uint64, _int, ctypes.c_uint64, _p], _int),
     "exodus_hbm_regions_destroy": ([_int], _int),
+    "exodus_hbm_alloc_striped": ([ctypes.c_size_t, _int, _p], _p),
+    "exodus_hbm_alloc_region0": ([ctypes.c_size_t, _int, _p], _p),
+    "exodus_hbm_alloc_region1": ([ctypes.c_size_t, _int, _p], _p),
+    "exodus_hbm_alloc_region2": ([ctypes.c_size_t, _int, _p], _p),
+    "exodus_hbm_free": ([_p, ctypes.c_size_t, _int, _p], None),
+    "exodus_hbm_usage": ([_int, _p, _p], _int),
 }
 
 
@@ -449,12 +455,12 @@ def layerLifForward(input, vmemPostInitial, isynInitial, alphaMem, alphaSyn, mem
         _rows(_dev(thetaLow, "thetaLow", input), "thetaLow", n)
     else:
         thetaLow = None
-    # big outputs go where hbm.enable() wants them (another region of HBM than what the kernel reads)
+    # big outputs go where hbm.enable() wants them (memory striped over the regions of HBM)
     spikes = hbm.empty_like(input) if outSpikes is None else outSpikes
     if spikes.shape != input.shape:
         raise RuntimeError("outSpikes must have the shape of input")
     _dev(spikes, "outSpikes", input)
-    new = lambda *shape: (hbm.empty(shape, input, away_from=[input, spikes]) if len(shape) == 3
+    new = lambda *shape: (hbm.empty(shape, input) if len(shape) == 3
                           else torch.empty(shape, dtype=torch.float32, device=input.device))
     n_ck = (t + checkpointInterval() - 1) // checkpointInterval()
     state_shape = (n,) if stateShape is None else tuple(stateShape)
@@ -491,9 +497,12 @@ def layerLifBackward(gradSpikes, gradVLast, gradILast, input, ckptV, ckptI, vmem
                      gradInput: Optional[torch.Tensor] = None, surr: Optional[torch.Tensor] = None,
                      gradVRec: Optional[torch.Tensor] = None, gradIRec: Optional[torch.Tensor] = None,
                      wantAlphaMemGrad: bool = True, wantAlphaSynGrad: bool = True, wantVInitGrad: bool = True,
-                     wantIInitGrad: bool = True):
+                     wantIInitGrad: bool = True, gradUniform: bool = False):
     """Returns (gradInput, alphaMemGrad, alphaSynGrad | None, vInitGrad, iInitGrad | None); a per-neuron
     gradient that is not wanted is neither computed nor allocated and comes back as None.
+    ``gradUniform``: ``gradSpikes`` is a one-element tensor whose value is the gradient of every spike (the
+    gradient of a sum of the output); the kernel then reads one tensor less.  Only with an in-kernel
+    surrogate and without ``gradVRec`` / ``gradIRec``.
     ``surrogateKind == SURR_TENSOR`` takes the spike function's derivative from ``surr`` (batch, time, neurons).
     ``gradVRec`` / ``gradIRec`` (batch, time, neurons) are gradients on the forward's state records; one that is
     missing while the other is given counts as zero.
@@ -503,7 +512,12 @@ def layerLifBackward(gradSpikes, gradVLast, gradILast, input, ckptV, ckptI, vmem
     b, t, m = input.shape
     n = b * m
     syn = alphaSyn is not None
-    if _btm(gradSpikes, "gradSpikes", input).shape != input.shape:
+    if gradUniform:
+        if _dev(gradSpikes, "gradSpikes", input).numel() != 1:
+            raise RuntimeError("gradSpikes must hold one value when gradUniform is set")
+        if surrogateKind == SURR_TENSOR or gradVRec is not None or gradIRec is not None:
+            raise RuntimeError("gradUniform needs an in-kernel surrogate and no gradients on the state records")
+    elif _btm(gradSpikes, "gradSpikes", input).shape != input.shape:
         raise RuntimeError("gradSpikes must have the shape of input")
     n_ck = (t + checkpointInterval() - 1) // checkpointInterval()
     from_input = ckptV is None
@@ -525,7 +539,7 @@ def layerLifBackward(gradSpikes, gradVLast, gradILast, input, ckptV, ckptI, vmem
     else:
         thetaLow = None
     if gradInput is None:
-        gradInput = hbm.empty_like(input, away_from=[input, gradSpikes])
+        gradInput = hbm.empty_like(input)
     elif _btm(gradInput, "gradInput", input).shape != input.shape:
         raise RuntimeError("gradInput must have the shape of input")
     if surrogateKind == SURR_TENSOR:
@@ -546,12 +560,11 @@ def layerLifBackward(gradSpikes, gradVLast, gradILast, input, ckptV, ckptI, vmem
     # the kernel writes every neuron's entry of each vector it is given -- unless there is no step to
     # walk: then nothing is launched, the decay factors have no influence and a gradient on a final
     # state is the gradient of the initial state it equals
-    if t == 0:
-        z = lambda want: torch.zeros(n, dtype=torch.float32, device=input.device) if want else None
-    else:
-        z = lambda want: torch.empty(n, dtype=torch.float32, device=input.device) if want else None
-    am_g, v0_g = z(wantAlphaMemGrad), z(wantVInitGrad)
-    as_g, i0_g = z(syn and wantAlphaSynGrad), z(syn and wantIInitGrad)
+    # (the wanted vectors are rows of one allocation)
+    wanted = [bool(wantAlphaMemGrad), bool(wantVInitGrad), bool(syn and wantAlphaSynGrad), bool(syn and wantIInitGrad)]
+    block = (torch.zeros if t == 0 else torch.empty)((sum(wanted), n), dtype=torch.float32, device=input.device)
+    taken = iter(block.unbind(0))
+    am_g, v0_g, as_g, i0_g = (next(taken) if w else None for w in wanted)
     if t == 0:
         if v0_g is not None and gradVLast is not None:
             v0_g.copy_(gradVLast.reshape(-1))
@@ -562,7 +575,7 @@ def layerLifBackward(gradSpikes, gradVLast, gradILast, input, ckptV, ckptI, vmem
     tail = (_ptr(vmemPostInitial), _ptr(isynInitial) if syn else None, _ptr(alphaMem), _ptr(alphaSyn) if syn else None,
             _ptr(membrSubtract), _ptr(theta), _ptr(thetaLow), int(bool(applyThetaLow)), int(maxNumSpikes),
             int(bool(decayEarly)), int(bool(normInput)), int(surrogateKind), float(surrP0), float(surrP1), _ptr(surr),
-            _ptr(gradVRec), _ptr(gradIRec), b, t, m, _stream(input))
+            _ptr(gradVRec), _ptr(gradIRec), int(bool(gradUniform)), b, t, m, _stream(input))
     with torch.cuda.device(input.device):
         if from_input:
             _check(lib.exodus_layer_lif_backward_from_input(*head, *tail), "exodus_layer_lif_backward_from_input")
@@ -597,24 +610,32 @@ def layerLeakyForward(input, vmemInitial, alpha, decayEarly: bool, normInput: bo
 
 
 def layerLeakyBackward(gradOut, gradVLast, out, input, vmemInitial, alpha, decayEarly: bool, normInput: bool,
-                       needAlphaGrad: bool):
-    """Returns (gradInput, alphaGrad | None, vInitGrad)."""
-    _btm(gradOut, "gradOut")
-    b, t, m = gradOut.shape
+                       needAlphaGrad: bool, shape: Optional[tuple] = None):
+    """Returns (gradInput, alphaGrad | None, vInitGrad).  With ``shape`` = (batch, time, neurons), ``gradOut`` is a
+    one-element tensor whose value is the gradient of every output (the gradient of a sum)."""
+    uniform = shape is not None
+    if uniform:
+        if _dev(gradOut, "gradOut").numel() != 1:
+            raise RuntimeError("gradOut must hold one value when shape is given")
+        b, t, m = (int(v) for v in shape)
+    else:
+        _btm(gradOut, "gradOut")
+        b, t, m = gradOut.shape
     n = b * m
     _rows(_dev(alpha, "alpha", gradOut), "alpha", n)
     if gradVLast is not None and _dev(gradVLast, "gradVLast", gradOut).numel() != n:
         raise RuntimeError(f"gradVLast must hold {n} values")
     need_x = needAlphaGrad and (decayEarly or normInput)
     if needAlphaGrad:
-        if _btm(out, "out", gradOut).shape != gradOut.shape:
+        if tuple(_btm(out, "out", gradOut).shape) != (b, t, m):
             raise RuntimeError("out must have the shape of gradOut")
         _rows(_dev(vmemInitial, "vmemInitial", gradOut), "vmemInitial", n)
-    if need_x and _btm(input, "input", gradOut).shape != gradOut.shape:
+    if need_x and tuple(_btm(input, "input", gradOut).shape) != (b, t, m):
         raise RuntimeError("input must have the shape of gradOut")
-    grad_input = hbm.empty_like(gradOut, away_from=[gradOut, out if needAlphaGrad else None, input if need_x else None])
-    alpha_grad = torch.zeros(n, dtype=torch.float32, device=gradOut.device) if needAlphaGrad else None
-    v_init_grad = torch.zeros(n, dtype=torch.float32, device=gradOut.device)
+    grad_input = hbm.empty((b, t, m), gradOut)
+    block = torch.zeros((2 if needAlphaGrad else 1, n), dtype=torch.float32, device=gradOut.device)
+    v_init_grad = block[0]
+    alpha_grad = block[1] if needAlphaGrad else None
     if t == 0 and gradVLast is not None:
         v_init_grad.copy_(gradVLast.reshape(-1))
     with torch.cuda.device(gradOut.device):
@@ -622,5 +643,5 @@ def layerLeakyBackward(gradOut, gradVLast, out, input, vmemInitial, alpha, decay
             _ptr(grad_input), _ptr(alpha_grad), _ptr(v_init_grad), _ptr(gradOut), _ptr(gradVLast),
             _ptr(out) if needAlphaGrad else None, _ptr(input) if need_x else None,
             _ptr(vmemInitial) if needAlphaGrad else None, _ptr(alpha), int(bool(decayEarly)), int(bool(normInput)),
-            b, t, m, _stream(gradOut)), "exodus_layer_leaky_backward")
+            int(uniform), b, t, m, _stream(gradOut)), "exodus_layer_leaky_backward")
     return grad_input, alpha_grad, v_init_grad

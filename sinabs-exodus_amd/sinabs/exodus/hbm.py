@@ -8,29 +8,36 @@ less: inputs in one region and outputs striped over the others is the best case,
 it, outputs in a single region 9-25 % (reads alone and writes alone in flat copies do not care).
 
 A process cannot ask the driver for memory of a region, and the order in which the driver hands memory out
-follows the regions only on a machine that has run nothing yet.  So the library sorts: it takes the free
-device memory in pages of 64 MiB, judges every 4 GiB of consecutively created pages with timed copies (which chunks
-disturb each other), and maps pages into four address ranges: one per region, and a *striped* one whose consecutive
-pages come from regions 0, 1, 2, 0, 1, 2, ... (``exodus_hbm_regions_create``, csrc/exodus_hbm.hip).  The rest goes
-back to the driver.  ``HbmRegions`` hands out tensors from these ranges.
+follows the regions only on a machine that has run nothing yet.  So the library takes the free device memory in
+chunks, optionally judges them with timed copies (which chunks disturb each other), and maps 64 MiB pages into four
+address ranges: one per region, and a *striped* one whose consecutive pages come from regions 0, 1, 2, 0, 1, 2, ...
+(``exodus_hbm_regions_create``, csrc/exodus_hbm.hip).  The rest goes back to the driver.
 
-``empty(shape)`` allocates in the striped range, ``empty(shape, region=k)`` in the range of region k (0, 1, 2).
-After ``enable()`` the kernels' wrappers (``_hip.layerLifForward`` and friends, the (rows, time) wrappers, the
-``IntegrateAndFire`` Function) allocate their big outputs through ``empty_like`` / ``empty`` of this module -- striped when there is a striped range; with region ranges only, in a
-range that none of the tensors the kernel reads lies in (tensors of the ranges are recognised by their addresses;
-for a tensor from the ordinary allocator the range it copies to slowest is looked up once per storage with three
-short timed copies).  Without ``enable()`` nothing changes.  The reference has no counterpart (its CUDA
-extension allocates outputs with ``torch.empty_like``, reference cuda/bindings.cu:98,144,183).
+Tensors come out of a range through PyTorch's own caching allocator: every range is a ``torch.cuda.MemPool`` whose
+segments the library's ``exodus_hbm_alloc_*`` / ``exodus_hbm_free`` supply (``CUDAPluggableAllocator``).  PyTorch
+splits, caches and reuses the segments as it does ordinary memory, which includes keeping track of the streams a
+block was used on (``Tensor.record_stream``): a tensor of a range is as safe across streams as any other tensor.
 
-Memory of a released tensor is handed out again at once, without regard to streams: a tensor from here is for
-work on one stream, or has to outlive (``torch.cuda.synchronize``) what other streams do with it.
+``enable()`` makes the ranges and from then on the kernels' wrappers (``_hip.layerLifForward`` and friends, the
+(rows, time) wrappers, the ``IntegrateAndFire`` Function) allocate their big outputs in the striped range.
+``with placement():`` sends *every* allocation of the calling thread there (what torch itself allocates in a forward
+pass: activations of other layers, temporaries); ``enable(everything=True)`` does that for all threads until
+``disable()``, which covers the gradients that autograd's own thread allocates in a backward pass.  Without
+``enable()`` nothing changes.  The reference has no counterpart (its CUDA extension allocates outputs with
+``torch.empty_like``, reference cuda/bindings.cu:98,144,183).
+
+While a HIP graph is being captured the wrappers leave allocation to the capture's own pool (a graph's memory must
+not be handed to anybody else between replays, which is what that pool guarantees); ``everything=True`` would
+override that pool and must not be active during a capture.
 """
 from __future__ import annotations
 
+import contextlib
 import ctypes
 import threading
+import time
 import warnings
-from typing import Dict, Iterable, List, Optional, Sequence
+from typing import Dict, List, Optional, Sequence
 
 import torch
 
@@ -39,13 +46,13 @@ CHUNK = 4 * GIB                 # physical memory is sorted in pieces of this si
 FINER_CHUNK = 256 * 2 ** 20     # ... and in pieces of this size when the big ones show no regions (memory that earlier
                                 # processes left mixed below 4 GiB is mostly still in order at this scale)
 REGIONS_NOT_FOUND = -3          # EXODUS_ERROR_REGIONS_NOT_FOUND of include/exodus_hip.h
-ALIGN = 2 * 2 ** 20             # every tensor of a range starts on a 2 MiB boundary
+RANGE_IN_USE = -4               # EXODUS_ERROR_RANGE_IN_USE
 PROBES = 15                     # EXODUS_HBM_PROBES of include/exodus_hip.h
 ARENAS = 4                      # EXODUS_HBM_ARENAS: one range per region and the striped one
 STRIPED = 3                     # index of the striped range
-SMALLEST_PLACED = 2 ** 20       # smaller requests are left to the ordinary allocator
-PROBE_BYTES = GIB               # the slice of a foreign tensor that is timed against the ranges
-SMALLEST_PROBE = 256 * 2 ** 20  # foreign tensors below this are not classified (too short to time, too small to matter)
+SMALLEST_PLACED = 2 ** 20       # the wrappers leave smaller outputs to the ordinary allocator
+_ALLOC_NAMES = ("exodus_hbm_alloc_region0", "exodus_hbm_alloc_region1", "exodus_hbm_alloc_region2",
+                "exodus_hbm_alloc_striped")
 
 
 class _Report(ctypes.Structure):
@@ -58,32 +65,19 @@ class _Report(ctypes.Structure):
                 ("probe_other_kind_GBs", ctypes.c_float), ("copy_inside_GBs", ctypes.c_float * 3),
                 ("copy_across_GBs", ctypes.c_float * 6), ("copy_striped_GBs", ctypes.c_float),
                 ("probe_chunk", ctypes.c_int32 * PROBES),
-                ("probe_kind", ctypes.c_int32 * PROBES), ("probe_pair_GBs", (ctypes.c_float * PROBES) * PROBES)]
+                ("probe_kind", ctypes.c_int32 * PROBES), ("probe_pair_GBs", (ctypes.c_float * PROBES) * PROBES),
+                ("phase_s", ctypes.c_float * 4)]
 
 
-class _Block:
-    """What torch keeps alive for as long as a tensor of a range has storage; gives the bytes back after."""
-
-    def __init__(self, owner: "HbmRegions", k: int, offset: int, nbytes: int, rounded: int):
-        self.owner, self.k, self.offset, self.rounded = owner, k, offset, rounded
-        self.__cuda_array_interface__ = {"shape": (nbytes,), "typestr": "|u1", "version": 2,
-                                         "data": (owner.bases[k] + offset, False)}
-
-    def __del__(self):
-        try:
-            self.owner._give_back(self.k, self.offset, self.rounded)
-        except Exception:                                  # interpreter shutdown: nothing left to give back to
-            pass
-
-
-def _create(lib, device_index: int, bytes_per_region: int, bytes_striped: int, chunk_sizes: Sequence[int], sort: bool):
+def _create(lib, device_index: int, bytes_per_region: int, bytes_striped: int, chunk_sizes: Sequence[int], sort: bool,
+            take_limit: int = 0):
     """``exodus_hbm_regions_create`` with each of ``chunk_sizes`` in turn until one shows the regions (or none is
     left); returns (status, report, chunk size used).  A striped range that came out unsorted is given back before
     the next try."""
     for attempt, size in enumerate(chunk_sizes):
         rep = _Report()
         rc = lib.exodus_hbm_regions_create(device_index, bytes_per_region, bytes_striped, int(size), int(sort),
-                                           ctypes.byref(rep))
+                                           int(take_limit), ctypes.byref(rep))
         no_regions = rc == REGIONS_NOT_FOUND or (rc == 0 and sort and rep.kinds_found != 3)
         if not no_regions or attempt + 1 == len(chunk_sizes):
             break
@@ -92,41 +86,32 @@ def _create(lib, device_index: int, bytes_per_region: int, bytes_striped: int, c
     return rc, rep, int(size)
 
 
-def _copy_rate(dst: torch.Tensor, src: torch.Tensor, reps: int = 5) -> float:
-    """bytes moved per millisecond by dst.copy_(src), median of `reps` (events on the current stream)"""
-    dst.copy_(src)
-    dst.copy_(src)
-    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
-    for a, b in ev:
-        a.record()
-        dst.copy_(src)
-        b.record()
-    torch.cuda.synchronize()
-    ms = sorted(a.elapsed_time(b) for a, b in ev)[reps // 2]
-    return 2 * src.numel() * src.element_size() / ms
-
-
 class HbmRegions:
     """Address ranges of device memory sorted by region of HBM: one per region (``gib_per_region`` each, may be 0)
-    and a striped one (``gib_striped``, may be 0) whose 64 MiB pages alternate between the regions.
+    and a striped one (``gib_striped``, may be 0) whose 64 MiB pages alternate between the regions; each range
+    is the backing store of a ``torch.cuda.MemPool``.
 
-    The sizes are what the ranges hold for good (until ``close()``); a request that a range cannot
-    serve is passed to the ordinary allocator, which is harmless but loses the placement.  Creating the ranges
-    takes nearly all free device memory for a second or two and gives back what it does not keep, so do it
-    early, before the program's big allocations.  ``chunk_bytes`` is the amount of memory judged as one piece
-    (4 GiB; smaller pieces copy too quickly to tell the regions apart as reliably); when pieces of that size show no
-    regions -- memory that earlier processes left mixed -- the sorting is repeated once with ``finer_chunk_bytes``.  ``report`` holds what the sorting
-    measured; ``sort=False`` skips the timed copies and makes the striped range from chunks spread evenly over the
-    free memory (what is done anyway when the memory shows no regions); ``verified`` says
-    whether copies between regions beat copies inside them on the finished ranges (on the probe chunks when there
-    are no region ranges).
+    The sizes are what the ranges hold for good (until ``close()``); what a range cannot serve comes from the
+    ordinary allocator, which is harmless but loses the placement.  Creating the ranges takes nearly all free
+    device memory for a moment and gives back what it does not keep, so do it early, before the program's big
+    allocations, and not while another process is starting up on the same GPU (``take_limit_gib`` bounds what is
+    held, at the price stated in include/exodus_hip.h).
+    ``sort=False`` (the default for a striped range alone) builds the striped range from chunks of the first,
+    second and last third of the free memory in turn: on a machine that hands memory out in address order those are
+    the regions, on one that does not the memory is a mixture already; nothing is timed, so nothing depends on what
+    else the machine is doing.  ``sort=True`` (the default when ranges of single regions are asked for, which need
+    it) judges the memory with timed copies in pieces of ``chunk_bytes`` (4 GiB; smaller pieces copy too
+    quickly to tell the regions apart as reliably), and once more with ``finer_chunk_bytes`` when those show no
+    regions -- memory that earlier processes left mixed; it takes several seconds.  ``report`` holds what was measured, ``setup_s`` the time
+    the whole set-up took, ``verified`` whether copies between regions beat copies inside them on the finished
+    ranges (on the probe chunks when there are no region ranges).
     Raises RuntimeError when too little memory is free, or when ranges of single regions are asked for and the
     device's memory shows no three regions (a striped range alone is then still made, ``sorted`` False).
     """
 
     def __init__(self, gib_per_region: float = 0.0, gib_striped: float = 48.0,
-                 device: Optional[torch.device] = None, chunk_bytes: int = CHUNK, sort: bool = True,
-                 finer_chunk_bytes: Optional[int] = FINER_CHUNK):
+                 device: Optional[torch.device] = None, chunk_bytes: int = CHUNK, sort: Optional[bool] = None,
+                 finer_chunk_bytes: Optional[int] = FINER_CHUNK, take_limit_gib: Optional[float] = None):
         from . import _hip
         self.device = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
         if self.device.type != "cuda":
@@ -135,6 +120,8 @@ class HbmRegions:
             self.device = torch.device("cuda", torch.cuda.current_device())
         if gib_per_region < 0 or gib_striped < 0 or (gib_per_region == 0 and gib_striped == 0):
             raise ValueError("gib_per_region and gib_striped must not be negative, and one of them positive")
+        if sort is None:
+            sort = gib_per_region > 0
         if not sort and gib_per_region:
             raise ValueError("ranges of single regions (gib_per_region) need the sorting")
         if chunk_bytes <= 0 or chunk_bytes % (64 * 2 ** 20):
@@ -142,16 +129,21 @@ class HbmRegions:
         if gib_per_region + gib_striped / 3 > 80:
             raise ValueError("gib_per_region + gib_striped / 3 must not exceed 80 (rounded up to whole chunks of "
                              "4 GiB): that much is taken from each region, and a region has 96 GiB")
+        if take_limit_gib is not None and take_limit_gib <= 0:
+            raise ValueError("take_limit_gib must be positive (None: no bound)")
         self._lib = _hip.lib
+        self._lib_path = _hip.LIB_PATH
         sizes = [int(chunk_bytes)]
         if sort and finer_chunk_bytes and finer_chunk_bytes < chunk_bytes:
             sizes.append(int(finer_chunk_bytes))
+        t0 = time.perf_counter()
         with torch.cuda.device(self.device):
             torch.zeros(1, device=self.device)             # the device's context exists
             torch.cuda.empty_cache()                       # what torch has cached cannot be sorted
             torch.cuda.synchronize()
             rc, rep, size = _create(self._lib, self.device.index, int(gib_per_region * GIB), int(gib_striped * GIB),
-                                    sizes, bool(sort))
+                                    sizes, bool(sort), 0 if take_limit_gib is None else int(take_limit_gib * GIB))
+        self.setup_s = time.perf_counter() - t0
         self.chunk_bytes = size                            # the size the ranges were sorted in
         self.report: Dict[str, object] = {
             "chunks_examined": rep.chunks_examined, "kinds_found": rep.kinds_found,
@@ -159,7 +151,8 @@ class HbmRegions:
             "threshold_GBs": rep.threshold_GBs, "probe_chunks_same_region_GBs": rep.probe_same_kind_GBs,
             "probe_chunks_other_region_GBs": rep.probe_other_kind_GBs,
             "inside_one_range_GBs": list(rep.copy_inside_GBs), "across_ranges_GBs": list(rep.copy_across_GBs),
-            "inside_striped_range_GBs": rep.copy_striped_GBs}
+            "inside_striped_range_GBs": rep.copy_striped_GBs,
+            "seconds_taking_sorting_building_checking": [round(v, 3) for v in rep.phase_s]}
         # the probe chunks: position, group, and the copy rate between every two (what the groups were read from)
         self.probes = {"chunk": list(rep.probe_chunk), "kind": list(rep.probe_kind),
                        "pair_GBs": [[rep.probe_pair_GBs[a][b] for b in range(PROBES)] for a in range(PROBES)]}
@@ -171,14 +164,15 @@ class HbmRegions:
         self.bases: List[int] = [int(rep.base[k] or 0) for k in range(ARENAS)]
         self.sizes: List[int] = [int(rep.bytes[k]) for k in range(ARENAS)]
         self.page_bytes = int(rep.page_bytes)
-        # False: the copies showed no three regions (memory that came back from earlier processes as a mixture of
-        # them); the striped range is then made of chunks spread over the memory, as they are
+        # False: no timed copies were made, or they showed no three regions (memory that came back from earlier
+        # processes as a mixture of them); the striped range is then made of chunks spread over the memory, as they are
         self.sorted = rep.kinds_found == 3
-        self._free: List[List[List[int]]] = [[[0, n]] for n in self.sizes]   # per range: [offset, bytes], by offset
+        self._pools: Dict[int, "torch.cuda.MemPool"] = {}
+        self._allocators: Dict[int, object] = {}           # the pools' allocators have to outlive them
         self._lock = threading.Lock()
-        self._live, self._closing, self._closed = 0, False, False
-        self._foreign: Dict[int, int] = {}
-        self._anchors: Optional[List[torch.Tensor]] = None
+        self._closing, self._closed = False, False
+        self._everything = False
+        self._local = threading.local()                    # .depth: placement() contexts this thread is inside
         inside = [r for r in rep.copy_inside_GBs if r > 0] or [rep.probe_same_kind_GBs]
         across = [r for r in rep.copy_across_GBs if r > 0] or [rep.probe_other_kind_GBs]
         # single pairs of chunks scatter by a few percent around 6.0 (same region) and 6.35 TB/s (two regions);
@@ -188,46 +182,72 @@ class HbmRegions:
             warnings.warn(f"HbmRegions: copies between the regions are not clearly faster than copies "
                           f"inside them ({self.report}); allocation works, the gain may not be there")
 
-    # ------------------------------------------------------------------ the ranges' free lists
-    def _take(self, k: int, nbytes: int) -> Optional[int]:
-        rounded = -(-nbytes // ALIGN) * ALIGN
+    # ------------------------------------------------------------------ the pools
+    def pool(self, k: int = STRIPED) -> "torch.cuda.MemPool":
+        """The ``torch.cuda.MemPool`` on range ``k`` (0, 1, 2: a region's; ``STRIPED``), made on first use."""
+        k = int(k)
+        if not 0 <= k < ARENAS or not self.sizes[k]:
+            raise ValueError(f"these ranges have no range {k}")
         with self._lock:
             if self._closing:
-                return None
-            for slot, (off, n) in enumerate(self._free[k]):
-                if n >= rounded:
-                    if n == rounded:
-                        del self._free[k][slot]
-                    else:
-                        self._free[k][slot] = [off + rounded, n - rounded]
-                    self._live += 1
-                    return off
-        return None
+                raise RuntimeError("these ranges were closed")
+            if k not in self._pools:
+                self._allocators[k] = torch.cuda.memory.CUDAPluggableAllocator(self._lib_path, _ALLOC_NAMES[k],
+                                                                               "exodus_hbm_free")
+                self._pools[k] = torch.cuda.MemPool(self._allocators[k].allocator())
+            return self._pools[k]
 
-    def _give_back(self, k: int, offset: int, rounded: int) -> None:
-        with self._lock:
-            free = self._free[k]
-            slot = 0
-            while slot < len(free) and free[slot][0] < offset:
-                slot += 1
-            free.insert(slot, [offset, rounded])
-            if slot + 1 < len(free) and free[slot][0] + free[slot][1] == free[slot + 1][0]:
-                free[slot][1] += free.pop(slot + 1)[1]
-            if slot > 0 and free[slot - 1][0] + free[slot - 1][1] == free[slot][0]:
-                free[slot - 1][1] += free.pop(slot)[1]
-            self._live -= 1
-            last = self._closing and self._live == 0
-        if last:
-            self._destroy()
+    def _covered(self) -> bool:
+        """True when this thread's allocations go to the striped range anyway."""
+        return self._everything or getattr(self._local, "depth", 0) > 0
 
-    def _destroy(self) -> None:
-        if not self._closed:
-            self._closed = True
-            self._lib.exodus_hbm_regions_destroy(self.device.index)     # waits for the device first
+    @contextlib.contextmanager
+    def allocating(self, k: int = STRIPED):
+        """Inside the block every device allocation of the calling thread comes from range ``k``
+        (``torch.cuda.use_mem_pool``).  Inside ``placement()`` or under ``enable(everything=True)`` the striped range
+        is being allocated from already and the block changes nothing."""
+        if self._covered() or self._closing:
+            yield
+            return
+        with torch.cuda.use_mem_pool(self.pool(k), device=self.device):
+            yield
 
-    def bytes_free(self, k: int) -> int:
-        with self._lock:
-            return sum(n for _, n in self._free[k])
+    @contextlib.contextmanager
+    def placement(self):
+        """Inside the block every device allocation of the calling thread comes from the striped range: whatever
+        torch allocates for the operations in it, not only the outputs of this package's kernels."""
+        if self._covered() or self._closing or not self.sizes[STRIPED]:
+            yield
+            return
+        with torch.cuda.use_mem_pool(self.pool(STRIPED), device=self.device):
+            self._local.depth = getattr(self._local, "depth", 0) + 1
+            try:
+                yield
+            finally:
+                self._local.depth -= 1
+
+    def _set_everything(self, on: bool) -> None:
+        if on == self._everything:
+            return
+        pool = self.pool(STRIPED)
+        if on:
+            torch._C._cuda_beginAllocateToPool(self.device.index, pool.id)
+        else:
+            torch._C._cuda_endAllocateToPool(self.device.index, pool.id)
+            torch._C._cuda_releasePool(self.device.index, pool.id)
+        self._everything = on
+
+    def bytes_in_use(self, k: int = STRIPED) -> int:
+        """Bytes of range ``k`` that PyTorch's allocator currently holds as segments (in use or cached)."""
+        used = (ctypes.c_uint64 * ARENAS)()
+        self._lib.exodus_hbm_usage(self.device.index, used, None)
+        return int(used[k])
+
+    def bytes_elsewhere(self) -> int:
+        """Bytes that the pools took from the ordinary device memory because their range was full."""
+        used, other = (ctypes.c_uint64 * ARENAS)(), ctypes.c_uint64(0)
+        self._lib.exodus_hbm_usage(self.device.index, used, ctypes.byref(other))
+        return int(other.value)
 
     # ------------------------------------------------------------------ queries
     def pool_of(self, t: torch.Tensor) -> Optional[int]:
@@ -238,110 +258,139 @@ class HbmRegions:
                 return k
         return None
 
-    def region_of(self, t: torch.Tensor) -> Optional[int]:
-        """The region (0, 1, 2) that holds ``t``: by address for tensors of the regions' ranges, by three timed
-        copies (once per storage) for others; None for tensors of the striped range, tensors too small to tell or
-        to matter, and when there are no region ranges to time against."""
-        k = self.pool_of(t)
-        if k is not None:
-            return k if k < STRIPED else None
-        nbytes = t.numel() * t.element_size()
-        if nbytes < SMALLEST_PROBE or not t.is_contiguous() or t.device != self.device or not self.sizes[0]:
-            return None
-        key = t.untyped_storage().data_ptr()
-        if key not in self._foreign:
-            if torch.cuda.is_current_stream_capturing():
-                return None                                # timing needs to wait for the device
-            with torch.cuda.device(self.device), torch.no_grad():
-                if self._anchors is None:
-                    n = min(PROBE_BYTES, min(self.sizes[:3]) // 4)
-                    self._anchors = [self.empty((n,), torch.uint8, region=j) for j in range(3)]
-                n = min(self._anchors[0].numel(), nbytes)
-                src = t.detach().reshape(-1).view(torch.uint8)[:n]
-                rates = [_copy_rate(a[:n], src) for a in self._anchors]
-            self._foreign[key] = min(range(3), key=lambda j: rates[j])   # slowest copy = same kind of memory
-            if len(self._foreign) > 4096:
-                self._foreign.pop(next(iter(self._foreign)))
-        return self._foreign[key]
-
-    def _pick(self, away_from: Iterable[Optional[torch.Tensor]]) -> int:
-        taken = [0, 0, 0]
-        for t in away_from:
-            if isinstance(t, torch.Tensor) and t.is_cuda and t.numel():
-                k = self.region_of(t)
-                if k is not None:
-                    taken[k] += t.numel() * t.element_size()
-        return min(range(3), key=lambda k: (taken[k], k))
+    def live_blocks(self) -> List[tuple]:
+        """(address, bytes, range) of every block of the ranges that a tensor still occupies, from PyTorch's own
+        book-keeping (``torch.cuda.memory_snapshot``): what keeps ``close()`` from giving the memory back."""
+        out = []
+        for seg in torch.cuda.memory_snapshot():
+            if seg.get("device") != self.device.index:
+                continue
+            address = seg.get("address", 0)
+            for block in seg.get("blocks", []):
+                size = block.get("size", 0)
+                if str(block.get("state", "")).startswith("active"):
+                    for k in range(ARENAS):
+                        if self.sizes[k] and self.bases[k] <= address < self.bases[k] + self.sizes[k]:
+                            out.append((address, size, k))
+                address += size
+        return out
 
     # ------------------------------------------------------------------ allocation
-    def empty(self, shape: Sequence[int], dtype=torch.float32, region: Optional[int] = None,
-              away_from: Iterable[Optional[torch.Tensor]] = ()) -> torch.Tensor:
-        """An uninitialised tensor in range ``region`` (0, 1, 2: that region; ``STRIPED``); without ``region`` in
-        the striped range, or -- when there is none -- in the region that holds none (or the least) of
-        ``away_from``.  From the ordinary allocator if it is tiny or the range is full or absent."""
+    def empty(self, shape: Sequence[int], dtype=torch.float32, region: Optional[int] = None) -> torch.Tensor:
+        """An uninitialised tensor in range ``region`` (0, 1, 2: that region; ``STRIPED``, the default).  From the
+        ordinary allocator when there is no such range, when the range is full, and while a HIP graph is being
+        captured (the capture's own pool must keep what the graph uses)."""
         shape = tuple(int(s) for s in shape)
-        count = 1
-        for s in shape:
-            count *= s
-        nbytes = count * torch.empty((), dtype=dtype).element_size()
-        if nbytes >= SMALLEST_PLACED:
-            k = int(region) if region is not None else (STRIPED if self.sizes[STRIPED] else self._pick(away_from))
-            offset = self._take(k, nbytes) if self.sizes[k] else None
-            if offset is not None:
-                block = _Block(self, k, offset, nbytes, -(-nbytes // ALIGN) * ALIGN)
-                return torch.as_tensor(block, device=self.device).view(dtype).view(shape)
+        k = STRIPED if region is None else int(region)
+        if self.sizes[k] and not self._closing and not torch.cuda.is_current_stream_capturing():
+            with self.allocating(k):
+                return torch.empty(shape, dtype=dtype, device=self.device)
         return torch.empty(shape, dtype=dtype, device=self.device)
 
-    def empty_like(self, like: torch.Tensor, away_from: Optional[Iterable[Optional[torch.Tensor]]] = None) -> torch.Tensor:
-        return self.empty(like.shape, like.dtype, away_from=[like] if away_from is None else away_from)
+    def empty_like(self, like: torch.Tensor) -> torch.Tensor:
+        return self.empty(like.shape, like.dtype)
 
-    def close(self) -> None:
-        """Give the ranges' memory back to the driver -- at once if no tensor lives in them, else when the last
-        one is released; from now on requests are served by the ordinary allocator."""
-        self._anchors = None
+    def close(self) -> bool:
+        """Give the ranges' memory back to the driver.  True when that happened; False when tensors of the ranges
+        are still alive: the ranges then stay mapped (new requests go to the ordinary allocator) and a later
+        ``close()`` -- ``disable()`` and the next ``enable()`` call it -- tries again."""
+        if self._closed:
+            return True
+        if self._everything:
+            self._set_everything(False)
         with self._lock:
             self._closing = True
-            last = self._live == 0
-        if last:
-            self._destroy()
+            self._pools.clear()                            # PyTorch may now release the pools' cached segments
+        with torch.cuda.device(self.device):
+            torch.cuda.synchronize()
+            torch.cuda.empty_cache()
+            rc = self._lib.exodus_hbm_regions_destroy(self.device.index)
+        if rc == RANGE_IN_USE:
+            return False
+        self._closed = True
+        self._allocators.clear()
+        if rc != 0:
+            text = self._lib.exodus_hip_error_string(rc)
+            raise RuntimeError(f"exodus_hbm_regions_destroy: {text.decode() if isinstance(text, bytes) else text}")
+        return True
 
 
 _active: Optional[HbmRegions] = None
+_lingering: List[HbmRegions] = []         # closed while tensors were alive: still mapped, to be closed again
 
 
-def enable(gib_per_region: float = 0.0, gib_striped: float = 48.0,
-           device: Optional[torch.device] = None, **how) -> HbmRegions:
+def _close_lingering() -> bool:
+    _lingering[:] = [r for r in _lingering if not r.close()]
+    return not _lingering
+
+
+def enable(gib_per_region: float = 0.0, gib_striped: float = 48.0, device: Optional[torch.device] = None,
+           everything: bool = False, **how) -> HbmRegions:
     """Create the ranges (``HbmRegions(gib_per_region, gib_striped, device, **how)``) and make the kernels' wrappers
-    allocate their outputs through them."""
+    allocate their big outputs in the striped range.  ``everything=True`` sends every allocation on the device
+    there, from every thread (autograd's included), until ``disable()``.
+    Raises RuntimeError when ranges made earlier cannot be given back because tensors in them are still alive."""
     global _active
     if _active is not None:
         disable()
-    _active = HbmRegions(gib_per_region, gib_striped, device, **how)
-    return _active
+    if not _close_lingering():
+        blocks = [b for r in _lingering for b in r.live_blocks()]
+        raise RuntimeError(f"hbm.enable(): {len(blocks)} tensors allocated in the previous ranges are still alive "
+                           f"({sum(b[1] for b in blocks)} bytes); release them (and what refers to them, e.g. layer "
+                           "states, .grad tensors and autograd graphs) before making new ranges")
+    regions = HbmRegions(gib_per_region, gib_striped, device, **how)
+    if everything:
+        if not regions.sizes[STRIPED]:
+            regions.close()
+            raise ValueError("everything=True needs a striped range")
+        regions._set_everything(True)
+    _active = regions
+    return regions
 
 
-def disable() -> None:
-    """Undo ``enable()``.  Tensors that live in the ranges stay valid; the memory goes back with the last one."""
+def disable() -> bool:
+    """Undo ``enable()``.  Tensors that live in the ranges stay valid; the memory goes back to the driver once none
+    is left (True: it went back now; False: tensors are alive, a later ``disable()`` or ``enable()`` tries again)."""
     global _active
     if _active is not None:
-        _active.close()
+        _lingering.append(_active)
     _active = None
+    return _close_lingering()
 
 
 def active() -> Optional[HbmRegions]:
     return _active
 
 
-def empty_like(like: torch.Tensor, away_from: Optional[Iterable[Optional[torch.Tensor]]] = None) -> torch.Tensor:
-    """``torch.empty_like(like)``, or -- after ``enable()`` -- a tensor of that shape in the striped range, or
-    (region ranges only) in a region of HBM that none of ``away_from`` (default: ``like`` itself) lies in."""
-    if _active is None or like.device != _active.device:
-        return torch.empty_like(like)
-    return _active.empty_like(like, away_from)
+@contextlib.contextmanager
+def placement():
+    """``with hbm.placement():`` -- every device allocation of the calling thread inside the block comes from the
+    striped range (nothing changes when ``enable()`` was not called)."""
+    if _active is None:
+        yield
+        return
+    with _active.placement():
+        yield
 
 
-def empty(shape, like: torch.Tensor, away_from: Optional[Iterable[Optional[torch.Tensor]]] = None) -> torch.Tensor:
+def _wanted(nbytes: int, device: torch.device) -> bool:
+    return (_active is not None and nbytes >= SMALLEST_PLACED and device == _active.device
+            and bool(_active.sizes[STRIPED]))
+
+
+def empty_like(like: torch.Tensor) -> torch.Tensor:
+    """``torch.empty_like(like)`` (contiguous) -- after ``enable()``, and for 1 MiB or more, in the striped range."""
+    if not _wanted(like.numel() * like.element_size(), like.device):
+        return torch.empty_like(like, memory_format=torch.contiguous_format)
+    return _active.empty(like.shape, like.dtype)
+
+
+def empty(shape, like: torch.Tensor) -> torch.Tensor:
     """``torch.empty(shape)`` with dtype and device of ``like``, placed as ``empty_like`` places its result."""
-    if _active is None or like.device != _active.device:
-        return torch.empty(tuple(shape), dtype=like.dtype, device=like.device)
-    return _active.empty(shape, like.dtype, away_from=[like] if away_from is None else away_from)
+    shape = tuple(int(s) for s in shape)
+    count = 1
+    for s in shape:
+        count *= s
+    if not _wanted(count * like.element_size(), like.device):
+        return torch.empty(shape, dtype=like.dtype, device=like.device)
+    return _active.empty(shape, like.dtype)

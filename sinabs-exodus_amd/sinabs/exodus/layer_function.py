@@ -21,6 +21,16 @@ from ._validate import check_parameters
 from .spike import classify_surrogate
 
 
+def _one_value(grad: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
+    """The single element that ``grad`` repeats everywhere, as a one-element tensor -- or None when ``grad`` is an
+    ordinary tensor.  The gradient of ``output.sum()`` (or of a multiple of it) arrives as a scalar expanded with
+    strides of zero; the kernels take the scalar itself and read one tensor less, instead of the expansion being
+    written out to memory first."""
+    if grad is None or grad.numel() < 2 or any(grad.stride()) or grad.dtype != torch.float32:
+        return None
+    return grad.as_strided((1,), (1,))
+
+
 class SpikingLayerFunction(torch.autograd.Function):
     @staticmethod
     def forward(
@@ -106,10 +116,23 @@ class SpikingLayerFunction(torch.autograd.Function):
         need = ctx.needs_input_grad
         if all(g is None for g in (grad_spikes, grad_v_last, grad_i_last, grad_total, grad_v_rec, grad_i_rec)):
             return (None,) * 15
-        if grad_spikes is None:
-            grad_spikes = torch.zeros_like(inp)
-        if grad_total is not None:                  # d(sum of spikes) / d(spike) = 1 for every element
-            grad_spikes = grad_spikes + grad_total.to(grad_spikes.dtype)
+        # one value for every spike (a sum as the loss, the spike total behind firing_rate): handed over as it is
+        uniform = None
+        if kind != _hip.SURR_TENSOR and grad_v_rec is None and grad_i_rec is None and inp.numel() > 1:
+            if grad_spikes is None:
+                uniform = torch.zeros(1, dtype=torch.float32, device=inp.device) if grad_total is None else None
+            else:
+                uniform = _one_value(grad_spikes)
+            if grad_total is not None and (uniform is not None or grad_spikes is None):
+                total = grad_total.to(torch.float32).reshape(1)   # d(sum of spikes) / d(spike) = 1 for every element
+                uniform = total if uniform is None else uniform + total
+        if uniform is not None:
+            grad_spikes = uniform
+        else:
+            if grad_spikes is None:
+                grad_spikes = torch.zeros_like(inp)
+            if grad_total is not None:
+                grad_spikes = grad_spikes + grad_total.to(grad_spikes.dtype)
         cont = lambda x: None if x is None else x.contiguous()
         surr = None
         if v_pre is not None:
@@ -124,6 +147,7 @@ class SpikingLayerFunction(torch.autograd.Function):
             max_spikes, decay_early, norm_input, kind, p0, p1, surr=surr,
             gradVRec=cont(grad_v_rec), gradIRec=cont(grad_i_rec) if syn else None,
             wantAlphaMemGrad=need[1], wantAlphaSynGrad=need[2], wantVInitGrad=need[3], wantIInitGrad=need[4],
+            gradUniform=uniform is not None,
         )
         return (grad_input if need[0] else None, g_am, g_as, g_v0, g_i0) + (None,) * 10
 
@@ -161,11 +185,23 @@ class LeakyLayerFunction(torch.autograd.Function):
             v_mem_init = out = inp = None
         if grad_out is None and grad_v_last is None and grad_total is None:
             return (None,) * 6
+        cont = lambda x: None if x is None else x.contiguous()
+        numel = shape[0] * shape[1] * shape[2]
+        if grad_out is None:
+            uniform = torch.zeros(1, dtype=torch.float32, device=alpha.device) if grad_total is None else None
+        else:
+            uniform = _one_value(grad_out) if numel > 1 else None
+        if grad_total is not None and (uniform is not None or grad_out is None) and numel > 1:
+            total = grad_total.to(torch.float32).reshape(1)
+            uniform = total if uniform is None else uniform + total
+        if uniform is not None and numel > 1:
+            grad_input, grad_alpha, grad_init = _hip.layerLeakyBackward(
+                uniform, cont(grad_v_last), out, inp, v_mem_init, alpha, decay_early, norm_input, need_alpha, shape=shape)
+            return grad_input, grad_alpha, grad_init, None, None, None
         if grad_out is None:
             grad_out = torch.zeros(shape, dtype=torch.float32, device=alpha.device)
         if grad_total is not None:
             grad_out = grad_out + grad_total.to(grad_out.dtype)
-        cont = lambda x: None if x is None else x.contiguous()
         grad_input, grad_alpha, grad_init = _hip.layerLeakyBackward(
             cont(grad_out), cont(grad_v_last), out, inp, v_mem_init, alpha, decay_early, norm_input, need_alpha)
         return grad_input, grad_alpha, grad_init, None, None, None

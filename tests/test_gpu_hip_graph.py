@@ -121,3 +121,58 @@ def test_kernels_run_on_the_current_stream(el):
     side.synchronize()
     assert torch.equal(got, want)
     assert torch.equal(layer.v_mem, ref_layer.v_mem)
+
+
+def test_graphed_step_helper_with_placement_enabled(el):
+    """``sinabs.exodus.graph.GraphedStep`` records the step; ``hbm.enable()`` is active meanwhile.  During the
+    capture the wrappers leave allocation to the capture's own memory pool (memory of the striped range handed out
+    there would go back to its pool when the Python tensors die, and be given to the next eager request while every
+    replay still writes to it).  Between replays the program allocates and writes eagerly in the striped range;
+    every replay must still equal the eager step."""
+    import gc
+    from sinabs.exodus import hbm
+    from sinabs.exodus.graph import GraphedStep
+    torch.manual_seed(12)
+    recorded = small_network(el, 4.0); eager = small_network(el, 4.0)
+    with torch.no_grad():
+        recorded[0].weight.mul_(6.0); recorded[2].weight.mul_(4.0)
+    eager.load_state_dict(recorded.state_dict())
+    batch, steps = 64, 400                                     # the first layer's output is 9.8 MB: a placed tensor
+    inputs = [(torch.rand(batch, steps, 24, generator=gen(50 + k)) * (1.0 + 0.5 * k)).cuda() for k in range(3)]
+    weight = torch.rand(batch, steps, 10, generator=gen(49)).cuda()
+    x_static = inputs[0].clone()
+    regions = hbm.enable(gib_striped=6.0)
+    try:
+        # eagerly the layer's output is placed.  (This pass runs on the default stream and leaves its autograd graph
+        # -- and the gradient accumulators of the parameters, bound to that stream -- in the layer's states and firing
+        # rate; GraphedStep cuts those loose before it warms up on its own stream.)
+        probe = recorded[1](recorded[0](x_static))
+        assert regions.pool_of(probe) == hbm.STRIPED
+        del probe
+        graphed = GraphedStep(recorded, lambda: step(recorded, x_static, weight))
+        assert regions.pool_of(graphed.output) is None         # inside the capture: the graph's own pool
+        scribbles = []
+        for k in (1, 2, 0, 1):
+            eager.zero_grad(set_to_none=True)
+            want = step(eager, inputs[k], weight)
+            # eager work in the striped range, of the sizes the recorded step uses: memory that the recording had
+            # taken from there and given back would be handed out here, and the next replay would write into it
+            for shape in ((batch, steps, 96), (4, 1024, 1024), (batch, 13, 96)):
+                scribbles.append(hbm.empty(shape, weight).fill_(float("nan")))
+            torch.cuda.synchronize()
+            x_static.copy_(inputs[k])
+            got = graphed.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(got, want), f"spikes differ on replay with input {k}"
+            assert torch.equal(recorded[1].v_mem, eager[1].v_mem) and torch.equal(recorded[3].v_mem, eager[3].v_mem)
+            for name, p in eager.named_parameters():
+                if p.grad is not None:
+                    assert_close(dict(recorded.named_parameters())[name].grad, p.grad, f"grad {name}, input {k}",
+                                 rtol=1e-5, atol=1e-6)
+            assert want.sum().item() > 0
+            assert all(bool(torch.isnan(t).all()) for t in scribbles), "a replay wrote into memory of the striped range"
+    finally:
+        scribbles = graphed = want = got = None
+        del eager, recorded
+        gc.collect()
+        assert hbm.disable() is True

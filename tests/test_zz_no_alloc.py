@@ -118,7 +118,7 @@ def test_the_call_allocates_nothing(hip):
     def call():
         rc = hip.lib.exodus_layer_lif_backward_from_input(
             *[P(o) for o in outs], P(go), None, None, P(x), P(zero), P(zero), P(am), P(asn), P(one), P(one), None,
-            0, 2, 1, 1, hip.SURR_SINGLE_EXP, 0.5, 1.0, None, None, None, b, t, m, stream)
+            0, 2, 1, 1, hip.SURR_SINGLE_EXP, 0.5, 1.0, None, None, None, 0, b, t, m, stream)
         assert rc == 0
 
     call()
