@@ -99,6 +99,8 @@ class Placement:
                 "one-region": "all big tensors in ONE region of HBM (the control experiment)",
                 "regions": "one region of HBM per tensor: inputs in the first, outputs in the second and third"}
         out = {"placement": text[self.mode], "placement_setup_s": round(self.regions.setup_s, 3),
+               "placement_setup_seconds_taking_sorting_building_checking":
+                   self.regions.report.get("seconds_taking_sorting_building_checking"),
                "placement_sorted_by_timed_copies": bool(self.regions.sorted)}
         if self.regions.sorted:
             out["placement_verified_by_timed_copies"] = bool(self.regions.verified)
@@ -107,11 +109,12 @@ class Placement:
         return out
 
 
-def build_layer_workload(key, torch, hip, act, dev, place=None):
+def build_layer_workload(key, torch, hip, act, dev, place=None, one_value=False):
     """The same workloads on the layer's own (batch, time, neurons) layout: one kernel per direction,
     forward keeps checkpoints only, backward re-reads the input and rebuilds v_mem / i_syn.
     Algorithmic bytes per neuron-timestep: forward 8 (x in, spikes out), backward 12 (grad_spikes
-    and x in, grad_x out)."""
+    and x in, grad_x out) -- or 8 with ``one_value``: the gradient of every output element is one number (what a
+    sum as the loss hands back), passed as such."""
     w = WORKLOADS[key]
     place = place or Placement(torch, dev)
     B, T, M = w["batch"], w["steps"], w["neurons"]
@@ -120,7 +123,8 @@ def build_layer_workload(key, torch, hip, act, dev, place=None):
     rx, rgo, rs, rgi = 0, 0, 1, 1                  # tensors the kernels read: 0; tensors they write: 1
     x = place.empty((B, T, M), rx)
     x.uniform_(0.0, 0.5, generator=g) if key == "c1" else x.normal_(w["mean"], w["std"], generator=g)
-    go = place.empty((B, T, M), rgo).fill_(1.0)
+    go = torch.ones(1, device=dev) if one_value else place.empty((B, T, M), rgo).fill_(1.0)
+    bwd_bytes = 8 if one_value else 12
     rows = lambda v: torch.as_tensor(v, dtype=torch.float32, device=dev).expand(B, M).flatten().contiguous()
     zeros = torch.zeros(N, device=dev); ones = torch.ones(N, device=dev)
     surr = act.SingleExponential()
@@ -143,11 +147,12 @@ def build_layer_workload(key, torch, hip, act, dev, place=None):
             holder["out"] = hip.layerLeakyForward(x, zeros, a_mem, False, False)[0]
 
         def bwd():
-            r = hip.layerLeakyBackward(go, None, holder["out"], x, zeros, a_mem, False, False, True)
+            r = hip.layerLeakyBackward(go, None, holder["out"], x, zeros, a_mem, False, False, True,
+                                       shape=(B, T, M) if one_value else None)
             return r[1].view(B, M).sum(0)
 
         return dict(fwd=fwd, bwd=bwd, N=N, T=T, fwd_name="exodus_layer_leaky_forward",
-                    bwd_name="exodus_layer_leaky_backward", bytes=(8, 12))
+                    bwd_name="exodus_layer_leaky_backward", bytes=(8, bwd_bytes))
     syn = cfg["a_syn"] is not None
     holder = {}
 
@@ -160,11 +165,11 @@ def build_layer_workload(key, torch, hip, act, dev, place=None):
         r = holder["r"]
         out = hip.layerLifBackward(go, None, None, x, r["ckpt_v"], r["ckpt_i"], zeros, zeros if syn else None,
                                    cfg["a_mem"], cfg["a_syn"], ones, ones, cfg["lo"], cfg["lo"] is not None,
-                                   cfg["cap"], True, cfg["norm"], kind, p0, p1, gradInput=gi)
+                                   cfg["cap"], True, cfg["norm"], kind, p0, p1, gradInput=gi, gradUniform=one_value)
         return out[1].view(B, M).sum(0)
 
     return dict(fwd=fwd, bwd=bwd, N=N, T=T, fwd_name="exodus_layer_lif_forward",
-                bwd_name="exodus_layer_lif_backward", bytes=(8, 12))
+                bwd_name="exodus_layer_lif_backward", bytes=(8, bwd_bytes))
 
 
 def build_workload(key, torch, hip, act, dev, place=None):
@@ -447,7 +452,7 @@ def measure_layer_api(key, loss, torch, dev, steps, warmup, place_all=False):
         x.uniform_(0.0, 0.5, generator=g) if key == "c1" else x.normal_(w["mean"], w["std"], generator=g)
         go = torch.empty(shape, device=dev).uniform_(0.5, 1.5, generator=g) if loss == "dense" else None
     x.requires_grad_(True)
-    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps)]
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(steps)]
 
     def step(e=None):
         layer.reset_states()
@@ -458,12 +463,15 @@ def measure_layer_api(key, loss, torch, dev, steps, warmup, place_all=False):
         out = layer(x)
         if e:
             e[1].record()
+        total = out.sum() if loss == "sum" else None            # torch's own reduction over the output
+        if e:
+            e[2].record()
         if loss == "dense":
             out.backward(go)
         else:
-            out.sum().backward()
+            total.backward()
         if e:
-            e[2].record()
+            e[3].record()
 
     for _ in range(warmup):
         step()
@@ -474,18 +482,21 @@ def measure_layer_api(key, loss, torch, dev, steps, warmup, place_all=False):
     torch.cuda.synchronize()
     wall = (time.perf_counter() - t0) / steps
     fwd_ms = sum(e[0].elapsed_time(e[1]) for e in ev) / steps
-    bwd_ms = sum(e[1].elapsed_time(e[2]) for e in ev) / steps
+    loss_ms = sum(e[1].elapsed_time(e[2]) for e in ev) / steps
+    bwd_ms = sum(e[2].elapsed_time(e[3]) for e in ev) / steps
     n_t = 1
     for v in shape:
         n_t *= v
     # bytes that have to move: forward x in, output out (8); backward with a dense gradient: gradient and x in, grad_x
-    # out (12); with the sum as the loss: torch's sum reads the output (4), the backward reads x and writes grad_x (8)
+    # out (12); with the sum as the loss the gradient is one value and the backward reads x and writes grad_x (8) --
+    # torch's sum over the output (4 more, "loss_ms") is the program's loss, not the layer, and is left out of the fraction
+    layer_bytes = 20 if loss == "dense" else 16
     return {"workload": w["name"], "path": "public layer API (sinabs.exodus.layers, autograd, outputs allocated per call)",
             "layer": repr(layer).split("(")[0].strip(), "loss": "out.backward(dense gradient)" if loss == "dense" else "out.sum().backward()",
             "rows": n_t // shape[1], "time_steps": shape[1], "steps": steps, "ms_per_step": wall * 1e3,
-            "fwd_ms": fwd_ms, "bwd_ms": bwd_ms, "value": n_t / wall, "unit": "neuron-timesteps/s",
-            "algorithmic_bytes_per_neuron_timestep": 20,
-            "fwd_bwd_combined_frac": n_t * 20 / ((fwd_ms + bwd_ms) * 1e-3) / 1e9 / HBM_PEAK_GBS}
+            "fwd_ms": fwd_ms, "loss_ms": loss_ms, "bwd_ms": bwd_ms, "value": n_t / wall, "unit": "neuron-timesteps/s",
+            "algorithmic_bytes_per_neuron_timestep": layer_bytes,
+            "fwd_bwd_combined_frac": n_t * layer_bytes / ((fwd_ms + bwd_ms) * 1e-3) / 1e9 / HBM_PEAK_GBS}
 
 
 def measure_small_layer(torch, dev, steps, warmup):
@@ -727,6 +738,9 @@ def main():
                     help="run the chosen workload's layer type and options at another (batch, steps, neurons) shape, "
                          "e.g. a neuron count that does not fill 128-byte memory lines; such a run is a measurement "
                          "aid, not the benchmark (roofline.traffic is then null)")
+    ap.add_argument("--one-value-gradient", action="store_true",
+                    help="with --path layer: the gradient of every output element is one number, handed to the backward "
+                         "kernel as such (what a sum as the loss gives): it reads one tensor less (8 + 8 bytes)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--others", default="all", choices=["all", "api", "none"],
                     help="all (default): also time the other configurations and the (rows, time) kernels for a few steps "
@@ -778,7 +792,8 @@ def main():
                                         name=w_["name"] + f" -- at shape ({b_},{t_},{m_})")
 
     plain_first = None
-    special = args.region_map or args.ceilings or args.conv_snn or args.shape or args.copy_probe or args.setup_only
+    special = (args.region_map or args.ceilings or args.conv_snn or args.shape or args.copy_probe or args.setup_only
+               or args.one_value_gradient)
     full_run = args.placement == "striped" and args.others == "all" and not special
     common = ["--no-cpu-baseline", "--workload", args.workload, "--path", args.path, "--steps", str(args.steps),
               "--warmup", str(args.warmup)]
@@ -786,6 +801,9 @@ def main():
         # the same measurements with the ordinary allocator, in a process of its own and before this one touches
         # the GPU, so that it sees what a program that allocates without further thought is handed
         plain_first = child_json(["--placement", "plain", "--others", "api"] + common)
+        # ... and, next, how long ranges sorted by timed copies take to make (a later process would find the memory
+        # mixed by the 64 MiB pages of the ranges before it, and nothing to sort)
+        sorted_setup = child_json(["--placement", "sorted-striped", "--setup-only"])
 
     import torch
     assert torch.cuda.is_available(), "bench.py needs the GPU"
@@ -817,6 +835,8 @@ def main():
             print("[bench] " + placement_note, file=sys.stderr, flush=True)
     if args.setup_only:
         out = dict(place.describe())
+        if placement_note:
+            out["placement_note"] = placement_note
         if place.regions is not None:
             out["gave_memory_back"] = hbm.disable()
         print(json.dumps(out))
@@ -827,8 +847,12 @@ def main():
     if args.conv_snn:
         print(json.dumps(dict(measure_conv_snn(args, torch, dev), **place.describe())))
         return
-    build = build_layer_workload if args.path == "layer" else build_workload
-    wl = build(args.workload, torch, hip, act, dev, place)
+    if args.one_value_gradient and args.path != "layer":
+        sys.exit("bench.py: --one-value-gradient goes with --path layer")
+    if args.path == "layer":
+        wl = build_layer_workload(args.workload, torch, hip, act, dev, place, one_value=args.one_value_gradient)
+    else:
+        wl = build_workload(args.workload, torch, hip, act, dev, place)
     fwd, bwd, N, T = wl["fwd"], wl["bwd"], wl["N"], wl["T"]
 
     if args.copy_probe:
@@ -841,7 +865,7 @@ def main():
     m = measure(wl, args.steps, args.warmup, torch)
     ms_step, fwd_ms, bwd_ms = m["ms_per_step"], m["fwd_ms"], m["bwd_ms"]
     bf, bb = wl.get("bytes", WORKLOADS[args.workload]["bytes"])
-    roof = roofline(args.workload, wl, fwd_ms, bwd_ms, bf, bb, traffic_known=not args.shape)
+    roof = roofline(args.workload, wl, fwd_ms, bwd_ms, bf, bb, traffic_known=not (args.shape or args.one_value_gradient))
     # the same durations priced with the bytes of a kernel pair that stores and re-reads the states (the
     # figure the workload description quotes); "frac" uses what this design has to move, which is less
     # because the backward pass recomputes the states
@@ -899,6 +923,16 @@ def main():
                 "algorithmic_bytes_per_neuron_timestep": obf + obb,
                 "roofline": roofline(key, other, mo["fwd_ms"], mo["bwd_ms"], obf, obb)})
             del other
+        # the headline workload with one number as the gradient of every spike (a sum as the loss)
+        other = build_layer_workload(args.workload, torch, hip, act, dev, place, one_value=True)
+        mo = measure(other, max(3, args.steps // 2), max(2, args.warmup // 2), torch)
+        result["others"].append({
+            "workload": WORKLOADS[args.workload]["name"] + " -- one value as the gradient of every output element",
+            "path": "layer", "rows": other["N"], "time_steps": other["T"], "steps": mo["steps"],
+            "ms_per_step": mo["ms_per_step"], "value": other["N"] * other["T"] / (mo["ms_per_step"] * 1e-3),
+            "unit": "neuron-timesteps/s", "algorithmic_bytes_per_neuron_timestep": sum(other["bytes"]),
+            "roofline": roofline(args.workload, other, mo["fwd_ms"], mo["bwd_ms"], *other["bytes"], traffic_known=False)})
+        del other
     if args.others in ("all", "api") and not args.shape:
         # every configuration through the public layer API, with the ordinary allocator's figures (from the child
         # run) beside those of this process's placement
@@ -911,7 +945,7 @@ def main():
             e.pop("placement_measured", None)
             twin = plain_api.get((e["workload"], e["loss"]))
             if twin:
-                e["ordinary_allocator"] = {k: twin[k] for k in ("ms_per_step", "fwd_ms", "bwd_ms", "value",
+                e["ordinary_allocator"] = {k: twin[k] for k in ("ms_per_step", "fwd_ms", "loss_ms", "bwd_ms", "value",
                                                                  "fwd_bwd_combined_frac")}
             result["others"].append(e)
     if args.others == "all" and not args.shape:
@@ -937,8 +971,8 @@ def main():
             {"frac": ar["frac"], "fwd_bwd_combined_frac": ar["fwd_bwd_combined_frac"], "kernel_ms": ar["kernel_ms"],
              "other_kernel_ms": ar["other_kernel"]["kernel_ms"]} if ar else allst)
         result["placement_setup"] = {
-            "hbm.enable() (default: sort=False)": {"setup_s": result["config"].get("placement_setup_s")},
-            "hbm.enable(sort=True)": child_json(["--placement", "sorted-striped", "--setup-only"])}
+            "hbm.enable() (default: sort=False)": {k: v for k, v in result["config"].items() if k.startswith("placement_setup")},
+            "hbm.enable(sort=True)": sorted_setup}
     print(json.dumps(result))
 
 

@@ -50,6 +50,9 @@ namespace {
 #ifndef EXODUS_LAYER_BWD_WAVES
 #define EXODUS_LAYER_BWD_WAVES 3      // resident waves per SIMD the backward kernel is compiled for
 #endif
+#ifndef EXODUS_LAYER_BWD_WAVES_G1
+#define EXODUS_LAYER_BWD_WAVES_G1 4   // ... and its instances that stream one tensor less (one gradient value for all)
+#endif
 constexpr int CKPT = EXODUS_LAYER_CKPT;               // steps between checkpoints = length of a backward chunk
 constexpr int FWD_UNROLL = EXODUS_LAYER_FWD_UNROLL;  // forward steps per software-pipeline stage (divides CKPT)
 constexpr int BLOCK = EXODUS_LAYER_BLOCK;
@@ -160,6 +163,7 @@ struct Neuron {
     float k;            // factor on the current entering the membrane: 1 - alpha_mem (norm_input) or 1
     float xs;           // factor on the input entering the synapse: alpha_syn (decay_early) or 1
     float c, th;        // subtract value, threshold
+    float c2;           // 2 * subtract value (exact), what two spikes take away
     float th2;          // 2 * threshold: from here on a second spike (+inf where th <= 0)
     float thd;          // from here on the spike count needs the quotient v / th (+inf if never)
     float lo;           // lower bound of the potential, -inf without one
@@ -181,6 +185,7 @@ __device__ __forceinline__ void neuron_load(Neuron &n, const LayerConsts &p, int
     n.k = p.norm_input ? __fsub_rn(1.0f, n.am) : 1.0f;
     n.xs = (SYN && p.decay_early) ? n.as : 1.0f;
     n.c = p.c[row];
+    n.c2 = __fadd_rn(n.c, n.c);
     n.th = p.theta[row];
     // For th > 0:  v >= th <=> RN(v/th) >= 1  and  v >= 2 th <=> RN(v/th) >= 2  (2 th is exact and no
     // float lies between its predecessor and the rounding boundary of the quotient), so counts up to
@@ -234,6 +239,19 @@ __device__ __forceinline__ float spike_count_fast(float v, const Neuron &n, cons
     float count = count_by_compare<CAPK>(v, n, cc);
     if (v >= n.thd) count = count_by_quotient(v, n, cc);
     return count;
+}
+
+// count * c, what the reset subtracts from the potential, for callers that do not need the count itself: with a cap
+// of one or two spikes the product is 0, c or 2c (all exact), picked by the comparisons that would have picked the
+// count -- the same bits as the multiplication, one instruction less.
+template <int CAPK>
+__device__ __forceinline__ float reset_amount(float v, const Neuron &n, const Cap &cc)
+{
+    if (CAPK == 0) return __fmul_rn(spike_count_fast<0>(v, n, cc), n.c);
+    float taken = v >= n.th ? n.c : 0.f;
+    if (CAPK == 2) taken = v >= n.th2 ? n.c2 : taken;
+    if (v >= n.thd) taken = __fmul_rn(count_by_quotient(v, n, cc), n.c);   // thresholds that are not positive
+    return taken;
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -431,8 +449,9 @@ __global__ void __launch_bounds__(BLOCK) layer_lif_forward(
 // kernel streams one tensor less (8 instead of 12 bytes per neuron-timestep).
 template <bool SYN, int KIND, int CAPK, bool NT, bool EXTRA, bool GO1 = false>
 __global__ void __launch_bounds__(BWD_BLOCK)
-    __attribute__((amdgpu_waves_per_eu((KIND == EXODUS_SURR_TENSOR || EXTRA) ? 2 : EXODUS_LAYER_BWD_WAVES,
-                                       (KIND == EXODUS_SURR_TENSOR || EXTRA) ? 2 : EXODUS_LAYER_BWD_WAVES)))
+    __attribute__((amdgpu_waves_per_eu(
+        (KIND == EXODUS_SURR_TENSOR || EXTRA) ? 2 : (GO1 ? EXODUS_LAYER_BWD_WAVES_G1 : EXODUS_LAYER_BWD_WAVES),
+        (KIND == EXODUS_SURR_TENSOR || EXTRA) ? 2 : (GO1 ? EXODUS_LAYER_BWD_WAVES_G1 : EXODUS_LAYER_BWD_WAVES))))
 layer_lif_backward(
     float *__restrict__ grad_x, float *__restrict__ alpha_mem_grad, float *__restrict__ alpha_syn_grad,
     float *__restrict__ v_init_grad, float *__restrict__ i_init_grad, const float *__restrict__ grad_spikes,
@@ -493,7 +512,7 @@ layer_lif_backward(
         constexpr bool GUARD = decltype(guard)::value;
         const int64_t t0 = j * CKPT;
         const int len = GUARD ? static_cast<int>(T - t0) : CKPT;
-        float xr[CKPT], gr[CKPT], vr[CKPT], sr[FROM_TENSOR ? CKPT : 1];
+        float xr[CKPT], gr[GO1 ? 1 : CKPT], vr[CKPT], sr[FROM_TENSOR ? CKPT : 1];   // (GO1: results go where the inputs were)
         float qv[EXTRA ? CKPT : 1], qi[(EXTRA && SYN) ? CKPT : 1];
         __syncthreads();                                   // keeps the block's waves at the same step
         if (!active) return;
@@ -509,7 +528,7 @@ layer_lif_backward(
             for (int k = 0; k < CKPT; ++k) {
                 const unsigned so = (GUARD ? (k < last ? k : last) : k) * step_bytes;
                 xr[k] = IO::load(rx, voff, so);
-                if (!GO1) gr[k] = IO::load(rg, voff, so);
+                if (!GO1) gr[GO1 ? 0 : k] = IO::load(rg, voff, so);
                 if (FROM_TENSOR) sr[k] = IO::load(rs, voff, so);
                 if (EXTRA) qv[k] = IO::load(rqv, voff, so);
                 if (EXTRA && SYN) qi[k] = IO::load(rqi, voff, so);
@@ -524,7 +543,7 @@ layer_lif_backward(
         for (int k = 0; k < CKPT; ++k)
             if (!GUARD || k < len) {
                 const float v = neuron_advance<SYN>(nr, xr[k]);
-                nr.vpost = __fsub_rn(v, __fmul_rn(spike_count_fast<CAPK>(v, nr, cc), nr.c));
+                nr.vpost = __fsub_rn(v, reset_amount<CAPK>(v, nr, cc));
                 vr[k] = v;
                 xr[k] = nr.i;
             }
@@ -536,12 +555,12 @@ layer_lif_backward(
             if (!GUARD || k < len) {
                 const float v = vr[k], cur_i = xr[k];
                 const float sg = FROM_TENSOR ? sr[FROM_TENSOR ? k : 0] : surrogate<KIND>(v, nr.th, inv_p0, sk);
-                const float vpost = __fsub_rn(v, __fmul_rn(nr.c, spike_count_fast<CAPK>(v, nr, cc)));
+                const float vpost = __fsub_rn(v, reset_amount<CAPK>(v, nr, cc));
                 acc_m.add(lam, vpost);                          // lambda_{t+1} * vpost_t
                 const float through = __fsub_rn(1.0f, __fmul_rn(nr.c, sg));   // d vpost_t / d v_t
                 // a gradient on the recorded vpost_t joins what the next step sends down to vpost_t
                 const float below = EXTRA ? __fadd_rn(h, qv[EXTRA ? k : 0]) : h;
-                const float l = __fadd_rn(__fmul_rn(sg, GO1 ? g1 : gr[k]), __fmul_rn(through, below));
+                const float l = __fadd_rn(__fmul_rn(sg, GO1 ? g1 : gr[GO1 ? 0 : k]), __fmul_rn(through, below));
                 lam = v > nr.lo ? l : 0.f;                      // clamped (or NaN) steps pass nothing on
                 h = __fmul_rn(nr.am, lam);
                 acc_n.add(lam, cur_i);                          // lambda_t * i_t
@@ -552,9 +571,9 @@ layer_lif_backward(
                     if (EXTRA) mu = __fadd_rn(mu, qi[(EXTRA && SYN) ? k : 0]);
                     hm = __fmul_rn(nr.as, mu);
                     acc_s.add(pair_new ? mu : mu_next, cur_i);
-                    gr[k] = __fmul_rn(mu, xg);
+                    (GO1 ? xr[k] : gr[GO1 ? 0 : k]) = __fmul_rn(mu, xg);
                 } else {
-                    gr[k] = du;
+                    (GO1 ? xr[k] : gr[GO1 ? 0 : k]) = du;
                 }
             }
         }
@@ -562,7 +581,7 @@ layer_lif_backward(
             const Rsrc ro = make_rsrc(op + t0 * M);
 #pragma unroll
             for (int k = 0; k < CKPT; ++k)
-                if (!GUARD || k < len) IO::store(gr[k], ro, voff, k * step_bytes);
+                if (!GUARD || k < len) IO::store(GO1 ? xr[k] : gr[GO1 ? 0 : k], ro, voff, k * step_bytes);
         }
         acc_m.fold();
         acc_n.fold();

@@ -32,10 +32,11 @@ class StatefulLayer(nn.Module):
         return super().zero_grad(set_to_none)
 
     def is_state_initialised(self) -> bool:
-        return all(buf.shape != torch.Size([0]) for buf in self.buffers())
+        return all(buf.shape != torch.Size([0]) for buf in self._buffers.values())
 
     def state_has_shape(self, shape) -> bool:
-        return all(buf.shape == torch.Size(shape) for buf in self.buffers())
+        shape = torch.Size(shape)
+        return all(buf.shape == shape for buf in self._buffers.values())
 
     def init_state_with_shape(self, shape, randomize: bool = False) -> None:
         for name, buf in self.named_buffers():
@@ -45,7 +46,7 @@ class StatefulLayer(nn.Module):
     def reset_states(self, randomize: bool = False, value_ranges: Optional[dict] = None) -> None:
         if not self.is_state_initialised():
             return
-        for name, buf in self.named_buffers():
+        for name, buf in self._buffers.items():
             buf.detach_()
             if randomize:
                 lo, hi = (value_ranges or {}).get(name, (0.0, 1.0))

@@ -120,11 +120,28 @@ def _mat(x: torch.Tensor, name: str, n: int, t: int) -> torch.Tensor:
 
 
 def _ptr(x: Optional[torch.Tensor]):
-    return None if x is None else ctypes.c_void_p(x.data_ptr())
+    return None if x is None else x.data_ptr()             # ctypes takes a plain integer for a void pointer
 
 
 def _stream(x: torch.Tensor):
-    return ctypes.c_void_p(torch.cuda.current_stream(x.device).cuda_stream)
+    return torch.cuda.current_stream(x.device).cuda_stream or None
+
+
+class _NoGuard:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_GUARD = _NoGuard()
+
+
+def _on_device_of(device: torch.device):
+    """Device guard for a launch: ``device`` becomes current for the call -- which it nearly always is already, and
+    then nothing needs switching."""
+    return _NO_GUARD if torch.cuda.current_device() == device.index else torch.cuda.device(device)
 
 
 # ------------------------------------------------------------------------------------------
@@ -147,7 +164,7 @@ def lifForward(outputSpikes, vmem, input, vmemPostInitial, alpha, membrSubtract,
         _rows(_dev(thetaLow, "thetaLow", input), "thetaLow", n)
     else:
         thetaLow = None
-    with torch.cuda.device(input.device):
+    with _on_device_of(input.device):
         _check(lib.exodus_lif_forward(_ptr(outputSpikes), _ptr(vmem), _ptr(input), _ptr(vmemPostInitial),
                                       _ptr(alpha), _ptr(membrSubtract), _ptr(theta), _ptr(thetaLow),
                                       int(bool(applyThetaLow)), int(maxNumSpikes), n, t, _stream(input)),
@@ -165,7 +182,7 @@ def lifBackward(surr, outputGrad, notClipped, alpha, membrSubtract) -> torch.Ten
     _rows(_dev(alpha, "alpha", surr), "alpha", n)
     _rows(_dev(membrSubtract, "membrSubtract", surr), "membrSubtract", n)
     inputGrad = hbm.empty_like(surr)
-    with torch.cuda.device(surr.device):
+    with _on_device_of(surr.device):
         _check(lib.exodus_lif_backward(_ptr(inputGrad), _ptr(surr), _ptr(outputGrad), _ptr(notClipped),
                                        _ptr(alpha), _ptr(membrSubtract), n, t, _stream(surr)),
                "exodus_lif_backward")
@@ -184,7 +201,7 @@ def lifBackwardAlpha(surr, outputGrad, vmemPost, vmemPostInitial, notClipped, al
     for nm, x in (("vmemPostInitial", vmemPostInitial), ("alpha", alpha), ("membrSubtract", membrSubtract)):
         _rows(_dev(x, nm, surr), nm, n)
     alphaGrad = torch.zeros_like(alpha)
-    with torch.cuda.device(surr.device):
+    with _on_device_of(surr.device):
         _check(lib.exodus_lif_backward_alpha(_ptr(alphaGrad), _ptr(surr), _ptr(outputGrad), _ptr(vmemPost),
                                              _ptr(vmemPostInitial), _ptr(notClipped), _ptr(alpha),
                                              _ptr(membrSubtract), int(bool(gateInitial)), n, t, _stream(surr)),
@@ -201,7 +218,7 @@ def leakyForward(input, vmemInitial, alpha, *, output=None) -> torch.Tensor:
     _rows(_dev(vmemInitial, "vmemInitial", input), "vmemInitial", n)
     _rows(_dev(alpha, "alpha", input), "alpha", n)
     out = hbm.empty_like(input) if output is None else _mat(_dev(output, "output", input), "output", n, t)
-    with torch.cuda.device(input.device):
+    with _on_device_of(input.device):
         _check(lib.exodus_leaky_forward(_ptr(out), _ptr(input), _ptr(vmemInitial), _ptr(alpha), n, t,
                                         _stream(input)), "exodus_leaky_forward")
     return out
@@ -215,7 +232,7 @@ def leakyBackward(outputGrad, alpha) -> torch.Tensor:
     n, t = outputGrad.shape
     _rows(_dev(alpha, "alpha", outputGrad), "alpha", n)
     inputGrad = hbm.empty_like(outputGrad)
-    with torch.cuda.device(outputGrad.device):
+    with _on_device_of(outputGrad.device):
         _check(lib.exodus_leaky_backward(_ptr(inputGrad), _ptr(outputGrad), _ptr(alpha), n, t,
                                          _stream(outputGrad)), "exodus_leaky_backward")
     return inputGrad
@@ -231,7 +248,7 @@ def leakyBackwardAlpha(outputGrad, output, vmemInitial, alpha) -> torch.Tensor:
     _rows(_dev(vmemInitial, "vmemInitial", outputGrad), "vmemInitial", n)
     _rows(_dev(alpha, "alpha", outputGrad), "alpha", n)
     alphaGrad = torch.zeros_like(alpha)
-    with torch.cuda.device(outputGrad.device):
+    with _on_device_of(outputGrad.device):
         _check(lib.exodus_leaky_backward_alpha(_ptr(alphaGrad), _ptr(outputGrad), _ptr(output),
                                                _ptr(vmemInitial), _ptr(alpha), n, t, _stream(outputGrad)),
                "exodus_leaky_backward_alpha")
@@ -247,7 +264,7 @@ def spikeForward(vmem, alpha: float, membrSubtract: float, theta: float, thetaLo
         raise RuntimeError("vmem must be 2-D (rows, time)")
     n, t = vmem.shape
     spikes = hbm.empty_like(vmem)
-    with torch.cuda.device(vmem.device):
+    with _on_device_of(vmem.device):
         _check(lib.exodus_spike_forward(_ptr(spikes), _ptr(vmem), float(alpha), float(membrSubtract), float(theta),
                                         float(thetaLow), int(bool(applyThetaLow)), int(maxNumSpikes), n, t,
                                         _stream(vmem)), "exodus_spike_forward")
@@ -263,7 +280,7 @@ def spikeBackward(surr, outputGrad, notClipped, alpha: float, membrSubtract: flo
     _mat(_dev(outputGrad, "outputGrad", surr), "outputGrad", n, t)
     _mat(_dev(notClipped, "notClipped", surr), "notClipped", n, t)
     inputGrad = hbm.empty_like(surr)
-    with torch.cuda.device(surr.device):
+    with _on_device_of(surr.device):
         _check(lib.exodus_spike_backward(_ptr(inputGrad), _ptr(surr), _ptr(outputGrad), _ptr(notClipped),
                                          float(alpha), float(membrSubtract), n, t, _stream(surr)),
                "exodus_spike_backward")
@@ -291,7 +308,7 @@ def leakyBackwardFused(outputGrad, alpha, output=None, vmemInitial=None, needAlp
         _mat(_dev(inputGrad, "inputGrad", outputGrad), "inputGrad", n, t)
     initGrad = torch.zeros_like(alpha)
     alphaGrad = torch.zeros_like(alpha) if needAlphaGrad else None
-    with torch.cuda.device(outputGrad.device):
+    with _on_device_of(outputGrad.device):
         _check(lib.exodus_leaky_backward_fused(_ptr(inputGrad), _ptr(alphaGrad), _ptr(initGrad), _ptr(outputGrad),
                                                _ptr(output) if needAlphaGrad else None,
                                                _ptr(vmemInitial) if needAlphaGrad else None, _ptr(alpha), n, t,
@@ -332,7 +349,7 @@ def lifBackwardFused(gradSpikes, gradVmem, vmem, vmemPostInitial, alpha, membrSu
         _mat(_dev(inputGrad, "inputGrad", vmem), "inputGrad", n, t)
     initGrad = torch.zeros_like(alpha)
     alphaGrad = torch.zeros_like(alpha) if needAlphaGrad else None
-    with torch.cuda.device(vmem.device):
+    with _on_device_of(vmem.device):
         _check(lib.exodus_lif_backward_fused(_ptr(inputGrad), _ptr(alphaGrad), _ptr(initGrad), _ptr(gradSpikes),
                                              _ptr(gradVmem), _ptr(vmem), _ptr(surr),
                                              _ptr(vmemPostInitial) if needAlphaGrad else None, _ptr(alpha),
@@ -363,7 +380,7 @@ def synLifForward(input, vmemPostInitial, isynInitial, alphaMem, alphaSyn, membr
     spikes, vmem, isyn = out
     for nm, x in (("spikes", spikes), ("vmem", vmem), ("isyn", isyn)):
         _mat(_dev(x, nm, input), nm, n, t)
-    with torch.cuda.device(input.device):
+    with _on_device_of(input.device):
         _check(lib.exodus_synlif_forward(_ptr(spikes), _ptr(vmem), _ptr(isyn), _ptr(input), _ptr(vmemPostInitial),
                                          _ptr(isynInitial), _ptr(alphaMem), _ptr(alphaSyn), _ptr(membrSubtract),
                                          _ptr(theta), _ptr(thetaLow), int(bool(applyThetaLow)), int(maxNumSpikes),
@@ -400,7 +417,7 @@ def synLifBackward(gradSpikes, gradVmem, gradIsyn, vmem, isyn, vmemPostInitial, 
     else:
         _mat(_dev(inputGrad, "inputGrad", vmem), "inputGrad", n, t)
     per_row = [torch.zeros_like(alphaMem) for _ in range(4)]
-    with torch.cuda.device(vmem.device):
+    with _on_device_of(vmem.device):
         _check(lib.exodus_synlif_backward(_ptr(inputGrad), *[_ptr(x) for x in per_row], _ptr(gradSpikes),
                                           _ptr(gradVmem), _ptr(gradIsyn), _ptr(vmem), _ptr(isyn),
                                           _ptr(vmemPostInitial), _ptr(isynInitial), _ptr(alphaMem), _ptr(alphaSyn),
@@ -419,8 +436,11 @@ def synLifBackward(gradSpikes, gradVmem, gradIsyn, vmem, isyn, vmemPostInitial, 
 LAYER_MAX_NEURONS = 1 << 25
 
 
+_CHECKPOINT_INTERVAL = int(lib.exodus_layer_checkpoint_interval())
+
+
 def checkpointInterval() -> int:
-    return int(lib.exodus_layer_checkpoint_interval())
+    return _CHECKPOINT_INTERVAL
 
 
 def _btm(x: torch.Tensor, name: str, like: Optional[torch.Tensor] = None):
@@ -476,7 +496,7 @@ def layerLifForward(input, vmemPostInitial, isynInitial, alphaMem, alphaSyn, mem
         res["v_last"].copy_(vmemPostInitial.reshape(state_shape))
         if syn:
             res["i_last"].copy_(isynInitial.reshape(state_shape))
-    with torch.cuda.device(input.device):
+    with _on_device_of(input.device):
         _check(lib.exodus_layer_lif_forward(
             _ptr(spikes), _ptr(res["v_rec"]), _ptr(res["i_rec"]), _ptr(res["ckpt_v"]), _ptr(res["ckpt_i"]),
             _ptr(res["v_last"]), _ptr(res["i_last"]), _ptr(res["spike_sum"]), _ptr(input), _ptr(vmemPostInitial),
@@ -576,7 +596,7 @@ def layerLifBackward(gradSpikes, gradVLast, gradILast, input, ckptV, ckptI, vmem
             _ptr(membrSubtract), _ptr(theta), _ptr(thetaLow), int(bool(applyThetaLow)), int(maxNumSpikes),
             int(bool(decayEarly)), int(bool(normInput)), int(surrogateKind), float(surrP0), float(surrP1), _ptr(surr),
             _ptr(gradVRec), _ptr(gradIRec), int(bool(gradUniform)), b, t, m, _stream(input))
-    with torch.cuda.device(input.device):
+    with _on_device_of(input.device):
         if from_input:
             _check(lib.exodus_layer_lif_backward_from_input(*head, *tail), "exodus_layer_lif_backward_from_input")
         else:
@@ -602,7 +622,7 @@ def layerLeakyForward(input, vmemInitial, alpha, decayEarly: bool, normInput: bo
     out_sum = torch.zeros((), dtype=torch.float64, device=input.device) if wantSum else None
     if t == 0:
         v_last.copy_(vmemInitial.reshape(state_shape))
-    with torch.cuda.device(input.device):
+    with _on_device_of(input.device):
         _check(lib.exodus_layer_leaky_forward(_ptr(out), _ptr(v_last), _ptr(out_sum), _ptr(input), _ptr(vmemInitial),
                                               _ptr(alpha), int(bool(decayEarly)), int(bool(normInput)), b, t, m,
                                               _stream(input)), "exodus_layer_leaky_forward")
@@ -638,7 +658,7 @@ def layerLeakyBackward(gradOut, gradVLast, out, input, vmemInitial, alpha, decay
     alpha_grad = block[1] if needAlphaGrad else None
     if t == 0 and gradVLast is not None:
         v_init_grad.copy_(gradVLast.reshape(-1))
-    with torch.cuda.device(gradOut.device):
+    with _on_device_of(gradOut.device):
         _check(lib.exodus_layer_leaky_backward(
             _ptr(grad_input), _ptr(alpha_grad), _ptr(v_init_grad), _ptr(gradOut), _ptr(gradVLast),
             _ptr(out) if needAlphaGrad else None, _ptr(input) if need_x else None,

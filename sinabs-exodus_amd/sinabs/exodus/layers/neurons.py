@@ -275,8 +275,29 @@ class LIF(LIFBase):
     def _needs_grad(self, input_data: torch.Tensor) -> bool:
         if not torch.is_grad_enabled():
             return False
-        return (input_data.requires_grad or any(p.requires_grad for p in self.parameters())
-                or any(b.requires_grad for b in self.buffers()))
+        return (input_data.requires_grad or any(p is not None and p.requires_grad for p in self._parameters.values())
+                or any(b is not None and b.requires_grad for b in self._buffers.values()))
+
+    # ``firing_rate`` (spikes per neuron and step of the last call, reference lif.py:305) is worked out when somebody
+    # asks for it: the kernels hand back the spike total, and dividing it costs two more kernel launches that a
+    # training loop which never looks at the rate need not pay.  It stays differentiable (the total is an output of the
+    # autograd Function).  Assigning to the attribute works as before.
+    @property
+    def firing_rate(self):
+        parts = self.__dict__.get("_firing_rate_parts")
+        if parts is not None:
+            total, count = parts
+            self.__dict__["_firing_rate_value"] = (total / max(count, 1)).float()
+            self.__dict__["_firing_rate_parts"] = None
+        return self.__dict__.get("_firing_rate_value")
+
+    @firing_rate.setter
+    def firing_rate(self, value):
+        self.__dict__["_firing_rate_value"] = value
+        self.__dict__["_firing_rate_parts"] = None
+
+    def _firing_rate_from(self, total: torch.Tensor, count: int) -> None:
+        self.__dict__["_firing_rate_parts"] = (total, count)
 
     def _forward_native_leaky(self, input_data: torch.Tensor) -> torch.Tensor:
         batch_size, time_steps, *trailing_dim = input_data.shape
@@ -296,7 +317,7 @@ class LIF(LIFBase):
         out = out.reshape(input_data.shape)
         self.recordings = {"v_mem": out} if self.record_states else dict()
         self._set_state("v_mem", v_last)
-        self.firing_rate = (total / max(out.numel(), 1)).float()
+        self._firing_rate_from(total, out.numel())
         return out
 
     def _forward_native(self, input_data: torch.Tensor) -> torch.Tensor:
@@ -343,7 +364,7 @@ class LIF(LIFBase):
             self._set_state("v_mem", res["v_last"])
             if has_syn:
                 self._set_state("i_syn", res["i_last"])
-            self.firing_rate = (res["spike_sum"] / max(flat_input.numel(), 1)).float()
+            self._firing_rate_from(res["spike_sum"], flat_input.numel())
             return res["spikes"].reshape(input_data.shape)
         spikes, v_last, i_last, spike_total, v_rec, i_rec = SpikingLayerFunction.apply(
             flat_input,
@@ -372,7 +393,7 @@ class LIF(LIFBase):
         self._set_state("v_mem", v_last)
         if has_syn:
             self._set_state("i_syn", i_last)
-        self.firing_rate = (spike_total / max(spikes.numel(), 1)).float()
+        self._firing_rate_from(spike_total, spikes.numel())
         return spikes.reshape(input_data.shape)
 
     def forward(self, input_data: torch.Tensor) -> torch.Tensor:
