@@ -741,6 +741,9 @@ def main():
     ap.add_argument("--one-value-gradient", action="store_true",
                     help="with --path layer: the gradient of every output element is one number, handed to the backward "
                          "kernel as such (what a sum as the loss gives): it reads one tensor less (8 + 8 bytes)")
+    ap.add_argument("--one-lane-per-neuron", action="store_true",
+                    help="keep the backward kernel that walks a neuron's whole sequence in one lane also for layers with few "
+                         "neurons (by default those run the kernel that gives every 32 steps a lane of its own)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--others", default="all", choices=["all", "api", "none"],
                     help="all (default): also time the other configurations and the (rows, time) kernels for a few steps "
@@ -809,6 +812,8 @@ def main():
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.one_lane_per_neuron:
+        hip.backwardTimeSplit(0)
     if args.region_map:
         measure_region_map(args, torch, dev)
         return

@@ -223,6 +223,16 @@ int exodus_layer_lif_backward(float *grad_input, float *alpha_mem_grad, float *a
                               const float *grad_v_rec, const float *grad_i_rec, int grad_spikes_uniform,
                               int64_t batch, int64_t t, int64_t neurons, void *stream);
 
+/* How exodus_layer_lif_backward spreads a layer over the machine.  Its ordinary kernel gives every neuron one lane that
+ * walks the whole sequence, which leaves most of the GPU idle when a layer has few neurons (the reference's kernels
+ * have the same shape: one thread per row, reference cuda/lif_kernels.h:296-311).  For layers without synapse, with an
+ * in-kernel surrogate (kind 1..3), without grad_v_rec and with 33 to 512 steps a second kernel gives every chunk of 32
+ * steps of every neuron a lane of its own (the adjoint recurrence is affine, so the chunks can be composed afterwards):
+ * the same gradients to fp32 rounding, not bit for bit.  mode 0: never use it; 1 (default): for layers of up to 16 384
+ * neurons (batch * neurons); 2: whenever it applies; any other value changes nothing.  Returns the mode that was set
+ * before.  Process-wide. */
+int exodus_layer_backward_time_split(int mode);
+
 /* exodus_layer_lif_backward for callers that cannot allocate device memory -- code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the
  * reference.  Same arguments, outputs and arithmetic as exodus_layer_lif_backward, except that no

@@ -911,6 +911,174 @@ inline bool bad3(int64_t b, int64_t t, int64_t m)
     return (b * t) > INT64_MAX / m;
 }
 
+// ---------------------------------------------------------------------------------------------
+// backward, split over time (layers with few neurons and many steps)
+// ---------------------------------------------------------------------------------------------
+// The kernel above gives every neuron one lane, which walks the whole sequence: a layer of a few thousand neurons
+// fills a fraction of the machine, and its run time is the length of one lane's chain, 2 T steps.  Two facts allow
+// cutting the chain into pieces: the chunks of CKPT steps can be rebuilt independently from their checkpoints, and
+// the adjoint recurrence is affine once the forward values are known,
+//     lambda_t = nc_t (s_t g_t + (1 - c s_t) h_{t+1}),   h_t = a_mem lambda_t,   h_T = gradient on the final potential,
+// so a chunk maps the h that enters it (from later steps) to the h that leaves it as h_out = A + B h_in, and every
+// lambda_t inside the chunk is P_t + Q_t h_in.  Here a lane owns one chunk of one neuron (threadIdx.x = neuron,
+// threadIdx.y = chunk): it rebuilds the chunk, walks it in reverse ONCE carrying (P, Q), the chunks of a neuron
+// exchange (A, B) through LDS, every lane folds the maps of the chunks after its own into its h_in, and turns its
+// (P_t, Q_t) into gradients.  The chain is then 2 CKPT steps plus the fold over at most SPLIT_MAX_CHUNKS entries,
+// whatever T is.  Layers without synapse, with an in-kernel surrogate and without gradients on state records (the
+// spiking layers of the small configurations); everything else, and every layer large enough to fill the machine,
+// takes the kernel above.  Sums associate differently than in the sequential walk: results agree with it to fp32
+// rounding, not bit for bit.
+constexpr int SPLIT_MAX_CHUNKS = 16;       // chunks per neuron (= threadIdx.y range): sequences of up to 512 steps
+constexpr int SPLIT_NEURONS = 64;          // neurons per block: one wave per chunk
+
+template <int KIND, int CAPK, bool GO1>
+__global__ void __launch_bounds__(SPLIT_NEURONS *SPLIT_MAX_CHUNKS) layer_lif_backward_split(
+    float *__restrict__ grad_x, float *__restrict__ alpha_mem_grad, float *__restrict__ v_init_grad,
+    const float *__restrict__ grad_spikes, const float *__restrict__ grad_v_last, const float *__restrict__ x,
+    const float *__restrict__ ckpt_v, const LayerConsts p, const float p0, const float p1, const float inv_p0,
+    const int64_t blocks_per_batch, const int64_t T, const int64_t M)
+{
+    __shared__ float map_a[SPLIT_MAX_CHUNKS][SPLIT_NEURONS], map_b[SPLIT_MAX_CHUNKS][SPLIT_NEURONS];
+    __shared__ float first_lambda[SPLIT_MAX_CHUNKS + 1][SPLIT_NEURONS];
+    __shared__ double partial[SPLIT_MAX_CHUNKS][SPLIT_NEURONS];
+    const int64_t b = blockIdx.x / blocks_per_batch;
+    const int64_t m0 = static_cast<int64_t>(blockIdx.x - b * blocks_per_batch) * SPLIT_NEURONS;
+    const int lane = threadIdx.x, j = threadIdx.y;
+    const int n_ck = blockDim.y;                                 // = ceil(T / CKPT), the host sees to that
+    const bool active = m0 + lane < M;
+    const int64_t row = b * M + m0 + lane;
+    const int64_t t0 = static_cast<int64_t>(j) * CKPT;
+    const int len = static_cast<int>(T - t0 < CKPT ? T - t0 : CKPT);   // uniform over a wave (one chunk per wave)
+
+    Cap cc;
+    cc.cap = p.cap;
+    cc.one = p.cap >= 1u ? 1.f : 0.f;
+    cc.two = p.cap >= 2u ? 2.f : cc.one;
+    Neuron nr = {};
+    float lam_p[CKPT], lam_q[CKPT];                              // first x and v of the chunk, then P_t and Q_t
+    float hp = 0.f, hq = 1.f;                                    // h_{t+1} = hp + hq h_in
+    TileSum m1, m2, n1, n2;                                      // sums of lambda_{t+1} vpost_t and lambda_t i_t, split by h_in
+    m1.clear(); m2.clear(); n1.clear(); n2.clear();
+    float vpost_last = 0.f;                                      // potential after the reset of the chunk's last step
+    const float g1 = GO1 ? grad_spikes[0] : 0.f;
+    if (active) {
+        neuron_load<false, CAPK>(nr, p, row);
+        const SurrConst sk = surrogate_consts<KIND>(nr.th, p0, p1);
+        const float *xp = x + (b * T + t0) * M + m0 + lane;
+        const float *gp = GO1 ? nullptr : grad_spikes + (b * T + t0) * M + m0 + lane;
+        float gr[GO1 ? 1 : CKPT];
+#pragma unroll
+        for (int k = 0; k < CKPT; ++k)
+            if (k < len) {
+                lam_q[k] = xp[k * M];
+                if (!GO1) gr[GO1 ? 0 : k] = gp[k * M];
+            }
+        nr.vpost = ckpt_v[(b * n_ck + j) * M + m0 + lane];
+        // rebuild: the same operations in the same order as the forward pass; lam_p[k] = pre-reset potential
+#pragma unroll
+        for (int k = 0; k < CKPT; ++k)
+            if (k < len) {
+                const float v = neuron_advance<false>(nr, lam_q[k]);
+                nr.vpost = __fsub_rn(v, reset_amount<CAPK>(v, nr, cc));
+                lam_p[k] = v;
+            }
+        // reverse walk with the affine pair instead of the value
+        float next_p = 0.f, next_q = 0.f;                        // lambda_{t+1} of the step above, inside this chunk
+#pragma unroll
+        for (int kq = 0; kq < CKPT; ++kq) {
+            const int k = CKPT - 1 - kq;
+            if (k < len) {
+                const float v = lam_p[k], cur_i = lam_q[k];
+                const float sg = surrogate<KIND>(v, nr.th, inv_p0, sk);
+                const float vpost = __fsub_rn(v, reset_amount<CAPK>(v, nr, cc));
+                if (k == len - 1) vpost_last = vpost;            // its partner lambda belongs to the next chunk
+                else { m1.add(next_p, vpost); m2.add(next_q, vpost); }
+                const float through = __fsub_rn(1.0f, __fmul_rn(nr.c, sg));
+                const bool open = v > nr.lo;                     // clamped (or NaN) steps pass nothing on
+                const float lp = open ? __fadd_rn(__fmul_rn(sg, GO1 ? g1 : gr[GO1 ? 0 : k]), __fmul_rn(through, hp)) : 0.f;
+                const float lq = open ? __fmul_rn(through, hq) : 0.f;
+                hp = __fmul_rn(nr.am, lp);
+                hq = __fmul_rn(nr.am, lq);
+                n1.add(lp, cur_i);
+                n2.add(lq, cur_i);
+                lam_p[k] = lp;
+                lam_q[k] = lq;
+                next_p = lp;
+                next_q = lq;
+            }
+        }
+    }
+    map_a[j][lane] = hp;
+    map_b[j][lane] = hq;
+    __syncthreads();
+    // what enters this chunk from later steps: the gradient on the final potential, through the chunks after this one
+    float h_in = (active && grad_v_last) ? grad_v_last[row] : 0.f;
+    for (int c = n_ck - 1; c > j; --c) h_in = __fadd_rn(map_a[c][lane], __fmul_rn(map_b[c][lane], h_in));
+    if (active) {
+        float *op = grad_x + (b * T + t0) * M + m0 + lane;
+#pragma unroll
+        for (int k = 0; k < CKPT; ++k)
+            if (k < len) {
+                lam_p[k] = __fadd_rn(lam_p[k], __fmul_rn(lam_q[k], h_in));     // lambda_t
+                op[k * M] = __fmul_rn(lam_p[k], nr.k);
+            }
+    }
+    first_lambda[j][lane] = active ? lam_p[0] : 0.f;
+    if (j == 0) first_lambda[n_ck][lane] = 0.f;                  // beyond the sequence: lambda_T = 0
+    m1.fold(); m2.fold(); n1.fold(); n2.fold();
+    __syncthreads();
+    double mine = 0.0;
+    if (active && alpha_mem_grad) {
+        // sum_t lambda_{t+1} vpost_t over this chunk (the last step pairs with the next chunk's first lambda) ...
+        mine = m1.total + m2.total * static_cast<double>(h_in) +
+               static_cast<double>(first_lambda[j + 1][lane]) * static_cast<double>(vpost_last);
+        // ... the initial state's term, and what the input normalisation contributes: - sum_t lambda_t i_t
+        if (j == 0) mine += static_cast<double>(lam_p[0]) * static_cast<double>(p.v_init[row]);
+        if (p.norm_input) mine -= n1.total + n2.total * static_cast<double>(h_in);
+    }
+    partial[j][lane] = mine;
+    __syncthreads();
+    if (j == 0 && active) {
+        if (alpha_mem_grad) {
+            double total = 0.0;
+            for (int c = 0; c < n_ck; ++c) total += partial[c][lane];
+            alpha_mem_grad[row] = static_cast<float>(total);
+        }
+        if (v_init_grad) v_init_grad[row] = __fadd_rn(hp, __fmul_rn(hq, h_in));    // h_0 = a_mem lambda_0
+    }
+}
+
+// 0: never, 1: for layers that leave most of the machine idle (default), 2: whenever the kernel applies
+std::atomic<int> split_mode{1};
+constexpr int64_t SPLIT_MOST_NEURONS = 16384;                    // batch * neurons up to which mode 1 splits
+
+template <int KIND, int CAPK>
+int launch_bwd_split(float *grad_x, float *am_g, float *v0_g, const float *grad_spikes, const float *gvl, const float *x,
+                     const float *ckpt_v, const LayerConsts &p, float p0, float p1, bool uniform, int64_t B, int64_t T,
+                     int64_t M, hipStream_t s)
+{
+    const int64_t blocks_per_batch = (M + SPLIT_NEURONS - 1) / SPLIT_NEURONS;
+    if (blocks_per_batch > 0x7fffffffLL / B) return hipErrorInvalidValue;
+    const dim3 grid(static_cast<unsigned>(blocks_per_batch * B));
+    const dim3 block(SPLIT_NEURONS, static_cast<unsigned>((T + CKPT - 1) / CKPT));
+    const float inv_p0 = p0 != 0.f ? 1.f / p0 : 0.f;
+    if (uniform)
+        hipLaunchKernelGGL((layer_lif_backward_split<KIND, CAPK, true>), grid, block, 0, s, grad_x, am_g, v0_g, grad_spikes,
+                           gvl, x, ckpt_v, p, p0, p1, inv_p0, blocks_per_batch, T, M);
+    else
+        hipLaunchKernelGGL((layer_lif_backward_split<KIND, CAPK, false>), grid, block, 0, s, grad_x, am_g, v0_g, grad_spikes,
+                           gvl, x, ckpt_v, p, p0, p1, inv_p0, blocks_per_batch, T, M);
+    return static_cast<int>(hipGetLastError());
+}
+
+template <int KIND, class... A>
+int dispatch_bwd_split_cap(unsigned cap, A... a)
+{
+    if (cap == 1u) return launch_bwd_split<KIND, 1>(a...);
+    if (cap == 2u) return launch_bwd_split<KIND, 2>(a...);
+    return launch_bwd_split<KIND, 0>(a...);
+}
+
 template <bool SYN, int KIND, int CAPK>
 int launch_bwd(float *grad_x, float *am_g, float *as_g, float *v0_g, float *i0_g, const float *grad_spikes,
                const float *gvl, const float *gil, const float *x, const float *surr, const float *gvr,
@@ -1143,6 +1311,23 @@ EXODUS_API int exodus_layer_lif_backward(float *grad_input, float *alpha_mem_gra
     p.cap = static_cast<unsigned>(max_num_spikes);
     p.rec_pre = 0;
     hipStream_t s = static_cast<hipStream_t>(stream);
+    // few neurons, many steps: one lane per chunk of 32 steps instead of one lane per neuron
+    const int mode = split_mode.load(std::memory_order_relaxed);
+    const int64_t n_ck = (t + CKPT - 1) / CKPT;
+    if (mode != 0 && !syn && surrogate_kind != EXODUS_SURR_TENSOR && !grad_v_rec && n_ck >= 2 && n_ck <= SPLIT_MAX_CHUNKS &&
+        (mode == 2 || batch * neurons <= SPLIT_MOST_NEURONS)) {
+#define EXODUS_SPLIT(K)                                                                                           \
+    return dispatch_bwd_split_cap<K>(p.cap, grad_input, alpha_mem_grad, vmem_init_grad, grad_spikes, grad_v_last, \
+                                     input, ckpt_v, p, surr_p0, surr_p1, grad_spikes_uniform != 0, batch, t,      \
+                                     neurons, s)
+        switch (surrogate_kind) {
+            case EXODUS_SURR_SINGLE_EXP: EXODUS_SPLIT(EXODUS_SURR_SINGLE_EXP);
+            case EXODUS_SURR_PERIODIC_EXP: EXODUS_SPLIT(EXODUS_SURR_PERIODIC_EXP);
+            case EXODUS_SURR_HEAVISIDE: EXODUS_SPLIT(EXODUS_SURR_HEAVISIDE);
+            default: return hipErrorInvalidValue;
+        }
+#undef EXODUS_SPLIT
+    }
 #define EXODUS_BWD(SYN, K)                                                                                        \
     return dispatch_bwd_cap<SYN, K>(p.cap, grad_input, alpha_mem_grad, alpha_syn_grad, vmem_init_grad,            \
                                     isyn_init_grad, grad_spikes, grad_v_last, grad_i_last, input, surr,           \
@@ -1156,6 +1341,13 @@ EXODUS_API int exodus_layer_lif_backward(float *grad_input, float *alpha_mem_gra
         default: return hipErrorInvalidValue;
     }
 #undef EXODUS_BWD
+}
+
+EXODUS_API int exodus_layer_backward_time_split(int mode)
+{
+    const int before = split_mode.load(std::memory_order_relaxed);
+    if (mode >= 0 && mode <= 2) split_mode.store(mode, std::memory_order_relaxed);
+    return before;
 }
 
 EXODUS_API int64_t exodus_layer_scratch_floats(void) { return SCRATCH_FLOATS; }

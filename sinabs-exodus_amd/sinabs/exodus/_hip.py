@@ -48,6 +48,7 @@ _SIGNATURES = {
     "exodus_layer_checkpoint_interval": ([], _int),
     "exodus_layer_lif_forward": ([_p] * 16 + [_int, _int, _int, _int, _int, _i64, _i64, _i64, _p], _int),
     "exodus_layer_lif_backward": ([_p] * 18 + [_int, _int, _int, _int, _int, _f, _f, _p, _p, _p, _int, _i64, _i64, _i64, _p], _int),
+    "exodus_layer_backward_time_split": ([_int], _int),
     "exodus_layer_scratch_floats": ([], _i64),
     "exodus_layer_lif_backward_from_input": ([_p] * 16 + [_int, _int, _int, _int, _int, _f, _f, _p, _p, _p, _int, _i64, _i64, _i64, _p], _int),
     "exodus_layer_leaky_forward": ([_p] * 6 + [_int, _int, _i64, _i64, _i64, _p], _int),
@@ -504,6 +505,13 @@ def layerLifForward(input, vmemPostInitial, isynInitial, alphaMem, alphaSyn, mem
             _ptr(theta), _ptr(thetaLow), int(bool(applyThetaLow)), int(maxNumSpikes), int(bool(decayEarly)),
             int(bool(normInput)), int(bool(wantPreReset)), b, t, m, _stream(input)), "exodus_layer_lif_forward")
     return res
+
+
+def backwardTimeSplit(mode: int = -1) -> int:
+    """How ``layerLifBackward`` treats layers with few neurons and many steps (``exodus_layer_backward_time_split``):
+    0 never splits the sequence over lanes, 1 (default) does for layers of up to 16 384 neurons, 2 whenever the kernel
+    applies; -1 only asks.  Returns the mode that was set before."""
+    return int(lib.exodus_layer_backward_time_split(int(mode)))
 
 
 def scratchFloats() -> int:

@@ -17,6 +17,16 @@ from _util import gen, note_scaled
 pytestmark = pytest.mark.gpu
 
 
+@pytest.fixture(autouse=True, params=["one lane per neuron", "small layers split over time"])
+def backward_kernel_choice(request):
+    """Every test of this file runs twice: with the backward kernel that walks a neuron's sequence in one lane only, and
+    with the default choice, which hands small layers to the kernel that gives every 32 steps a lane."""
+    from sinabs.exodus import _hip
+    before = _hip.backwardTimeSplit(0 if request.param.startswith("one") else 1)
+    yield
+    _hip.backwardTimeSplit(before)
+
+
 def excess(got, want, rtol=1e-4, atol=1e-5, of_max=1e-5):
     if not got.numel():
         return 0.0
