@@ -744,6 +744,9 @@ def main():
     ap.add_argument("--one-lane-per-neuron", action="store_true",
                     help="keep the backward kernel that walks a neuron's whole sequence in one lane also for layers with few "
                          "neurons (by default those run the kernel that gives every 32 steps a lane of its own)")
+    ap.add_argument("--split-any-size", action="store_true",
+                    help="the opposite: run the kernel that gives every 32 steps a lane of its own for layers of any size "
+                         "that it can handle (to see where it stops paying; the default draws the line at 16384 neurons)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--others", default="all", choices=["all", "api", "none"],
                     help="all (default): also time the other configurations and the (rows, time) kernels for a few steps "
@@ -812,8 +815,8 @@ def main():
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    if args.one_lane_per_neuron:
-        hip.backwardTimeSplit(0)
+    if args.one_lane_per_neuron or args.split_any_size:
+        hip.backwardTimeSplit(0 if args.one_lane_per_neuron else 2)
     if args.region_map:
         measure_region_map(args, torch, dev)
         return
@@ -840,6 +843,10 @@ def main():
         if placement_note:
             out["placement_note"] = placement_note
         if place.regions is not None:
+            if args.placement != "striped" and args.placement != "all-striped" and not place.regions.sorted:
+                out["placement_note"] = ("timed copies found no three regions in the memory this process was handed (it comes "
+                                         "mixed once other processes have used striped ranges): after retries with finer pieces "
+                                         "the striped range was made unsorted, as sort=False makes it")
             out["gave_memory_back"] = hbm.disable()
         print(json.dumps(out))
         return
