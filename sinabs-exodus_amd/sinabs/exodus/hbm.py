@@ -23,7 +23,8 @@ block was used on (``Tensor.record_stream``): a tensor of a range is as safe acr
 ``with placement():`` sends *every* allocation of the calling thread there (what torch itself allocates in a forward
 pass: activations of other layers, temporaries); ``enable(everything=True)`` does that for all threads until
 ``disable()``, which covers the gradients that autograd's own thread allocates in a backward pass.  Without
-``enable()`` nothing changes.  The reference has no counterpart (its CUDA extension allocates outputs with
+``enable()`` nothing changes -- unless the environment asks for it: ``SINABS_EXODUS_HBM=striped[:GiB]`` or
+``everything[:GiB]`` stands for that call in a program that is to run unchanged (``_from_environment``).  The reference has no counterpart (its CUDA extension allocates outputs with
 ``torch.empty_like``, reference cuda/bindings.cu:98,144,183).
 
 While a HIP graph is being captured the wrappers leave allocation to the capture's own pool (a graph's memory must
@@ -34,6 +35,7 @@ from __future__ import annotations
 
 import contextlib
 import ctypes
+import os
 import threading
 import time
 import warnings
@@ -373,7 +375,54 @@ def placement():
         yield
 
 
+ENVIRONMENT_SWITCH = "SINABS_EXODUS_HBM"
+FIRST_PLACED_UNASKED = 64 * 2 ** 20   # the environment switch makes the ranges when the first output this big is due
+_switch_tried = False
+
+
+def _read_switch(asked: str):
+    """``striped`` / ``everything``, optionally ``:<GiB>`` -> (GiB of the striped range, everything); None for an empty
+    value or one that says no; ValueError for anything else."""
+    asked = asked.strip().lower()
+    if not asked or asked in ("0", "off", "no", "false"):
+        return None
+    mode, _, size = asked.partition(":")
+    if mode in ("1", "on", "yes", "true"):
+        mode = "striped"
+    if mode not in ("striped", "everything"):
+        raise ValueError(f"unknown mode '{mode}' (striped or everything, optionally followed by :<GiB>)")
+    gib = float(size) if size else 48.0
+    if not gib > 0:
+        raise ValueError("the size must be positive")
+    return gib, mode == "everything"
+
+
+def _from_environment(nbytes: int, device: torch.device) -> None:
+    """``SINABS_EXODUS_HBM=striped`` (or ``striped:<GiB>``, ``everything``, ``everything:<GiB>``; default 48 GiB) in the
+    environment stands for a call of ``enable(gib_striped=<GiB>, everything=...)``, for programs that are to run
+    unchanged: the ranges are made on the device of the first kernel output of 64 MiB or more (a program with small
+    layers never pays the set-up).  A value that cannot be read, or ranges that cannot be made, give one warning and
+    the ordinary allocator."""
+    global _switch_tried
+    if _switch_tried or nbytes < FIRST_PLACED_UNASKED or device.type != "cuda":
+        return
+    asked = os.environ.get(ENVIRONMENT_SWITCH, "")
+    if not asked.strip():
+        return
+    if torch.cuda.is_current_stream_capturing():
+        return                                             # not now: try again at the next eager call
+    _switch_tried = True
+    try:
+        how = _read_switch(asked)
+        if how is not None:
+            enable(gib_striped=how[0], device=device, everything=how[1])
+    except (RuntimeError, ValueError) as err:
+        warnings.warn(f"{ENVIRONMENT_SWITCH}={asked}: no placement, ordinary allocator used ({err})")
+
+
 def _wanted(nbytes: int, device: torch.device) -> bool:
+    if _active is None:
+        _from_environment(nbytes, device)
     return (_active is not None and nbytes >= SMALLEST_PLACED and device == _active.device
             and bool(_active.sizes[STRIPED]))
 

@@ -313,3 +313,39 @@ def test_too_little_free_memory_is_refused(hbm):
         hbm.HbmRegions(gib_striped=24.0)
     del held
     assert hbm.active() is None
+
+
+def test_environment_switch_stands_for_enable(hbm, monkeypatch):
+    """``SINABS_EXODUS_HBM=striped:<GiB>``: a program that never calls ``enable()`` gets the ranges at its first kernel
+    output of 64 MiB or more -- not for small layers, not again after ``disable()``, and with a warning instead of an
+    error for a value that cannot be read."""
+    import sinabs.exodus.layers as el
+    dev = torch.device("cuda:0")
+    layer = el.IAF().to(dev)
+    small = (torch.rand(2, 50, 256, generator=gen(31)) * 0.6).to(dev)
+    big = (torch.rand(8, 200, 16384, generator=gen(32)) * 0.6).to(dev)          # 100 MiB per tensor
+
+    def run(x):
+        layer.reset_states()
+        return layer(x)
+
+    want = run(big)
+    monkeypatch.setattr(hbm, "_switch_tried", False)
+    monkeypatch.setenv(hbm.ENVIRONMENT_SWITCH, "nonsense:4")
+    with pytest.warns(UserWarning, match="no placement"):
+        assert torch.equal(run(big), want)
+    assert hbm.active() is None and hbm._switch_tried is True
+    monkeypatch.setattr(hbm, "_switch_tried", False)
+    monkeypatch.setenv(hbm.ENVIRONMENT_SWITCH, "striped:6")
+    run(small)
+    assert hbm.active() is None                                 # nothing big enough yet
+    got = run(big)
+    regions = hbm.active()
+    assert regions is not None and regions.sizes[hbm.STRIPED] == 12 * GIB
+    assert regions.pool_of(got) == hbm.STRIPED and torch.equal(got, want)
+    del got
+    layer.reset_states()
+    gc.collect()
+    assert hbm.disable() is True
+    again = run(big)
+    assert hbm.active() is None and torch.equal(again, want)    # switched off by hand: it stays off

@@ -277,6 +277,13 @@ def test_hbm_argument_checks_and_sorting_retries_without_a_device():
                 dict(gib_per_region=1.0, sort=False), dict(chunk_bytes=100 * MIB), dict(take_limit_gib=-2.0)):
         with pytest.raises((ValueError, RuntimeError)):      # RuntimeError: no device in this process
             hbm.HbmRegions(**bad)
+    # the environment's way of asking for enable()
+    assert hbm._read_switch("") is None and hbm._read_switch(" off ") is None
+    assert hbm._read_switch("striped") == (48.0, False) and hbm._read_switch("Striped:72") == (72.0, False)
+    assert hbm._read_switch("everything:12.5") == (12.5, True) and hbm._read_switch("on") == (48.0, False)
+    for bad in ("bogus", "striped:x", "striped:-1", "everything:0"):
+        with pytest.raises(ValueError):
+            hbm._read_switch(bad)
     # sorting is tried again with finer pieces when the big ones show no regions
     class Lib:
         def __init__(self, outcomes):
