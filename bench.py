@@ -109,6 +109,20 @@ class Placement:
         return out
 
 
+SURROGATE = "single"      # --surrogate: which of the surrogate gradients evaluated inside the kernels the workloads use
+
+
+def chosen_surrogate(hip, act):
+    """(kind, p0, p1) as the kernels take them; SingleExponential is what every configuration names."""
+    if SURROGATE == "periodic":
+        fn = act.PeriodicExponential()
+        return hip.SURR_PERIODIC_EXP, fn.grad_width, fn.grad_scale
+    if SURROGATE == "heaviside":
+        return hip.SURR_HEAVISIDE, act.Heaviside().window, 1.0
+    fn = act.SingleExponential()
+    return hip.SURR_SINGLE_EXP, fn.grad_width, fn.grad_scale
+
+
 def build_layer_workload(key, torch, hip, act, dev, place=None, one_value=False):
     """The same workloads on the layer's own (batch, time, neurons) layout: one kernel per direction,
     forward keeps checkpoints only, backward re-reads the input and rebuilds v_mem / i_syn.
@@ -127,8 +141,7 @@ def build_layer_workload(key, torch, hip, act, dev, place=None, one_value=False)
     bwd_bytes = 8 if one_value else 12
     rows = lambda v: torch.as_tensor(v, dtype=torch.float32, device=dev).expand(B, M).flatten().contiguous()
     zeros = torch.zeros(N, device=dev); ones = torch.ones(N, device=dev)
-    surr = act.SingleExponential()
-    kind, p0, p1 = hip.SURR_SINGLE_EXP, surr.grad_width, surr.grad_scale
+    kind, p0, p1 = chosen_surrogate(hip, act)
     spikes = place.empty(x.shape, rs); gi = place.empty(x.shape, rgi)
     if key == "c5":
         cfg = dict(a_mem=rows(math.exp(-1 / 20.0)), a_syn=rows(math.exp(-1 / 5.0)), lo=rows(-1.0), cap=2, norm=True)
@@ -184,8 +197,7 @@ def build_workload(key, torch, hip, act, dev, place=None):
     rows = lambda v: torch.as_tensor(v, dtype=torch.float32, device=dev).expand(B, M).flatten().contiguous()
     zeros = torch.zeros(N, device=dev)
     ones = torch.ones(N, device=dev)
-    surr = act.SingleExponential()
-    kind, p0, p1 = hip.SURR_SINGLE_EXP, surr.grad_width, surr.grad_scale
+    kind, p0, p1 = chosen_surrogate(hip, act)
     fwd_name = bwd_name = None
 
     if key == "c5":
@@ -741,6 +753,10 @@ def main():
     ap.add_argument("--one-value-gradient", action="store_true",
                     help="with --path layer: the gradient of every output element is one number, handed to the backward "
                          "kernel as such (what a sum as the loss gives): it reads one tensor less (8 + 8 bytes)")
+    ap.add_argument("--surrogate", default="single", choices=["single", "periodic", "heaviside"],
+                    help="surrogate gradient of the spiking workloads' kernels (wrappers, --path layer / rows): "
+                         "SingleExponential as the configurations name it (default), PeriodicExponential or Heaviside -- "
+                         "a measurement aid: the default run and its public-API entries always use SingleExponential")
     ap.add_argument("--one-lane-per-neuron", action="store_true",
                     help="keep the backward kernel that walks a neuron's whole sequence in one lane also for layers with few "
                          "neurons (by default those run the kernel that gives every 32 steps a lane of its own)")
@@ -798,8 +814,10 @@ def main():
                                         name=w_["name"] + f" -- at shape ({b_},{t_},{m_})")
 
     plain_first = None
+    global SURROGATE
+    SURROGATE = args.surrogate
     special = (args.region_map or args.ceilings or args.conv_snn or args.shape or args.copy_probe or args.setup_only
-               or args.one_value_gradient)
+               or args.one_value_gradient or args.surrogate != "single")
     full_run = args.placement == "striped" and args.others == "all" and not special
     common = ["--no-cpu-baseline", "--workload", args.workload, "--path", args.path, "--steps", str(args.steps),
               "--warmup", str(args.warmup)]
@@ -902,6 +920,8 @@ def main():
     }
     if placement_note:
         result["config"]["placement_note"] = placement_note
+    if args.surrogate != "single":
+        result["config"]["surrogate"] = args.surrogate + " (a measurement aid: the configuration names SingleExponential)"
     if plain_first is not None:
         # the ordinary allocator's figures beside the headline: what the same kernels reach without hbm.enable()
         pr = plain_first.get("roofline", {})

@@ -122,7 +122,7 @@ __device__ __forceinline__ float spike_count(float v, float theta, unsigned cap)
 // (tolerance rtol 1e-4), never spike decisions, so divisions by per-row constants become
 // multiplications by their reciprocals and exp() is the hardware exponential (relative error
 // about |argument| * 6e-8).
-struct SurrConst { float a, b; };
+struct SurrConst { float a, b, c; };
 
 constexpr float NEG_LOG2_E = -1.44269504088896340736f;         // exp(-x) = exp2(x * NEG_LOG2_E)
 
@@ -130,6 +130,7 @@ template <int KIND>
 __device__ __forceinline__ SurrConst surrogate_consts(float theta, float p0, float p1)
 {
     SurrConst k;
+    k.c = 0.f;
     if (KIND == EXODUS_SURR_SINGLE_EXP) {
         const float w = __fmul_rn(theta, p0);                 // p1/(theta p0) * exp(-|v - theta| / (theta p0))
         k.a = __fdiv_rn(NEG_LOG2_E, w);
@@ -137,11 +138,28 @@ __device__ __forceinline__ SurrConst surrogate_consts(float theta, float p0, flo
     } else if (KIND == EXODUS_SURR_PERIODIC_EXP) {
         k.a = __fmul_rn(theta, 0.5f);                          // p1 * exp(-|u - theta/2| / p0) / theta
         k.b = __fdiv_rn(p1, theta);
+        k.c = __fdiv_rn(1.f, theta);
     } else {
         k.a = __fsub_rn(theta, p0);                            // (v >= theta - p0) / theta
         k.b = __fdiv_rn(1.f, theta);
     }
     return k;
+}
+
+// u modulo theta for theta > 0 (result in [0, theta), as the floor-modulo of the Python definition gives it), without
+// the library's fmodf, whose loop costs the backward kernels a third of their registers and half their speed.  The
+// quotient comes from the reciprocal; floor(u * inv) is the true quotient or one off next to a multiple of theta, and
+// the fused multiply-add takes q * theta away without rounding when q is right.  A second pass deals with quotients
+// beyond 2^24 (q itself rounded), the two corrections with a quotient that was one off.  Exact whenever the first
+// quotient is (then the second pass and the corrections change nothing); otherwise within an ulp of theta.
+__device__ __forceinline__ float wrap_into_period(float u, float theta, float inv_theta)
+{
+    float r = u;
+#pragma unroll
+    for (int pass = 0; pass < 2; ++pass) r = __fmaf_rn(-floorf(__fmul_rn(r, inv_theta)), theta, r);
+    if (r < 0.f) r = __fadd_rn(r, theta);
+    if (r >= theta) r = __fsub_rn(r, theta);
+    return r;
 }
 
 // exp() is the hardware's base-2 exponential with the change of base folded into the constants
@@ -153,7 +171,7 @@ __device__ __forceinline__ float surrogate(float v, float theta, float inv_p0, S
         return k.b * __builtin_amdgcn_exp2f(fabsf(v - theta) * k.a);
     } else if (KIND == EXODUS_SURR_PERIODIC_EXP) {
         float u = v - k.a;
-        if (v >= theta) u = fmodf(u, theta);                 // u > 0 here, so fmod == floor-mod
+        if (v >= theta) u = wrap_into_period(u, theta, k.c);
         return k.b * __builtin_amdgcn_exp2f(fabsf(u - k.a) * (NEG_LOG2_E * inv_p0));
     } else {
         return v >= k.a ? k.b : 0.f;

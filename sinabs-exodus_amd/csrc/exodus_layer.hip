@@ -51,7 +51,8 @@ namespace {
 #define EXODUS_LAYER_BWD_WAVES 3      // resident waves per SIMD the backward kernel is compiled for
 #endif
 #ifndef EXODUS_LAYER_BWD_WAVES_G1
-#define EXODUS_LAYER_BWD_WAVES_G1 4   // ... and its instances that stream one tensor less (one gradient value for all)
+#define EXODUS_LAYER_BWD_WAVES_G1 3   // ... and its instances that stream one tensor less (one gradient value for all): a
+                                      // fourth wave fits them only with spills and measures no faster
 #endif
 constexpr int CKPT = EXODUS_LAYER_CKPT;               // steps between checkpoints = length of a backward chunk
 constexpr int FWD_UNROLL = EXODUS_LAYER_FWD_UNROLL;  // forward steps per software-pipeline stage (divides CKPT)
@@ -553,7 +554,12 @@ layer_lif_backward(
         for (int kq = 0; kq < CKPT; ++kq) {
             const int k = CKPT - 1 - kq;
             if (!GUARD || k < len) {
-                const float v = vr[k], cur_i = xr[k];
+                float v = vr[k];
+                const float cur_i = xr[k];
+                // The longer surrogate is evaluated when its step is reached, not for all 32 steps ahead of the walk
+                // (which the compiler otherwise does: 32 more live values, spilled to memory): the empty statement makes
+                // this step's potential depend on the adjoint that the previous one has produced.
+                if (KIND == EXODUS_SURR_PERIODIC_EXP) asm volatile("" : "+v"(v) : "v"(h));
                 const float sg = FROM_TENSOR ? sr[FROM_TENSOR ? k : 0] : surrogate<KIND>(v, nr.th, inv_p0, sk);
                 const float vpost = __fsub_rn(v, reset_amount<CAPK>(v, nr, cc));
                 acc_m.add(lam, vpost);                          // lambda_{t+1} * vpost_t
