@@ -628,7 +628,10 @@ struct LeakyConsts {
     int decay_early, norm_input;
 };
 
-constexpr int LEAKY_UNROLL = 8;
+#ifndef EXODUS_LEAKY_UNROLL
+#define EXODUS_LEAKY_UNROLL 8
+#endif
+constexpr int LEAKY_UNROLL = EXODUS_LEAKY_UNROLL;
 
 // Both leaky kernels walk time in pairs of stages of LEAKY_UNROLL steps with two register buffers:
 // while one stage is consumed, the loads of the other are in flight, and because every fetch
