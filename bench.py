@@ -65,7 +65,10 @@ MEASURED_TRAFFIC = load_measured_traffic()
 # what the default run reports next to its headline workload: (workload, path)
 OTHERS = [("c2", "layer"), ("c3", "layer"), ("c5", "rows"), ("c2", "rows"), ("c3", "rows")]
 # ... and through the public layer API: (workload, loss)
-API_RUNS = [("c5", "dense"), ("c5", "sum"), ("c2", "dense"), ("c2", "sum"), ("c3", "dense"), ("c3", "sum")]
+# loss: "dense" = out.backward(gradient tensor); "sum" = out.sum().backward(), torch's own reduction over the output;
+# "total" = the same loss taken from the layer: firing_rate * numel, i.e. the total the forward kernel counted anyway
+API_RUNS = [("c5", "dense"), ("c5", "sum"), ("c5", "total"), ("c2", "dense"), ("c2", "sum"), ("c2", "total"),
+            ("c3", "dense"), ("c3", "sum")]
 
 
 class Placement:
@@ -475,7 +478,11 @@ def measure_layer_api(key, loss, torch, dev, steps, warmup, place_all=False):
         out = layer(x)
         if e:
             e[1].record()
-        total = out.sum() if loss == "sum" else None            # torch's own reduction over the output
+        total = None
+        if loss == "sum":
+            total = out.sum()                                   # torch's own reduction over the output
+        elif loss == "total":
+            total = layer.firing_rate * float(out.numel())      # the same number, counted by the forward kernel
         if e:
             e[2].record()
         if loss == "dense":
@@ -504,7 +511,9 @@ def measure_layer_api(key, loss, torch, dev, steps, warmup, place_all=False):
     # torch's sum over the output (4 more, "loss_ms") is the program's loss, not the layer, and is left out of the fraction
     layer_bytes = 20 if loss == "dense" else 16
     return {"workload": w["name"], "path": "public layer API (sinabs.exodus.layers, autograd, outputs allocated per call)",
-            "layer": repr(layer).split("(")[0].strip(), "loss": "out.backward(dense gradient)" if loss == "dense" else "out.sum().backward()",
+            "layer": repr(layer).split("(")[0].strip(), "loss": {"dense": "out.backward(dense gradient)", "sum": "out.sum().backward()",
+                     "total": "(layer.firing_rate * out.numel()).backward() -- the sum of the output as the forward kernel "
+                              "counted it"}[loss],
             "rows": n_t // shape[1], "time_steps": shape[1], "steps": steps, "ms_per_step": wall * 1e3,
             "fwd_ms": fwd_ms, "loss_ms": loss_ms, "bwd_ms": bwd_ms, "value": n_t / wall, "unit": "neuron-timesteps/s",
             "algorithmic_bytes_per_neuron_timestep": layer_bytes,
