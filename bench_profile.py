@@ -150,13 +150,14 @@ def main():
         sys.exit(f"no profiled runs found under {args.directory}")
     os.makedirs(os.path.join(ROOT, "profiles"), exist_ok=True)
     flags = (" " + args.extra_flags.strip()) if args.extra_flags.strip() else ""
+    where = args.directory.rstrip("/")                         # as given on the command line
     md = [f"# Kernel trace and HBM counters of the bench workloads — {args.name.replace('_', ' ')}", "",
           f"Placement: {args.placement}.", "",
           "Commands (GPU box, repo root, after `cd /tmp && export TMPDIR=/tmp && cd $GRAFT_REPO_ROOT`), for each `<w>_<p>` below:", "",
-          f"    rocprofv3 --kernel-trace --stats --output-format csv -d gpurun_out/<dir>/<w>_<p>/stats -o x -- python3 bench.py --workload <w> --path <p> --no-cpu-baseline --no-others --copy-probe --steps 10 --warmup 3{flags}",
-          f"    rocprofv3 --pmc FETCH_SIZE --output-format csv -d gpurun_out/<dir>/<w>_<p>/fetch -o x -- python3 bench.py --workload <w> --path <p> --no-cpu-baseline --no-others --copy-probe --steps 3 --warmup 1{flags}",
-          f"    rocprofv3 --pmc WRITE_SIZE --output-format csv -d gpurun_out/<dir>/<w>_<p>/write -o x -- python3 bench.py --workload <w> --path <p> --no-cpu-baseline --no-others --copy-probe --steps 3 --warmup 1{flags}",
-          f"    python bench_profile.py gpurun_out/<dir> --name {args.name}", "",
+          f"    rocprofv3 --kernel-trace --stats --output-format csv -d {where}/<w>_<p>/stats -o x -- python3 bench.py --workload <w> --path <p> --no-cpu-baseline --no-others --copy-probe --steps 10 --warmup 3{flags}",
+          f"    rocprofv3 --pmc FETCH_SIZE --output-format csv -d {where}/<w>_<p>/fetch -o x -- python3 bench.py --workload <w> --path <p> --no-cpu-baseline --no-others --copy-probe --steps 3 --warmup 1{flags}",
+          f"    rocprofv3 --pmc WRITE_SIZE --output-format csv -d {where}/<w>_<p>/write -o x -- python3 bench.py --workload <w> --path <p> --no-cpu-baseline --no-others --copy-probe --steps 3 --warmup 1{flags}",
+          f"    python bench_profile.py {where} --name {args.name}", "",
           "Durations in ms from the kernel trace.  Read / written: mean FETCH_SIZE / WRITE_SIZE per dispatch, scaled by what the same",
           "counter reads for the 1 GiB elementwise kernel of the same run (`--copy-probe`: 1 048 576 KiB read and written):", ""]
     md += [f"* {n}" for n in notes]
